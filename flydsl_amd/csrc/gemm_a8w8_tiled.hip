@@ -1,0 +1,242 @@
+// Compute-bound mainloop of the 8-bit preshuffle GEMM for gfx950.
+//
+//   C[M,N] = A[M,K] * W[N,K]^T, W preshuffled into 1 KB fragment blocks [N/16][K/64][klane 4][nlane 16][16 B].
+//
+// One workgroup = 4 wavefronts side by side along N; tile = (16*MR) x (64*NR) x 128 bytes of K.
+//   * A tile: global -> VGPR -> LDS (XOR-swizzled 128-byte rows), double buffered, read back as
+//     MFMA fragments with ds_read_b128.
+//   * B fragments: each wave loads its own 1 KB blocks straight from global memory into the MFMA
+//     operand registers (lane l reads bytes [16l, 16l+16) of a block: one fully coalesced 1 KB load).
+//   * MFMA: operands are swapped (B fragment = src0, A fragment = src1) so that a lane ends up with
+//     four CONSECUTIVE N columns of one M row: the epilogue stores 8 bytes per lane per fragment.
+//       fp8 : v_mfma_f32_16x16x128_f8f6f4 (unscaled form), 32 bytes of K per lane, taken as
+//             bytes [16g,16g+16) and [64+16g, 64+16g+16) of the 128-byte K step (g = lane/16) so that
+//             each half is exactly one preshuffled block; A uses the same K order.
+//       int8: two v_mfma_i32_16x16x64_i8 per K step (one per 64-byte half), int32 accumulate (exact).
+//   * Workgroup ids are remapped so that the ids the hardware deals to one XCD cover a compact
+//     group_m x tiles_n patch of tiles (A and B panels stay in that XCD's L2).
+#include "psg_common.h"
+
+namespace {
+
+constexpr int TK = 128;  // bytes of K per mainloop step
+
+template <int KIND>
+struct Acc {
+    using type = v4f;
+};
+template <>
+struct Acc<KIND_INT8> {
+    using type = v4i;
+};
+
+// LDS byte offset of 16-byte chunk `kc` (0..7) of row `row` inside one A stage
+__device__ __forceinline__ int lds_off(int row, int kc) { return row * TK + ((kc ^ ((row >> 1) & 7)) << 4); }
+
+__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
+    const int num = tiles_m * tiles_n;
+    const int q = num >> 3, r = num & 7;
+    const int xcd = id & 7, in_xcd = id >> 3;
+    const int wg = xcd * q + (xcd < r ? xcd : r) + in_xcd;
+    const int per_group = group_m * tiles_n;
+    const int g = wg / per_group;
+    const int first_m = g * group_m;
+    const int size_m = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+    const int in_g = wg - g * per_group;
+    tm = first_m + in_g % size_m;
+    tn = in_g / size_m;
+}
+
+template <int KIND, int MR, int NR, int STORE>
+__global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
+    using acc_t = typename Acc<KIND>::type;
+    constexpr int TM = 16 * MR;
+    constexpr int TN = 64 * NR;
+    constexpr int A_LOADS = TM / 32;  // 16-byte chunks of the A tile per thread
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * TK];
+
+    const int tid = threadIdx.x;
+    const int wave = wave_id();
+    const int lane = tid & 63;
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+
+    const int tiles_m = (p.M + TM - 1) / TM;
+    const int tiles_n = (p.N + TN - 1) / TN;
+    int tm, tn;
+    tile_coords((int)blockIdx.x, tiles_m, tiles_n, p.group_m, tm, tn);
+    const int m0 = tm * TM;
+    const int n0 = tn * TN;
+    const int K = p.K;
+    const int KT = (K + TK - 1) / TK;
+
+    // A: this tile's rows; rows >= M read as zero through the descriptor bound
+    const uint64_t a_rows = (uint64_t)(p.M - m0);
+    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a + (uint64_t)m0 * K, a_rows * (uint64_t)K);
+    // B: this wave's NR n-blocks; blocks >= N/16 read as zero
+    const int nb0 = (n0 >> 4) + wave * NR;
+    const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)K;
+    const uint64_t b_total = (uint64_t)p.N * (uint64_t)K;
+    __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
+
+    // per-thread A copy geometry: chunk c = tid + 256*j -> (row = c/8, kc = c%8)
+    const int a_row0 = tid >> 3;
+    const int a_kc = tid & 7;
+    const uint32_t a_goff0 = (uint32_t)a_row0 * (uint32_t)K + (uint32_t)a_kc * 16u;
+
+    acc_t acc[MR][NR];
+#pragma unroll
+    for (int mi = 0; mi < MR; mi++)
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (acc_t){0, 0, 0, 0};
+
+    v4i areg[A_LOADS];
+    v4i blo[2][NR], bhi[2][NR];
+
+    auto load_a = [&](int kt) {
+        const uint32_t k0 = (uint32_t)kt * TK;
+        // a 16-byte chunk is either fully inside K or fully outside (K % 64 == 0)
+        const bool in_k = (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++) {
+            // the whole byte offset sits in the bounds-checked VGPR offset: rows >= M (and the tail of the
+            // last row when K % 128 == 64) come back as zero instead of touching memory past A
+            v4i v = buf_load16(ra, a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0, 0);
+            areg[j] = in_k ? v : (v4i){0, 0, 0, 0};
+        }
+    };
+    auto store_a = [&](int stage) {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++) {
+            const int row = a_row0 + 32 * j;
+            *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, a_kc)]) = areg[j];
+        }
+    };
+    auto load_b = [&](int kt, v4i* lo, v4i* hi) {
+        const bool has_hi = (kt * TK + 64) < K;
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) {
+            // n-block select in the bounds-checked VGPR offset (blocks >= N/16 read as zero), K position in
+            // the scalar offset; a missing upper half re-reads the lower one instead of running past W
+            const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
+            const uint32_t koff = (uint32_t)kt * 2048u;
+            lo[ni] = buf_load16(rb, voff, koff);
+            v4i h = buf_load16(rb, voff, has_hi ? koff + 1024u : koff);
+            hi[ni] = has_hi ? h : (v4i){0, 0, 0, 0};
+        }
+    };
+    auto compute = [&](int stage, const v4i* lo, const v4i* hi) {
+#pragma unroll
+        for (int mi = 0; mi < MR; mi++) {
+            const int row = mi * 16 + li;
+            const v4i alo = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
+            const v4i ahi = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
+            if constexpr (KIND == KIND_INT8) {
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    acc[mi][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo[ni], alo, acc[mi][ni], 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi[ni], ahi, acc[mi][ni], 0, 0, 0);
+                }
+            } else {
+                const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    const v8i bf = {lo[ni][0], lo[ni][1], lo[ni][2], lo[ni][3], hi[ni][0], hi[ni][1], hi[ni][2], hi[ni][3]};
+                    acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[mi][ni], 0, 0, 0, 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    // prologue: stage 0
+    load_a(0);
+    load_b(0, blo[0], bhi[0]);
+    store_a(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; kt += 2) {
+        {  // even step: compute stage 0, prefetch stage 1
+            const bool next = (kt + 1) < KT;
+            if (next) {
+                load_a(kt + 1);
+                load_b(kt + 1, blo[1], bhi[1]);
+            }
+            compute(0, blo[0], bhi[0]);
+            if (next) store_a(1);
+            __syncthreads();
+        }
+        if (kt + 1 < KT) {  // odd step: compute stage 1, prefetch stage 0
+            const bool next = (kt + 2) < KT;
+            if (next) {
+                load_a(kt + 2);
+                load_b(kt + 2, blo[0], bhi[0]);
+            }
+            compute(1, blo[1], bhi[1]);
+            if (next) store_a(0);
+            __syncthreads();
+        }
+    }
+
+    // epilogue: lane owns C[m0 + mi*16 + li][n0 + (wave*NR + ni)*16 + lg*4 + 0..3]
+#pragma unroll
+    for (int mi = 0; mi < MR; mi++) {
+        const int m = m0 + mi * 16 + li;
+        if (m >= p.M) continue;
+        float sa = 0.f;
+        if constexpr (STORE == STORE_C) sa = p.sa[m];
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) {
+            const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+            if (n >= p.N) continue;
+            const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
+            if constexpr (STORE == STORE_ACC) {
+                *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = acc[mi][ni];
+            } else {
+                const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
+                float x[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) x[e] = ((float)acc[mi][ni][e] * sa) * sb[e];
+                store_c4(p, idx, n, x);
+            }
+        }
+    }
+}
+
+template <int KIND, int MR, int NR, int STORE>
+hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
+    constexpr int TM = 16 * MR, TN = 64 * NR;
+    const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, STORE>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <int KIND, int STORE>
+hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t stream) {
+#define PSG_CASE(MR_, NR_) \
+    if (tile_m == 16 * MR_ && tile_n == 64 * NR_) return launch_one<KIND, MR_, NR_, STORE>(p, stream);
+    PSG_CASE(16, 4)
+    PSG_CASE(8, 4)
+    PSG_CASE(4, 4)
+    PSG_CASE(2, 4)
+    PSG_CASE(8, 2)
+    PSG_CASE(4, 1)
+#undef PSG_CASE
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace
+
+// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8.  tile_m x tile_n must be one of the
+// instantiated shapes: 256x256, 128x256, 64x256, 32x256, 128x128, 64x64.
+hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
+    if (kind == KIND_INT8) {
+        if (store == STORE_ACC) return launch_shape<KIND_INT8, STORE_ACC>(p, tile_m, tile_n, stream);
+        return launch_shape<KIND_INT8, STORE_C>(p, tile_m, tile_n, stream);
+    }
+    if (kind == KIND_FP8) {
+        if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);
+        return launch_shape<KIND_FP8, STORE_C>(p, tile_m, tile_n, stream);
+    }
+    return hipErrorInvalidValue;
+}

@@ -1,0 +1,205 @@
+// C ABI of libpsgemm.so: argument validation, regime selection and launch on the caller's stream.
+// Nothing here allocates, synchronises or touches any stream but the caller's.
+#include "../../include/psgemm.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "psg_common.h"
+
+hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
+hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, hipStream_t stream);
+hipError_t psg_launch_mxfp4_tiled(const MxParams& p, int store, int tile_m, int tile_n, hipStream_t stream);
+hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    return (int)e;
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+constexpr int kSmallM = 32;      // rows the split-K path covers
+constexpr int kTargetWaves = 2048;  // wavefronts wanted in flight for the streaming path (8 per CU)
+
+int pick_ksplit(int units, int steps) {
+    int ks = 1;
+    while (ks < 8 && units * ks < kTargetWaves && ks * 2 <= steps) ks *= 2;
+    return ks;
+}
+
+struct Tile {
+    int m, n;
+};
+
+// Tile choice for the MFMA mainloop: widest N tile that N supports, then the M tile with the best
+// product of CU fill, padding efficiency and per-tile efficiency (bigger tiles reuse operands more).
+Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
+    static const int shapes8[][2] = {{256, 256}, {128, 256}, {64, 256}, {32, 256}, {128, 128}, {64, 64}};
+    static const int shapesx[][2] = {{256, 256}, {128, 256}, {64, 256}, {32, 256}, {64, 128}, {32, 128}};
+    const int(*shapes)[2] = mx ? shapesx : shapes8;
+    for (int i = 0; i < 6; i++)
+        if (shapes[i][0] == hint_m && shapes[i][1] == hint_n) return {hint_m, hint_n};
+    double best = -1.0;
+    Tile t = {shapes[0][0], shapes[0][1]};
+    for (int i = 0; i < 6; i++) {
+        const int tm = shapes[i][0], tn = shapes[i][1];
+        const long tiles_m = (M + tm - 1) / tm, tiles_n = (N + tn - 1) / tn;
+        const long tiles = tiles_m * tiles_n;
+        const long rounds = (tiles + 255) / 256;
+        const double fill = (double)tiles / (double)(rounds * 256);
+        const double pad = ((double)M / (double)(tiles_m * tm)) * ((double)N / (double)(tiles_n * tn));
+        // operand bytes fetched per MFMA: (tm + tn) / (tm * tn), relative to the 256x256 tile
+        const double reuse = (2.0 / 256.0) / ((double)(tm + tn) / ((double)tm * tn));
+        const double score = fill * pad * (0.35 + 0.65 * reuse);
+        if (score > best) {
+            best = score;
+            t = {tm, tn};
+        }
+    }
+    return t;
+}
+
+int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!a->a || !a->b) return fail(PSG_E_NULL, "a and b must be non-NULL");
+    if (acc_only) {
+        if (!acc) return fail(PSG_E_NULL, "acc must be non-NULL");
+    } else {
+        if (!a->c) return fail(PSG_E_NULL, "c must be non-NULL");
+        if (!a->scale_a || !a->scale_b) return fail(PSG_E_NULL, "scale_a and scale_b must be non-NULL for 8-bit inputs");
+        if (a->epilogue != PSG_EPI_NONE && !a->bias) return fail(PSG_E_NULL, "bias must be non-NULL when epilogue != none");
+    }
+    if (a->in_dtype == PSG_IN_FP16 || a->in_dtype == PSG_IN_BF16)
+        return fail(PSG_E_UNSUPPORTED, "fp16/bf16 inputs are not built in this library yet");
+    if (a->in_dtype != PSG_IN_INT8 && a->in_dtype != PSG_IN_FP8_E4M3FN) return fail(PSG_E_DTYPE, "in_dtype %d unknown", a->in_dtype);
+    if (a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
+    if (a->epilogue < PSG_EPI_NONE || a->epilogue > PSG_EPI_BIAS_GELU) return fail(PSG_E_DTYPE, "epilogue %d unknown", a->epilogue);
+    if (a->M < 1 || a->M > 65536) return fail(PSG_E_SHAPE, "M=%d outside [1, 65536]", a->M);
+    if (a->N < 16 || a->N % 16) return fail(PSG_E_SHAPE, "N=%d must be a positive multiple of 16", a->N);
+    if (a->K < 64 || a->K % 64) return fail(PSG_E_SHAPE, "K=%d must be a positive multiple of 64", a->K);
+    if ((uint64_t)a->N * (uint64_t)a->K > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "N*K=%llu exceeds the 4 GiB descriptor range", (unsigned long long)a->N * a->K);
+    if (!aligned(a->a, 16) || !aligned(a->b, 16)) return fail(PSG_E_ALIGN, "a and b must be 16-byte aligned");
+    if (acc_only) {
+        if (!aligned(acc, 16)) return fail(PSG_E_ALIGN, "acc must be 16-byte aligned");
+    } else {
+        if (!aligned(a->c, 8)) return fail(PSG_E_ALIGN, "c must be 8-byte aligned");
+        if (!aligned(a->scale_b, 16)) return fail(PSG_E_ALIGN, "scale_b must be 16-byte aligned");
+        if (!aligned(a->scale_a, 4)) return fail(PSG_E_ALIGN, "scale_a must be 4-byte aligned");
+        if (a->epilogue != PSG_EPI_NONE && !aligned(a->bias, 8)) return fail(PSG_E_ALIGN, "bias must be 8-byte aligned");
+    }
+    if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
+    if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    return 0;
+}
+
+int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
+    A8W8Params p;
+    p.c = out;
+    p.a = static_cast<const uint8_t*>(a->a);
+    p.b = static_cast<const uint8_t*>(a->b);
+    p.sa = a->scale_a;
+    p.sb = a->scale_b;
+    p.bias = static_cast<const uint16_t*>(a->bias);
+    p.M = a->M;
+    p.N = a->N;
+    p.K = a->K;
+    p.epi = a->epilogue;
+    p.out = a->out_dtype;
+    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 4;
+    const int kind = a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : KIND_FP8;
+    const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
+    hipError_t e;
+    if (small) {
+        p.ksplit = pick_ksplit(a->N / 16, (a->K + 127) / 128);
+        e = psg_launch_a8w8_smallm(p, kind, store, static_cast<hipStream_t>(stream));
+    } else {
+        const Tile t = pick_tile(a->M, a->N, false, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
+        p.ksplit = 1;
+        e = psg_launch_a8w8_tiled(p, kind, store, t.m, t.n, static_cast<hipStream_t>(stream));
+    }
+    if (e != hipSuccess) return hip_fail(e, "psg_gemm_a8w8 launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int psg_abi_version(void) { return PSG_ABI_VERSION; }
+
+const char* psg_last_error(void) { return g_err; }
+
+uint64_t psg_workspace_bytes(int32_t, int32_t, int32_t, int32_t) {
+    // Both regimes reduce inside one workgroup (registers / LDS); no global scratch is needed.
+    return 0;
+}
+
+int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
+    if (int rc = validate_a8w8(args, false, nullptr)) return rc;
+    return run_a8w8(args, args->c, STORE_C, stream);
+}
+
+int psg_gemm_a8w8_acc(const psg_a8w8_args* args, void* acc, void* stream) {
+    if (int rc = validate_a8w8(args, true, acc)) return rc;
+    return run_a8w8(args, acc, STORE_ACC, stream);
+}
+
+static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!out || !a->a || !a->b || !a->scale_a || !a->scale_b) return fail(PSG_E_NULL, "c, a, b, scale_a, scale_b must be non-NULL");
+    if (a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
+    if (a->M < 1 || a->M > 65536) return fail(PSG_E_SHAPE, "M=%d outside [1, 65536]", a->M);
+    if (a->N < 32 || a->N % 32) return fail(PSG_E_SHAPE, "N=%d must be a positive multiple of 32", a->N);
+    if (a->K < 256 || a->K % 256) return fail(PSG_E_SHAPE, "K=%d must be a positive multiple of 256", a->K);
+    if ((uint64_t)a->N * (uint64_t)a->K / 2 > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "N*K/2 exceeds the 4 GiB descriptor range");
+    if (!aligned(a->a, 16) || !aligned(a->b, 16)) return fail(PSG_E_ALIGN, "a and b must be 16-byte aligned");
+    if (!aligned(a->scale_a, 4) || !aligned(a->scale_b, 4)) return fail(PSG_E_ALIGN, "scales must be 4-byte aligned");
+    if (!aligned(out, store == STORE_ACC ? 16 : 8)) return fail(PSG_E_ALIGN, "output must be %d-byte aligned", store == STORE_ACC ? 16 : 8);
+    if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
+    if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    MxParams p;
+    p.c = out;
+    p.a = static_cast<const uint8_t*>(a->a);
+    p.b = static_cast<const uint8_t*>(a->b);
+    p.sa = static_cast<const uint8_t*>(a->scale_a);
+    p.sb = static_cast<const uint8_t*>(a->scale_b);
+    p.M = a->M;
+    p.N = a->N;
+    p.K = a->K;
+    p.out = a->out_dtype;
+    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 4;
+    const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
+    hipError_t e;
+    if (small) {
+        p.ksplit = pick_ksplit(a->N / 32, a->K / 256);
+        e = psg_launch_mxfp4_smallm(p, store, static_cast<hipStream_t>(stream));
+    } else {
+        const Tile t = pick_tile(a->M, a->N, true, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
+        p.ksplit = 1;
+        e = psg_launch_mxfp4_tiled(p, store, t.m, t.n, static_cast<hipStream_t>(stream));
+    }
+    if (e != hipSuccess) return hip_fail(e, "psg_gemm_mxfp4 launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+int psg_gemm_mxfp4(const psg_mxfp4_args* args, void* stream) { return mx_common(args, args ? args->c : nullptr, STORE_C, stream); }
+
+int psg_gemm_mxfp4_acc(const psg_mxfp4_args* args, void* acc, void* stream) { return mx_common(args, acc, STORE_ACC, stream); }
+
+}  // extern "C"

@@ -1,0 +1,156 @@
+// Shared device helpers for the preshuffle GEMM kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3 };
+enum { OUT_BF16 = 0, OUT_FP16 = 1 };
+enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_RELU = 2, EPI_BIAS_SILU = 3, EPI_BIAS_GELU = 4 };
+// what a kernel writes: the scaled/activated C, or the raw accumulators
+enum { STORE_C = 0, STORE_ACC = 1 };
+
+// Raw buffer resource over [base, base+bytes): loads past the end return 0, stores past it are dropped.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint64_t bytes) {
+    uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
+__device__ __forceinline__ v4i buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+}
+
+// non-temporal variant for data that is streamed exactly once
+__device__ __forceinline__ v4i buf_load16_nt(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 2);
+}
+
+__device__ __forceinline__ int buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return (int)__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
+}
+
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// bias / activation of the fused epilogue, fp32 in, fp32 out
+template <int EPI>
+__device__ __forceinline__ float epi_act(float v, float bias) {
+    if constexpr (EPI != EPI_NONE) v = v + bias;
+    if constexpr (EPI == EPI_BIAS_RELU) v = fmaxf(v, 0.0f);
+    if constexpr (EPI == EPI_BIAS_SILU) {
+        float e = __expf(-v);
+        v = v * (1.0f / (1.0f + e));
+    }
+    if constexpr (EPI == EPI_BIAS_GELU) {
+        float x3 = v * v * v;
+        float y = 0.7978845608f * (v + 0.044715f * x3);
+        float e = __expf(-2.0f * fabsf(y));
+        float num = y > 0.0f ? 2.0f : 2.0f * e;
+        v = 0.5f * v * (num * (1.0f / (1.0f + e)));
+    }
+    return v;
+}
+
+template <int OUT>
+__device__ __forceinline__ uint16_t to_out16(float v) {
+    if constexpr (OUT == OUT_BF16) {
+        __bf16 h = (__bf16)v;
+        return __builtin_bit_cast(uint16_t, h);
+    } else {
+        _Float16 h = (_Float16)v;
+        return __builtin_bit_cast(uint16_t, h);
+    }
+}
+
+template <int OUT>
+__device__ __forceinline__ float from_out16(uint16_t b) {
+    if constexpr (OUT == OUT_BF16) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    } else {
+        return (float)__builtin_bit_cast(_Float16, b);
+    }
+}
+
+// four fp32 -> four 16-bit outputs packed into 8 bytes
+template <int OUT>
+__device__ __forceinline__ v2i pack4_out16(float a, float b, float c, float d) {
+    v2i r;
+    r[0] = (int)((uint32_t)to_out16<OUT>(a) | ((uint32_t)to_out16<OUT>(b) << 16));
+    r[1] = (int)((uint32_t)to_out16<OUT>(c) | ((uint32_t)to_out16<OUT>(d) << 16));
+    return r;
+}
+
+// Arguments shared by the 8-bit kernels.  Plain data, passed by value.
+struct A8W8Params {
+    void* c;             // [M,N] out16, or raw accumulators when STORE_ACC
+    const uint8_t* a;    // [M,K]
+    const uint8_t* b;    // preshuffled [N,K]
+    const float* sa;     // [M]
+    const float* sb;     // [N]
+    const uint16_t* bias;  // [N] out16
+    int M, N, K;
+    int group_m;  // M-tiles per group of the XCD-aware tile order (tiled kernel)
+    int ksplit;   // K splits per n-block (small-M kernel)
+    int epi;      // EPI_*
+    int out;      // OUT_*
+};
+
+struct MxParams {
+    void* c;
+    const uint8_t* a;    // [M,K/2]
+    const uint8_t* b;    // preshuffled [N,K/2]
+    const uint8_t* sa;   // shuffled e8m0 [ceil(M/32)*32, K/32]
+    const uint8_t* sb;   // shuffled e8m0 [N, K/32]
+    int M, N, K;
+    int group_m;
+    int ksplit;
+    int out;  // OUT_*
+};
+
+// bias + activation + 16-bit conversion of four consecutive columns, chosen at run time (the epilogue is
+// a vanishing part of any launch, so it is not worth a kernel instantiation per variant)
+template <int OUT>
+__device__ __forceinline__ v2i finish4(const float* x, const uint16_t* bias_n, int epi) {
+    float b[4] = {0.f, 0.f, 0.f, 0.f};
+    if (epi != EPI_NONE) {
+        const v2i braw = *reinterpret_cast<const v2i*>(bias_n);
+        b[0] = from_out16<OUT>((uint16_t)(braw[0] & 0xFFFF));
+        b[1] = from_out16<OUT>((uint16_t)((uint32_t)braw[0] >> 16));
+        b[2] = from_out16<OUT>((uint16_t)(braw[1] & 0xFFFF));
+        b[3] = from_out16<OUT>((uint16_t)((uint32_t)braw[1] >> 16));
+    }
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        switch (epi) {
+            case EPI_BIAS: v[e] = epi_act<EPI_BIAS>(x[e], b[e]); break;
+            case EPI_BIAS_RELU: v[e] = epi_act<EPI_BIAS_RELU>(x[e], b[e]); break;
+            case EPI_BIAS_SILU: v[e] = epi_act<EPI_BIAS_SILU>(x[e], b[e]); break;
+            case EPI_BIAS_GELU: v[e] = epi_act<EPI_BIAS_GELU>(x[e], b[e]); break;
+            default: v[e] = x[e]; break;
+        }
+    }
+    return pack4_out16<OUT>(v[0], v[1], v[2], v[3]);
+}
+
+// store four consecutive columns of row-major 16-bit C starting at element index idx (column n)
+template <class P>
+__device__ __forceinline__ void store_c4(const P& p, size_t idx, int n, const float* x) {
+    v2i r = p.out == OUT_BF16 ? finish4<OUT_BF16>(x, p.bias + n, p.epi) : finish4<OUT_FP16>(x, p.bias + n, p.epi);
+    *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(p.c) + idx) = r;
+}

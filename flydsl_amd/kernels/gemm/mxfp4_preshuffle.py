@@ -1,0 +1,96 @@
+"""MXFP4 preshuffle GEMM entry point (e2m1 x e2m1, e8m0 scale per 32 K elements).
+
+Drop-in for the reference's ``launch_gemm`` (kernels/gemm/mxfp4_preshuffle.py:57-91): same positional
+signature.  Operands are raw device pointers (what ``flyc.from_c_void_p(fx.Uint8, t.data_ptr())``
+produces: an object with an integer ``value``, or a plain int, or a tensor).  Supported subset:
+``a_dtype == b_dtype == "fp4"``, ``batch == 1`` and all strides ``-1``; the rest raises
+``NotImplementedError``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+from ... import _lib
+
+
+def _addr(x) -> int:
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return int(x.data_ptr())
+    v = getattr(x, "value", None)
+    if v is None:
+        raise TypeError(f"cannot take a device address from {type(x).__name__}")
+    return int(v)
+
+
+def launch_gemm(
+    arg_c,
+    arg_a,
+    arg_b,
+    arg_scale_a,
+    arg_scale_b,
+    i32_m,
+    i32_n,
+    stream,
+    N,
+    K,
+    tile_m,
+    tile_n,
+    tile_k,
+    a_dtype,
+    out_dtype,
+    b_dtype,
+    batch,
+    a_row_stride,
+    a_batch_stride,
+    sca_row_stride,
+    sca_batch_stride,
+    c_row_stride,
+    c_batch_stride,
+    waves_per_eu,
+    xcd_swizzle=0,
+    *,
+    _force_path=0,
+    _tile=None,
+    _acc=None,
+):
+    """Launch ``C[M,N] = A_mx[M,K] @ W_mx[N,K]^T`` on ``stream``.  The reference's constraints are kept:
+    ``tile_k in {128, 256}``, ``tile_n % 128 == 0``, ``K % tile_k == 0`` (mxfp4_preshuffle.py:122,316)."""
+    if a_dtype != "fp4" or b_dtype != "fp4":
+        raise NotImplementedError(f"only fp4 x fp4 is built (got a_dtype={a_dtype!r}, b_dtype={b_dtype!r})")
+    if int(batch) != 1:
+        raise NotImplementedError("strided-batched launch (batch > 1) is not built")
+    if any(int(s) >= 0 for s in (a_row_stride, a_batch_stride, sca_row_stride, sca_batch_stride, c_row_stride, c_batch_stride)):
+        raise NotImplementedError("caller-controlled row/batch strides are not built; pass -1")
+    if out_dtype not in _lib.OUT_DTYPE:
+        raise ValueError(f"out_dtype must be bf16/fp16, got {out_dtype!r}")
+    if tile_k not in (128, 256):
+        raise ValueError(f"tile_k must be 128 or 256, got {tile_k}")
+    if tile_n % 128 != 0:
+        raise ValueError(f"tile_n must be a multiple of 128, got {tile_n}")
+    if K % tile_k != 0:
+        raise ValueError(f"K={K} must be a multiple of tile_k={tile_k}")
+    if int(i32_n) != int(N):
+        raise ValueError(f"runtime N={i32_n} differs from the compile-time N={N}")
+    args = _lib.MxArgs()
+    args.c = _addr(arg_c) if _acc is None else None
+    args.a = _addr(arg_a)
+    args.b = _addr(arg_b)
+    args.scale_a = _addr(arg_scale_a)
+    args.scale_b = _addr(arg_scale_b)
+    args.M, args.N, args.K = int(i32_m), int(N), int(K)
+    args.out_dtype = _lib.OUT_DTYPE[out_dtype]
+    args.tile_m, args.tile_n, args.tile_k = int(tile_m), int(tile_n), int(tile_k)
+    if _tile is not None:
+        args.tile_m, args.tile_n = int(_tile[0]), int(_tile[1])
+    args.xcd_swizzle = int(xcd_swizzle)
+    args.force_path = int(_force_path)
+    lib = _lib.lib()
+    if _acc is None:
+        rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))
+    else:
+        rc = lib.psg_gemm_mxfp4_acc(ctypes.byref(args), _addr(_acc), _lib.stream_handle(stream))
+    if rc:
+        _lib.check(rc, "psg_gemm_mxfp4")

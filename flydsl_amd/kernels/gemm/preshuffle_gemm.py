@@ -1,0 +1,147 @@
+"""Preshuffle GEMM entry point (int8 / OCP fp8 per-token x per-channel scaled, bf16/fp16 out).
+
+Drop-in for the reference's ``compile_preshuffle_gemm`` (kernels/gemm/preshuffle_gemm.py:108-128):
+same keyword-only signature and defaults, same ``ValueError`` conditions, and the returned callable
+keeps the call shape ``fn(C, A, B, scale_a, scale_b, bias, M, N, stream)`` with ``M`` a run-time
+argument.  Underneath there is no JIT: the call fills a plain C struct and enters ``libpsgemm.so``.
+
+The reference's tuning keywords (``tile_*``, ``waves_per_eu``, ``enable_scheduler``,
+``use_async_copy``, ``xcd_swizzle``, ``lds_stage``, ``preload``) are validated exactly as the
+reference validates them and then treated as hints: the native dispatcher picks its own tiling per
+regime (MFMA mainloop for M > 32, split-K streaming kernel for M <= 32).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+from ... import _lib
+
+_A_COPY_GRANULARITY = 256 * 16  # threads x bytes per load of the reference's A-tile copy
+
+
+def _validate(N, K, tile_m, tile_n, tile_k, in_dtype, out_dtype, epilogue, use_async_copy, lds_stage, preload):
+    # kernels/gemm/preshuffle_gemm.py:129-136
+    if in_dtype not in ("fp8", "int8", "fp16", "bf16"):
+        raise ValueError(f"in_dtype must be fp8/int8/fp16/bf16, got {in_dtype!r}")
+    if tile_k <= 0 or K % tile_k != 0:
+        raise ValueError(f"tile_k must be a positive divisor of K; got tile_k={tile_k}, K={K}")
+    if epilogue not in _lib.EPILOGUE:
+        raise ValueError(f"epilogue must be none/bias/bias_relu/bias_silu/bias_gelu, got {epilogue!r}")
+    if lds_stage not in (1, 2):
+        raise ValueError(f"lds_stage must be 1 or 2, got {lds_stage}")
+    if out_dtype not in _lib.OUT_DTYPE:
+        raise ValueError(f"out_dtype must be bf16/fp16, got {out_dtype!r}")
+    elem_bytes = 1 if in_dtype in ("fp8", "int8") else 2
+    # :188-196 -- the reference's A-tile copy must divide evenly over 256 threads x 16 bytes
+    a_tile_bytes = tile_m * tile_k * elem_bytes
+    if a_tile_bytes % _A_COPY_GRANULARITY != 0:
+        raise ValueError(
+            f"tile_m * tile_k * elem_bytes must be a multiple of {_A_COPY_GRANULARITY} "
+            f"(total_threads * a_load_bytes); got tile_m={tile_m}, tile_k={tile_k}, "
+            f"elem_bytes={elem_bytes} -> {a_tile_bytes} bytes, leaving "
+            f"{a_tile_bytes % _A_COPY_GRANULARITY} bytes of the A tile unloaded"
+        )
+    # :200-203
+    if preload is not None:
+        if len(preload) != 2 or any(not isinstance(v, int) or v < 0 for v in preload):
+            raise ValueError(f"preload must be a pair of non-negative ints, got {preload!r}")
+    # :289-296 -- LDS swizzle width of the 8-bit / async path must be a power of two
+    if elem_bytes == 1 or use_async_copy:
+        k_blocks16 = (tile_k * elem_bytes) // 16
+        if k_blocks16 <= 0 or (k_blocks16 & (k_blocks16 - 1)) != 0:
+            raise ValueError(
+                f"Unsupported tile_k for LDS swizzle: tile_k={tile_k}, elem_bytes={elem_bytes} "
+                f"(k_blocks16={k_blocks16}); expected tile_k*elem_bytes to be a positive multiple "
+                "of 16 with (tile_k*elem_bytes/16) a power of two."
+            )
+    # layout requirements the reference leaves implicit (asserts in shuffle_weight, tests/utils.py:86-87)
+    if N % 16 != 0:
+        raise ValueError(f"N must be a multiple of 16 (preshuffled B layout), got {N}")
+    if (K * elem_bytes) % 64 != 0:
+        raise ValueError(f"K*elem_bytes must be a multiple of 64 (preshuffled B layout), got K={K}")
+
+
+class PreshuffleGemm:
+    """Launcher returned by :func:`compile_preshuffle_gemm`.  Holds no tensor references."""
+
+    def __init__(self, N, K, in_dtype, out_dtype, epilogue, tile_m, tile_n, tile_k, xcd_swizzle):
+        self.N, self.K = int(N), int(K)
+        self.in_dtype, self.out_dtype, self.epilogue = in_dtype, out_dtype, epilogue
+        self._lib = _lib.lib()
+        args = _lib.A8W8Args()
+        args.N, args.K = self.N, self.K
+        args.in_dtype = _lib.IN_DTYPE[in_dtype]
+        args.out_dtype = _lib.OUT_DTYPE[out_dtype]
+        args.epilogue = _lib.EPILOGUE[epilogue]
+        args.tile_m, args.tile_n, args.tile_k = int(tile_m), int(tile_n), int(tile_k)
+        args.xcd_swizzle = int(xcd_swizzle)
+        self._proto = args
+
+    def _fill(self, C, A, B, scale_a, scale_b, bias, M, N):
+        if int(N) != self.N:
+            raise ValueError(f"N={N} differs from the N={self.N} this launcher was built for")
+        args = _lib.A8W8Args()
+        ctypes.memmove(ctypes.byref(args), ctypes.byref(self._proto), ctypes.sizeof(args))
+        args.c = C.data_ptr()
+        args.a = A.data_ptr()
+        args.b = B.data_ptr()
+        args.scale_a = scale_a.data_ptr() if scale_a is not None and scale_a.numel() else None
+        args.scale_b = scale_b.data_ptr() if scale_b is not None and scale_b.numel() else None
+        args.bias = bias.data_ptr() if bias is not None and bias.numel() else None
+        args.M = int(M)
+        return args
+
+    def __call__(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
+        args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
+        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
+        if rc:
+            _lib.check(rc, "psg_gemm_a8w8")
+
+    def accumulators(self, acc, A, B, M, N, stream=None, force_path=0, tile=None):
+        """Write the raw accumulators ``[M, N]`` (int32 for int8, fp32 for fp8) into ``acc``."""
+        args = self._fill(acc, A, B, None, None, None, M, N)
+        args.force_path = int(force_path)
+        if tile is not None:
+            args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
+        rc = self._lib.psg_gemm_a8w8_acc(ctypes.byref(args), acc.data_ptr(), _lib.stream_handle(stream))
+        if rc:
+            _lib.check(rc, "psg_gemm_a8w8_acc")
+
+    def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None):
+        """Like ``__call__`` but pins the regime (1 = MFMA mainloop, 2 = small-M) and optionally the
+        native tile ``(tile_m, tile_n)``; for tests and benchmarks."""
+        args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
+        args.force_path = int(force_path)
+        if tile is not None:
+            args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
+        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
+        if rc:
+            _lib.check(rc, "psg_gemm_a8w8")
+
+
+def compile_preshuffle_gemm(
+    *,
+    N: int,
+    K: int,
+    tile_m: int,
+    tile_n: int,
+    tile_k: int,
+    in_dtype: str = "fp8",
+    out_dtype: str = "bf16",
+    epilogue: str = "none",
+    waves_per_eu: Optional[int] = None,
+    enable_scheduler: bool = True,
+    use_async_copy: bool = False,
+    xcd_swizzle: int = 0,
+    lds_stage: int = 2,
+    preload: Optional[tuple] = None,
+):
+    """Build the preshuffle GEMM launcher.  Signature of the result:
+    ``fn(C, A, B, scale_a, scale_b, bias, M, N, stream)``; ``bias`` is per-N in ``out_dtype`` and is
+    only read when ``epilogue != "none"``."""
+    _validate(N, K, tile_m, tile_n, tile_k, in_dtype, out_dtype, epilogue, use_async_copy, lds_stage, preload)
+    if in_dtype in ("fp16", "bf16"):
+        raise NotImplementedError(f"in_dtype={in_dtype!r}: 16-bit inputs are not built in this library yet")
+    return PreshuffleGemm(N, K, in_dtype, out_dtype, epilogue, tile_m, tile_n, tile_k, xcd_swizzle)

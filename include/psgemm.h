@@ -1,0 +1,147 @@
+/*
+ * psgemm.h -- C ABI of the MI355X-native preshuffle quantized GEMM library (libpsgemm.so).
+ *
+ *   C[M,N] = A[M,K] * B[N,K]^T      B preshuffled into MFMA-fragment order on the host
+ *
+ * Plain pointers and sizes only; no framework types.  Every pointer is a DEVICE pointer owned by
+ * the caller and only borrowed for the duration of the (asynchronous) launch.  Every launch goes to
+ * the caller's stream and nothing else touches the device: no allocation, no synchronisation, no
+ * default-stream work, so calls may be recorded into a HIP graph.  Entry points are re-entrant.
+ *
+ * Return value of every int function: 0 = ok, negative = argument validation failed (PSG_E_*),
+ * positive = hipError_t of a failed HIP call.  psg_last_error() returns a thread-local message.
+ *
+ * What each entry point replaces in the reference (paths relative to the reference tree):
+ *   psg_gemm_a8w8       the compiled launcher returned by compile_preshuffle_gemm()
+ *                       kernels/gemm/preshuffle_gemm.py:717-806 (launch_gemm) + :220-714 (kernel_gemm),
+ *                       reached through the JIT host stub -> mgpuLaunchKernel
+ *                       lib/Runtime/ROCm/FlyRocmRuntimeWrappers.cpp:58-64
+ *   psg_gemm_a8w8_acc   no counterpart: the reference never exposes accumulators; this dumps them
+ *                       (int32 for int8, fp32 for fp8) so parity tests can check them bit-exactly
+ *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm), fp4 x fp4, batch 1
+ *   psg_gemm_mxfp4_acc  no counterpart: fp32 accumulators of the MXFP4 mainloop, for parity tests
+ *   psg_workspace_bytes no counterpart (the reference has no split-K path)
+ */
+#ifndef PSGEMM_H
+#define PSGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PSG_ABI_VERSION 1
+
+/* input element types of A and B */
+enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
+/* output element types of C */
+enum psg_out_dtype { PSG_OUT_BF16 = 0, PSG_OUT_FP16 = 1 };
+/* fused epilogue, as the reference's `epilogue` keyword (kernels/gemm/preshuffle_gemm.py:118) */
+enum psg_epilogue {
+    PSG_EPI_NONE = 0,
+    PSG_EPI_BIAS = 1,
+    PSG_EPI_BIAS_RELU = 2,
+    PSG_EPI_BIAS_SILU = 3,
+    PSG_EPI_BIAS_GELU = 4
+};
+
+/* validation errors (negative return values) */
+enum psg_error {
+    PSG_E_NULL = -1,        /* a required pointer is NULL */
+    PSG_E_SHAPE = -2,       /* M/N/K violate the layout's divisibility or range rules */
+    PSG_E_DTYPE = -3,       /* unsupported dtype / epilogue combination */
+    PSG_E_WORKSPACE = -4,   /* workspace missing or too small for this call */
+    PSG_E_UNSUPPORTED = -5, /* valid in the reference but not built here (says which in the message) */
+    PSG_E_ALIGN = -6        /* a pointer is not 16-byte aligned */
+};
+
+/*
+ * Arguments of the 8-bit (and 16-bit) preshuffle GEMM.
+ *   c        [M,N] row-major, out_dtype; rows >= M of the allocation are never written
+ *   a        [M,K] row-major, 1 byte/element (int8 or e4m3fn); rows >= M are never read
+ *   b        preshuffle of W[N,K]: byte of W[n,k] at
+ *            (n/16)*16K + (k/64)*1024 + ((k%64)/16)*256 + (n%16)*16 + k%16      (tests/utils.py:76-96)
+ *   scale_a  [M] fp32 per-token scales; scale_b [N] fp32 per-channel scales
+ *   bias     [N] out_dtype, read only when epilogue != PSG_EPI_NONE
+ *   N % 16 == 0, K % 64 == 0, 1 <= M <= 65536 (kernels/gemm/preshuffle_gemm.py:783-785)
+ *   workspace / workspace_bytes: scratch for the small-M split-K path; may be NULL/0 when
+ *            psg_workspace_bytes() returns 0 for the same (M,N,K,in_dtype).  Contents need no
+ *            initialisation beyond being zero the first time the buffer is used; the kernels leave
+ *            it zeroed again.  Two launches that may overlap in time must not share one workspace.
+ *   tile_m/tile_n/tile_k, xcd_swizzle: the reference's tuning keywords; accepted as hints
+ *            (0 = library's choice).  The library picks its own tiling per regime.
+ */
+typedef struct psg_a8w8_args {
+    void *c;
+    const void *a;
+    const void *b;
+    const float *scale_a;
+    const float *scale_b;
+    const void *bias;
+    void *workspace;
+    uint64_t workspace_bytes;
+    int32_t M, N, K;
+    int32_t in_dtype;  /* enum psg_in_dtype */
+    int32_t out_dtype; /* enum psg_out_dtype */
+    int32_t epilogue;  /* enum psg_epilogue */
+    int32_t tile_m, tile_n, tile_k;
+    int32_t xcd_swizzle;
+    int32_t force_path; /* 0 = auto, 1 = tiled MFMA mainloop, 2 = small-M split-K (tests/benchmarks) */
+    int32_t reserved;
+} psg_a8w8_args;
+
+/*
+ * Arguments of the MXFP4 preshuffle GEMM (fp4 e2m1 x fp4 e2m1, one e8m0 scale per 32 K elements).
+ *   c        [M,N] row-major out_dtype
+ *   a        [M,K/2] row-major packed e2m1, even k in the low nibble
+ *   b        shuffle_weight_w4 of packed W[N,K/2] (same byte map as above with K/2 bytes per row)
+ *   scale_a  shuffle_scale_w4 of e8m0 [ceil(M/32)*32, K/32]; scale_b the same over [N, K/32]
+ *            byte of S[r,kb] at (r/32)*32*(K/32) + (kb/8)*256 + (kb%4)*64 + (r%16)*4 + ((kb%8)/4)*2 + (r%32)/16
+ *            (tests/kernels/utils/gemm_common_utils.py:645-672)
+ *   N % 32 == 0, K % 256 == 0, 1 <= M <= 65536
+ */
+typedef struct psg_mxfp4_args {
+    void *c;
+    const void *a;
+    const void *b;
+    const void *scale_a;
+    const void *scale_b;
+    void *workspace;
+    uint64_t workspace_bytes;
+    int32_t M, N, K;
+    int32_t out_dtype; /* enum psg_out_dtype */
+    int32_t tile_m, tile_n, tile_k;
+    int32_t xcd_swizzle;
+    int32_t force_path; /* 0 = auto, 1 = tiled, 2 = small-M */
+    int32_t reserved;
+} psg_mxfp4_args;
+
+/* ABI version of the loaded library (PSG_ABI_VERSION it was built with). */
+int psg_abi_version(void);
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char *psg_last_error(void);
+
+/* Bytes of workspace psg_gemm_a8w8 needs for this problem (0 when the chosen path needs none). */
+uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype);
+
+/* C = epilogue((acc * scale_a[m]) * scale_b[n]) on `stream` (a hipStream_t passed as void*). */
+int psg_gemm_a8w8(const psg_a8w8_args *args, void *stream);
+
+/* Same mainloop, but writes the raw accumulators [M,N] (int32 for int8, fp32 for fp8) to `acc`
+ * instead of C.  c, scale_a, scale_b, bias are ignored. */
+int psg_gemm_a8w8_acc(const psg_a8w8_args *args, void *acc, void *stream);
+
+/* C = bf16/fp16( sum over 32-blocks of 2^(ea-127) * 2^(eb-127) * dot32(A4, B4) ) on `stream`. */
+int psg_gemm_mxfp4(const psg_mxfp4_args *args, void *stream);
+
+/* Same mainloop, but writes the fp32 accumulators [M,N] to `acc` instead of C (no counterpart in the
+ * reference; parity tests use it to look at the sum before the 16-bit rounding). */
+int psg_gemm_mxfp4_acc(const psg_mxfp4_args *args, void *acc, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PSGEMM_H */

@@ -1,0 +1,469 @@
+"""CPU oracle for the preshuffle quantized GEMM path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing under ``flydsl_amd/`` or ``kernels/`` may import this module; only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` use it, and only as
+the checker.
+
+Everything here is a numpy restatement of what the reference computes on the host (torch CPU)
+for this path.  Each function names the reference lines it follows.  The reference keeps no
+golden vectors for this path, so each function is pinned in ``tests/test_oracle_*.py`` by
+independent means (closed-form index maps, exhaustive code tables, brute force on tiny inputs,
+library casts, float64 cross-checks); the pin for each function is named in its docstring.
+
+All tensors are numpy arrays.  fp8 / fp4 / e8m0 data are carried as ``uint8`` bit patterns.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# ----------------------------------------------------------------------------------------------
+# Codecs
+# ----------------------------------------------------------------------------------------------
+
+#: e2m1 magnitudes by 3-bit code; bit 3 of the 4-bit code is the sign
+#: (tests/kernels/utils/gemm_common_utils.py:31-48).
+E2M1_LUT = np.array(
+    [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0],
+    dtype=np.float32,
+)
+
+
+def e4m3fn_to_f32(code: np.ndarray) -> np.ndarray:
+    """Decode OCP e4m3fn bit patterns (bias 7, no inf, 0x7f/0xff = NaN) to fp32.
+
+    This is what ``tensor.to(torch.float32)`` does for ``torch.float8_e4m3fn`` in the reference's
+    oracle (tests/kernels/test_preshuffle_gemm.py:105-106).  Pinned by comparison with torch's own
+    cast on all 256 codes.
+    """
+    c = np.asarray(code, dtype=np.uint8).astype(np.int32)
+    s = (c >> 7) & 1
+    e = (c >> 3) & 0xF
+    m = c & 7
+    sub = np.ldexp(m.astype(np.float32) / 8.0, -6)
+    nor = np.ldexp(1.0 + m.astype(np.float32) / 8.0, e - 7)
+    v = np.where(e == 0, sub, nor).astype(np.float32)
+    v = np.where((e == 15) & (m == 7), np.float32(np.nan), v)
+    return np.where(s == 1, -v, v).astype(np.float32)
+
+
+_E4M3_TABLE = None
+
+
+def _e4m3_table():
+    global _E4M3_TABLE
+    if _E4M3_TABLE is None:
+        _E4M3_TABLE = e4m3fn_to_f32(np.arange(256, dtype=np.uint8))
+    return _E4M3_TABLE
+
+
+def f32_to_e4m3fn(x: np.ndarray) -> np.ndarray:
+    """fp32 -> e4m3fn bit pattern, round-to-nearest-even, no saturation (|x| >= 465 -> NaN).
+
+    Semantics of ``tensor.to(torch.float8_e4m3fn)`` used by ``pertoken_quant``
+    (tests/utils.py:71).  Pinned against torch's cast on a dense sweep including every midpoint
+    between adjacent codes.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    bits = x.view(np.uint32)
+    sign = ((bits >> 31) & 1).astype(np.uint8)
+    ax = np.abs(x).astype(np.float64)
+    out = np.zeros(x.shape, dtype=np.uint8)
+    nan = np.isnan(x) | (ax >= 480.0)
+    # exponent of the target binade, clamped to the subnormal binade (2^-6)
+    with np.errstate(divide="ignore"):
+        e = np.floor(np.log2(np.where(ax > 0, ax, 1.0))).astype(np.int64)
+    e = np.maximum(e, -6)
+    step = np.ldexp(1.0, e - 3)  # spacing of representable values in this binade
+    q = ax / step  # exact in float64 (power-of-two scaling)
+    r = np.rint(q)  # numpy rint = round half to even
+    val = r * step  # rounded magnitude (may carry into the next binade)
+    # encode the rounded magnitude
+    with np.errstate(divide="ignore"):
+        e2 = np.floor(np.log2(np.where(val > 0, val, 1.0))).astype(np.int64)
+    is_sub = val < 2.0**-6
+    mant_sub = np.rint(val / 2.0**-9).astype(np.int64)  # m/8 * 2^-6
+    mant_nor = np.rint((val / np.ldexp(1.0, e2) - 1.0) * 8.0).astype(np.int64)
+    code = np.where(is_sub, mant_sub, ((e2 + 7) << 3) | mant_nor).astype(np.int64)
+    nan = nan | (code >= 0x7F)
+    code = np.where(nan, 0x7F, code).astype(np.uint8)
+    out = code | (sign << 7).astype(np.uint8)
+    return out.astype(np.uint8)
+
+
+def e8m0_to_f32(b: np.ndarray) -> np.ndarray:
+    """e8m0 byte -> fp32 ``2^(b-127)``; byte 0 -> bits 0x00400000 (2^-127), byte 255 -> NaN.
+
+    tests/kernels/utils/gemm_common_utils.py:63-71.  Pinned on all 256 bytes against ``ldexp``.
+    """
+    b = np.asarray(b, dtype=np.uint8)
+    bits = b.astype(np.uint32) << np.uint32(23)
+    bits = np.where(b == 0, np.uint32(0x00400000), bits)
+    bits = np.where(b == 0xFF, np.uint32(0x7F800001), bits)
+    return bits.astype(np.uint32).view(np.float32)
+
+
+def f32_to_e8m0(x: np.ndarray) -> np.ndarray:
+    """fp32 -> e8m0 byte: biased exponent, plus one when mantissa bit 22 is set and (bit 21 or any
+    lower bit is set or the exponent is non-zero); NaN/Inf exponent stays 0xFF; the increment wraps
+    in uint8 like the reference's.
+
+    tests/kernels/utils/gemm_common_utils.py:53-60.  Pinned on exponent boundaries and the
+    mantissa cases (1.0, 1.25, 1.5-ulp, 1.5, 1.75, subnormals) by hand-computed expectations.
+    """
+    u = np.asarray(x, dtype=np.float32).view(np.uint32)
+    exponent = ((u >> 23) & 0xFF).astype(np.uint8)
+    nan_case = exponent == 0xFF
+    round_case = ((u & 0x400000) > 0) & (((u & 0x200000) > 0) | ((u & 0x1FFFFF) > 0) | (exponent > 0))
+    exponent = np.where(round_case, exponent + np.uint8(1), exponent).astype(np.uint8)
+    exponent = np.where(nan_case, np.uint8(0xFF), exponent).astype(np.uint8)
+    return exponent
+
+
+def f32_to_e2m1(x: np.ndarray) -> np.ndarray:
+    """fp32 -> 4-bit e2m1 code (one code per uint8), round-to-nearest-even, saturating to +-6.
+
+    Follows the bit-level algorithm of ``_f32_to_floatx_unpacked(x, 2, 1)``
+    (tests/kernels/utils/gemm_common_utils.py:162-275): saturate at >= 6, a denormal branch that
+    adds and subtracts a magic constant for |x| < 1, and a normal branch that re-biases the
+    exponent and adds a rounding bias with the tie bit.  Pinned against an independent
+    nearest-value search with ties-to-even on a dense sweep that contains every midpoint.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    ebits, mbits = 2, 1
+    exp_bias = 1
+    max_int = 7
+    magic_adder = (1 << (23 - mbits - 1)) - 1
+    max_normal = 6.0
+    min_normal = 1.0
+    denorm_exp = (127 - exp_bias) + (23 - mbits) + 1
+    denorm_mask_int = np.int32(denorm_exp << 23)
+    denorm_mask_float = np.array(denorm_mask_int, dtype=np.int32).view(np.float32)
+
+    xi = x.view(np.int32)
+    sign = xi & np.int32(-0x80000000)
+    ax_i = xi ^ sign
+    ax = ax_i.view(np.float32)
+
+    saturate = ax >= max_normal
+    denormal = (~saturate) & (ax < min_normal)
+    normal = ~(saturate | denormal)
+
+    with np.errstate(invalid="ignore", over="ignore"):
+        den = (ax + denorm_mask_float).astype(np.float32).view(np.int32) - denorm_mask_int
+    den = (den & 0xFF).astype(np.uint8)
+
+    nor = ax_i.astype(np.int64)
+    mant_odd = (nor >> (23 - mbits)) & 1
+    nor = nor + (((exp_bias - 127) << 23) + magic_adder)
+    nor = nor + mant_odd
+    nor = (nor >> (23 - mbits)) & 0xFF
+    nor = nor.astype(np.uint8)
+
+    out = np.full(x.shape, max_int, dtype=np.uint8)
+    out = np.where(denormal, den, out)
+    out = np.where(normal, nor, out)
+    sign_lp = ((sign.view(np.uint32) >> np.uint32(23 + 8 - mbits - ebits)) & np.uint32(1 << (ebits + mbits))).astype(
+        np.uint8
+    )
+    return (out | sign_lp).astype(np.uint8)
+
+
+def pack_uint4(codes: np.ndarray) -> np.ndarray:
+    """Two 4-bit codes per byte, even index in the LOW nibble
+    (tests/kernels/utils/gemm_common_utils.py:142-147).  Pinned by a two-element example."""
+    codes = np.asarray(codes, dtype=np.uint8)
+    assert codes.shape[-1] % 2 == 0
+    flat = codes.reshape(-1)
+    packed = (flat[1::2] << 4) | (flat[0::2] & 0xF)
+    return packed.reshape(codes.shape[:-1] + (codes.shape[-1] // 2,)).astype(np.uint8)
+
+
+def mxfp4_to_f32(packed: np.ndarray) -> np.ndarray:
+    """Packed e2m1 bytes -> fp32, low nibble first
+    (tests/kernels/utils/gemm_common_utils.py:23-50)."""
+    p = np.asarray(packed, dtype=np.uint8)
+    lo = p & 0xF
+    hi = p >> 4
+    codes = np.stack([lo, hi], axis=-1).reshape(p.shape[:-1] + (p.shape[-1] * 2,))
+    return E2M1_LUT[codes]
+
+
+# ----------------------------------------------------------------------------------------------
+# Host quantisers
+# ----------------------------------------------------------------------------------------------
+
+
+def pertoken_quant(x: np.ndarray, quant: str = "int8"):
+    """Per-row symmetric quantisation (tests/utils.py:29-73).
+
+    ``x`` fp32 ``[R, K]``; ``quant`` is ``"int8"`` (dtypeMax 127, cast truncates toward zero) or
+    ``"fp8"`` (e4m3fn, dtypeMax 448, cast rounds to nearest even).  Returns ``(y, scale)`` with
+    ``y`` int8 / uint8 bit patterns ``[R, K]`` and ``scale`` fp32 ``[R, 1]``.
+
+    Pinned by closed-form invariants (row max maps to +-dtypeMax, zero rows get scale 1,
+    reconstruction error bounds) and by an elementwise comparison with torch's own amax / divide /
+    cast ops.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    dtype_max = np.float32(127.0 if quant == "int8" else 448.0)
+    h = np.nan_to_num(x, nan=0.0, posinf=float(dtype_max), neginf=-float(dtype_max)).astype(np.float32)
+    row_max = h.max(axis=-1, keepdims=True)
+    row_min = h.min(axis=-1, keepdims=True)
+    amax = np.maximum(row_max, -row_min).astype(np.float32)
+    scale = (amax / dtype_max).astype(np.float32)
+    scale[scale == 0] = 1.0
+    scale = np.nan_to_num(scale, nan=1.0, posinf=1.0, neginf=1.0).astype(np.float32)
+    y = (h / scale).astype(np.float32)
+    if quant == "int8":
+        q = np.trunc(y).astype(np.int8)  # torch float->int8 truncates toward zero
+    elif quant == "fp8":
+        q = f32_to_e4m3fn(y)
+    else:
+        raise ValueError(quant)
+    return q, scale
+
+
+def per_1x32_f4_quant(x: np.ndarray):
+    """OCP-MX fp4 quantisation with one e8m0 scale per 32 consecutive K elements
+    (tests/kernels/utils/gemm_common_utils.py:675-704).
+
+    scale byte = ``f32_to_e8m0(amax / 4)``; ``y = x / e8m0_to_f32(scale)``; codes = e2m1 RNE with
+    saturation; packed two per byte.  Returns ``(packed [R, K/2] uint8, scale [R, K/32] uint8)``.
+
+    Pinned through its parts (each codec above is pinned on its own) plus composition invariants:
+    dequantised error is at most half an e2m1 step at the chosen scale unless saturated, the
+    block maximum never decodes above 6*scale, and all-zero blocks give scale byte 0 and zero codes.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    r, k = x.shape
+    assert k % 32 == 0
+    blocks = x.reshape(-1, 32)
+    amax = np.abs(blocks).max(axis=1).astype(np.float32)
+    sc = f32_to_e8m0((amax / np.float32(4.0)).astype(np.float32))
+    sf = e8m0_to_f32(sc)
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = (blocks / sf[:, None]).astype(np.float32)
+    codes = f32_to_e2m1(y)
+    packed = pack_uint4(codes.reshape(r, k))
+    return packed, sc.reshape(r, k // 32)
+
+
+# ----------------------------------------------------------------------------------------------
+# Wire formats
+# ----------------------------------------------------------------------------------------------
+
+
+def shuffle_weight(w: np.ndarray) -> np.ndarray:
+    """Preshuffle ``W[N, K]`` (1- or 2-byte elements) into MFMA-fragment order, layout (16, 16)
+    (tests/utils.py:76-96): ``view(N/16, 16, K/32, 32/Kp, Kp).permute(0, 2, 3, 1, 4)`` with
+    ``Kp = 16 / itemsize`` elements.  Shape and dtype are kept.
+
+    Pinned by the closed-form destination offset and explicit loops on tiny inputs.
+    """
+    w = np.ascontiguousarray(w)
+    n, k = w.shape
+    kp = 16 // w.dtype.itemsize
+    assert n % 16 == 0 and k % 32 == 0
+    v = w.reshape(n // 16, 16, k // 32, 32 // kp, kp).transpose(0, 2, 3, 1, 4)
+    return np.ascontiguousarray(v).reshape(n, k)
+
+
+def shuffle_weight_w4(packed: np.ndarray) -> np.ndarray:
+    """Preshuffle packed fp4 bytes ``[N, K/2]``: ``view(N/16, 16, Kpk/64, 4, 16).permute(0,2,3,1,4)``
+    (tests/kernels/utils/gemm_common_utils.py:634-642, NLane=16, non-MoE)."""
+    p = np.ascontiguousarray(np.asarray(packed, dtype=np.uint8))
+    n, kpk = p.shape
+    assert n % 16 == 0 and kpk % 64 == 0
+    v = p.reshape(n // 16, 16, kpk // 64, 4, 16).transpose(0, 2, 3, 1, 4)
+    return np.ascontiguousarray(v).reshape(n, kpk)
+
+
+def shuffle_scale_w4(scale: np.ndarray) -> np.ndarray:
+    """Permute e8m0 bytes ``[R, K/32]`` -> ``[R/32][K/256][klane 4][nlane 16][kpack 2][npack 2]``
+    (tests/kernels/utils/gemm_common_utils.py:645-672, one expert, not gate_up).
+
+    Pinned by the closed-form destination offset
+    ``(r/32)*32*KB + (kb/8)*256 + (kb%4)*64 + (r%16)*4 + ((kb%8)/4)*2 + (r%32)/16``.
+    """
+    s = np.ascontiguousarray(np.asarray(scale, dtype=np.uint8))
+    r, kb = s.shape
+    assert r % 32 == 0 and kb % 8 == 0
+    v = s.reshape(r // 32, 2, 16, kb // 8, 2, 4).transpose(0, 3, 5, 2, 4, 1)
+    return np.ascontiguousarray(v).reshape(r, kb)
+
+
+# ----------------------------------------------------------------------------------------------
+# GEMM oracles
+# ----------------------------------------------------------------------------------------------
+
+
+def _as_f32_operand(q: np.ndarray, kind: str) -> np.ndarray:
+    if kind == "int8":
+        return np.asarray(q).view(np.int8).astype(np.float32)
+    if kind == "fp8":
+        return _e4m3_table()[np.asarray(q).view(np.uint8)]
+    raise ValueError(kind)
+
+
+def run_torch(a_q, b_q, scale_a, scale_b, kind: str, bias=None) -> np.ndarray:
+    """The reference's parity oracle (tests/kernels/test_preshuffle_gemm.py:103-113): dequantise
+    both operands to fp32 (``a * sa[:, None]``, ``b * sb[:, None]``), fp32 matmul ``a @ b.T``,
+    optional ``+ bias``; fp32 ``[M, N]`` result.  ``b_q`` is the UN-shuffled weight.
+
+    Pinned by a float64 matmul of the same dequantised operands on small shapes.
+    """
+    a32 = _as_f32_operand(a_q, kind) * np.asarray(scale_a, dtype=np.float32).reshape(-1, 1)
+    b32 = _as_f32_operand(b_q, kind) * np.asarray(scale_b, dtype=np.float32).reshape(-1, 1)
+    c = a32 @ b32.T
+    if bias is not None:
+        c = c + np.asarray(bias, dtype=np.float32).reshape(1, -1)
+    return c.astype(np.float32)
+
+
+def int32_accumulators(a_q: np.ndarray, b_q: np.ndarray) -> np.ndarray:
+    """Exact integer matmul ``sum_k int(A[m,k]) * int(B[n,k])`` as int32 ``[M, N]``.
+
+    The reference has no int32 output; this is the accumulator the int8 kernel must hold before
+    its epilogue (kernels/gemm/preshuffle_gemm.py:538,738-740).  Computed in float64 blocks of K
+    small enough to be exact, summed in int64.  Pinned against a pure-integer loop on tiny inputs.
+    """
+    a = np.asarray(a_q).view(np.int8)
+    b = np.asarray(b_q).view(np.int8)
+    m, k = a.shape
+    n = b.shape[0]
+    acc = np.zeros((m, n), dtype=np.int64)
+    step = 1 << 14  # 127*127*16384 < 2^53: each float64 partial is exact
+    for k0 in range(0, k, step):
+        part = a[:, k0 : k0 + step].astype(np.float64) @ b[:, k0 : k0 + step].astype(np.float64).T
+        acc += part.astype(np.int64)
+    assert np.abs(acc).max(initial=0) < 2**31
+    return acc.astype(np.int32)
+
+
+def run_torch_w4(a_packed, b_packed, scale_a, scale_b) -> np.ndarray:
+    """MXFP4 parity oracle (tests/kernels/test_preshuffle_gemm.py:404-411): decode nibbles through
+    the LUT, multiply each 32-element block by ``2^(e-127)``, fp32 matmul.  Operands and scales are
+    UN-shuffled; scale arrays may have more rows than the operands (32-row padding)."""
+    x = mxfp4_to_f32(a_packed)
+    w = mxfp4_to_f32(b_packed)
+    xs = e8m0_to_f32(np.repeat(np.asarray(scale_a, dtype=np.uint8)[: x.shape[0]], 32, axis=1))
+    ws = e8m0_to_f32(np.repeat(np.asarray(scale_b, dtype=np.uint8)[: w.shape[0]], 32, axis=1))
+    return ((x * xs) @ (w * ws).T).astype(np.float32)
+
+
+# ----------------------------------------------------------------------------------------------
+# Epilogue (kernels/gemm/preshuffle_gemm.py:672-714)
+# ----------------------------------------------------------------------------------------------
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit pattern (uint16), round-to-nearest-even, NaN kept quiet."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32)
+    rounded = (u + np.uint32(0x7FFF) + ((u >> 16) & 1)) >> 16
+    nan = np.isnan(np.asarray(x, dtype=np.float32))
+    return np.where(nan, (u >> 16) | 0x40, rounded).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def epilogue_a8w8(acc: np.ndarray, scale_a, scale_b, bias=None, act: str = "none") -> np.ndarray:
+    """Kernel-order epilogue on raw accumulators: ``(f32(acc) * sa[m]) * sb[n]`` then ``+ bias[n]``
+    then the activation, all in fp32 (kernels/gemm/preshuffle_gemm.py:694-714).  Returns fp32."""
+    v = np.asarray(acc).astype(np.float32)
+    v = (v * np.asarray(scale_a, dtype=np.float32).reshape(-1, 1)).astype(np.float32)
+    v = (v * np.asarray(scale_b, dtype=np.float32).reshape(1, -1)).astype(np.float32)
+    return apply_bias_act(v, bias, act)
+
+
+def apply_bias_act(v: np.ndarray, bias=None, act: str = "none") -> np.ndarray:
+    """bias / ReLU / SiLU ``x/(1+e^-x)`` / tanh-GELU in the overflow-safe form
+    (kernels/gemm/preshuffle_gemm.py:672-692)."""
+    v = np.asarray(v, dtype=np.float32)
+    if bias is not None:
+        v = (v + np.asarray(bias, dtype=np.float32).reshape(1, -1)).astype(np.float32)
+    if act == "none":
+        return v
+    if act == "relu":
+        return np.maximum(v, np.float32(0.0))
+    if act == "silu":
+        return (v * (np.float32(1.0) / (np.float32(1.0) + np.exp(-v)))).astype(np.float32)
+    if act == "gelu":
+        y = (np.float32(0.7978845608) * (v + np.float32(0.044715) * v * v * v)).astype(np.float32)
+        e = np.exp(np.float32(-2.0) * np.abs(y)).astype(np.float32)
+        num = np.where(y > 0, np.float32(2.0), np.float32(2.0) * e)
+        return (np.float32(0.5) * v * (num * (np.float32(1.0) / (np.float32(1.0) + e)))).astype(np.float32)
+    raise ValueError(act)
+
+
+# ----------------------------------------------------------------------------------------------
+# Verification helpers (tests/test_common.py:353-423)
+# ----------------------------------------------------------------------------------------------
+
+
+def violating_fraction(out: np.ndarray, ref: np.ndarray, rtol: float, atol: float) -> float:
+    """Fraction of elements failing ``|out-ref| <= atol + rtol*|ref|`` (``checkAllclose``)."""
+    out = np.asarray(out, dtype=np.float32)
+    ref = np.asarray(ref, dtype=np.float32)
+    close = np.isclose(out, ref, rtol=rtol, atol=atol)
+    return float((~close).sum()) / max(1, out.size)
+
+
+def logits_diff(x: np.ndarray, y: np.ndarray) -> float:
+    """``1 - 2*sum(xy)/sum(x^2+y^2)`` in float64 (``verify_output``'s fallback metric)."""
+    x = np.asarray(x, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    den = (x * x + y * y).sum()
+    if den == 0:
+        return 0.0
+    d = 1.0 - 2.0 * (x * y).sum() / den
+    return 1.0 if np.isnan(d) else float(d)
+
+
+def verify_output(out, ref, atol=1e-2, rtol=1e-2, logits_diff_threshold=2e-3) -> bool:
+    """Reference acceptance rule: pass if fewer than 5 % of elements violate isclose, else pass if
+    the logits-diff metric is within the threshold (tests/test_common.py:397-423)."""
+    if violating_fraction(out, ref, rtol, atol) < 0.05:
+        return True
+    return logits_diff(out, ref) <= logits_diff_threshold
+
+
+def within_north_star_tolerance(out, ref, rel: float = 1e-2):
+    """The build's own (tighter) bar: ``|out-ref| <= rel*|ref| + rel*max|ref|`` everywhere.
+    Returns ``(ok, worst_ratio)`` where ``worst_ratio`` is max of ``|out-ref| / bound``."""
+    out = np.asarray(out, dtype=np.float32)
+    ref = np.asarray(ref, dtype=np.float32)
+    bound = rel * np.abs(ref) + rel * np.abs(ref).max(initial=0.0)
+    err = np.abs(out - ref)
+    if not np.all(np.isfinite(out)):
+        return False, float("inf")
+    ratio = float((err / np.maximum(bound, 1e-30)).max(initial=0.0))
+    return bool(np.all(err <= bound)), ratio
+
+
+# ----------------------------------------------------------------------------------------------
+# Workgroup-id remap (kernels/common/mma/mfma_preshuffle_pipeline.py:685-729)
+# ----------------------------------------------------------------------------------------------
+
+
+def xcd_remap_bx_by(bx: int, by: int, m: int, *, tile_m: int, tile_n: int, n: int, xcd_swizzle: int, num_xcds: int = 8):
+    """Remap ``(bx, by)`` so that workgroup ids dealt round-robin over XCDs form contiguous ranges
+    per XCD, grouped ``xcd_swizzle`` M-tiles per N sweep.  Pinned by bijectivity over whole grids."""
+    if xcd_swizzle <= 0:
+        return bx, by
+    gx = n // tile_n
+    gy = (m + tile_m - 1) // tile_m
+    linear = bx * gx + by
+    num = gx * gy
+    q, r = divmod(num, num_xcds)
+    xcd = linear % num_xcds
+    in_xcd = linear // num_xcds
+    wgid = xcd * q + min(xcd, r) + in_xcd
+    per_group = xcd_swizzle * gx
+    group = wgid // per_group
+    first_m = group * xcd_swizzle
+    size_m = min(gy - first_m, xcd_swizzle)
+    in_group = wgid % per_group
+    return first_m + in_group % size_m, in_group // size_m
