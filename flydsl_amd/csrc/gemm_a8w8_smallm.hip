@@ -105,10 +105,10 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     for (int mb = 0; mb < MB; mb++) red[wave][mb][lane] = acc[mb];
     __syncthreads();
 
-    // thread t < nbw*MB*64 finishes (n-block t/(MB*64), m-block, lane)
-    if (tid < nbw * MB * 64) {
-        const int nbi = tid / (MB * 64);
-        const int mb = (tid / 64) % MB;
+    // work item t < nbw*MB*64 finishes (n-block t/(MB*64), m-block, lane); up to 1024 items for 512 threads
+    for (int t = tid; t < nbw * MB * 64; t += NW * 64) {
+        const int nbi = t / (MB * 64);
+        const int mb = (t / 64) % MB;
         const int nb = (int)blockIdx.x * nbw + nbi;
         acc_t sum = red[nbi * ks][mb][lane];
         for (int j = 1; j < ks; j++) sum += red[nbi * ks + j][mb][lane];

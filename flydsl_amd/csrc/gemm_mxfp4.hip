@@ -277,10 +277,10 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
     }
     __syncthreads();
 
-    // thread t < npw*MB*2*64 finishes (n-pair, m-block, n-block of the pair, lane)
-    if (tid < npw * MB * 2 * 64) {
-        const int npi = tid / (MB * 2 * 64);
-        const int f = (tid / 64) % (MB * 2);
+    // work item t < npw*MB*2*64 finishes (n-pair, m-block, n-block of the pair, lane)
+    for (int t = tid; t < npw * MB * 2 * 64; t += NW * 64) {
+        const int npi = t / (MB * 2 * 64);
+        const int f = (t / 64) % (MB * 2);
         const int mb = f >> 1, nb = f & 1;
         const int np = (int)blockIdx.x * npw + npi;
         v4f sum = red[npi * ks][f][lane];

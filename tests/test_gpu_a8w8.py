@@ -21,7 +21,7 @@ def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, 
     from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
     dev = torch.device("cuda")
-    fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=128, in_dtype=d["kind"], out_dtype=out_dtype,
+    fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=64, in_dtype=d["kind"], out_dtype=out_dtype,
                                  epilogue=epilogue)
     tdt = torch.bfloat16 if out_dtype == "bf16" else torch.float16
     c_alloc = torch.full((M + guard_rows, N), SENTINEL, dtype=tdt, device=dev)
@@ -44,7 +44,7 @@ def _acc(d, M, N, K, *, force_path=0, tile=None):
     from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
     dev = torch.device("cuda")
-    fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=128, in_dtype=d["kind"])
+    fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=64, in_dtype=d["kind"])
     dt = torch.int32 if d["kind"] == "int8" else torch.float32
     acc = torch.full((M, N), -7, dtype=dt, device=dev)
     fn.accumulators(acc, d["a_q"].to(dev), d["b_shuf"].to(dev), M, N, torch.cuda.current_stream(), force_path=force_path,
@@ -88,6 +88,14 @@ def test_small_m_paths(kind, M):
             assert np.array_equal(got, O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"])))
             cref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")
             assert np.array_equal(bf16_bits(c[:M]), cref["c_bf16_bits"])
+
+
+def test_small_m_no_ksplit():
+    # N/16 >= 2048 n-blocks: the dispatcher keeps K whole (ksplit 1), 8 n-blocks per workgroup
+    M, N, K = 32, 32768, 256
+    d = make_a8w8(M, N, K, "int8", seed=1)
+    got = _acc(d, M, N, K, force_path=2)
+    assert np.array_equal(got, O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"])))
 
 
 # ---- config 2: fp8 decode, N=6144 K=4096 -------------------------------------------------------
