@@ -1,0 +1,288 @@
+#!/usr/bin/env python3
+"""Benchmark of the preshuffle quantized GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]
+
+A step is one GEMM launch on one set of synthetic operands (seed 0; activations N(0,1), weights
+N(0,0.02), quantised and preshuffled on the host, resident in HBM before the timed region).
+Steps rotate through enough independent operand sets that the weights cannot be served from the
+256 MB Infinity Cache.  The K timed steps are recorded once into a HIP graph and replayed, bracketed by
+``torch.cuda.synchronize()`` on both sides (wall clock -> ``value`` / ``ms_per_step``) and by HIP events
+on the launch stream (-> ``roofline.achieved``).  Prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# name -> (family, dtype label, M, N, K, roofline bound)
+WORKLOADS = {
+    "fp8_decode_m1": ("a8w8", "fp8", 1, 6144, 4096, "hbm"),
+    "fp8_decode_m16": ("a8w8", "fp8", 16, 6144, 4096, "hbm"),
+    "fp8_decode_m32": ("a8w8", "fp8", 32, 6144, 4096, "hbm"),
+    "fp8_prefill_m8192": ("a8w8", "fp8", 8192, 4096, 4096, "mfma"),
+    "int8_ffn_m4096": ("a8w8", "int8", 4096, 28672, 8192, "mfma"),
+    "mxfp4_m32": ("mxfp4", "fp4", 32, 7168, 2048, "hbm"),
+    "mxfp4_m4096": ("mxfp4", "fp4", 4096, 7168, 2048, "mfma"),
+    "int8_plumbing_m128": ("a8w8", "int8", 128, 1024, 1024, "mfma"),
+}
+DEFAULT_WORKLOAD = "fp8_decode_m16"
+PEAK = {"hbm": 8000.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0}  # GB/s, TFLOP/s (dense, published)
+MALL_BYTES = 256 << 20
+
+
+def algorithmic_bytes(family, M, N, K):
+    if family == "a8w8":
+        return M * K + N * K + 2 * M * N + 4 * (M + N)
+    return M * K // 2 + N * K // 2 + 2 * M * N + (M + N) * (K // 32)
+
+
+def make_launcher(family, kind, M, N, K):
+    import torch
+
+    if family == "a8w8":
+        from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
+
+        fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=64, in_dtype=kind)
+        bias = torch.empty(0, dtype=torch.bfloat16, device="cuda")
+
+        def launch(s):
+            fn(s["c"], s["a"], s["b"], s["sa"], s["sb"], bias, M, N, torch.cuda.current_stream())
+    else:
+        from kernels.gemm.mxfp4_preshuffle import launch_gemm
+
+        def launch(s):
+            launch_gemm(s["c"], s["a"], s["b"], s["sa"], s["sb"], M, N, torch.cuda.current_stream(), N, K, 64, 256, 256,
+                        "fp4", "bf16", "fp4", 1, -1, -1, -1, -1, -1, -1, 0, 0)
+    return launch
+
+
+def run_workload(name, steps, warmup, check=True):
+    import numpy as np
+    import torch
+
+    family, kind, M, N, K, bound = WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    nbytes = algorithmic_bytes(family, M, N, K)
+    flops = 2.0 * M * N * K
+    # enough operand sets that one pass over them exceeds twice the Infinity Cache
+    n_sets = max(2, min(32, math.ceil(2 * MALL_BYTES / nbytes)))
+    if nbytes * n_sets > (8 << 30):
+        n_sets = max(2, (8 << 30) // nbytes)
+    from flydsl_amd.synthetic import make_a8w8, make_mxfp4
+
+    host = make_a8w8(M, N, K, kind, seed=0) if family == "a8w8" else make_mxfp4(M, N, K, seed=0)
+    sets = []
+    for i in range(n_sets):
+        if family == "a8w8":
+            s = {"a": host["a_q"].to(dev), "b": host["b_shuf"].to(dev), "sa": host["sa"].to(dev), "sb": host["sb"].to(dev)}
+        else:
+            s = {"a": host["a_q"].to(dev), "b": host["b_shuf"].to(dev), "sa": host["sa_shuf"].to(dev), "sb": host["sb_shuf"].to(dev)}
+        s["c"] = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+        sets.append(s)
+    launch = make_launcher(family, kind, M, N, K)
+
+    for i in range(warmup):
+        launch(sets[i % n_sets])
+    torch.cuda.synchronize()
+
+    # record the K timed steps into one graph on a side stream
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for i in range(steps):
+            launch(sets[i % n_sets])
+    torch.cuda.synchronize()
+    graph.replay()  # untimed: first replay uploads the graph
+    torch.cuda.synchronize()
+
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_wall, best_ev = float("inf"), float("inf")
+    for _ in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record()
+        graph.replay()
+        ev1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        best_wall = min(best_wall, wall)
+        best_ev = min(best_ev, ev0.elapsed_time(ev1) * 1e-3)
+    sec_per_step = best_wall / steps
+    kernel_s = best_ev / steps
+
+    # hot-cache figure (one operand set): informative only
+    ghot = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(ghot, stream=side):
+        for i in range(steps):
+            launch(sets[0])
+    torch.cuda.synchronize()
+    ghot.replay()
+    torch.cuda.synchronize()
+    ev0.record()
+    ghot.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    hot_s = ev0.elapsed_time(ev1) * 1e-3 / steps
+
+    ok = None
+    if check:
+        from oracle import psg_oracle as O
+
+        out = sets[(steps - 1) % n_sets]["c"].float().cpu().numpy()
+        rows = np.arange(M) if M <= 256 else np.array(sorted({(i * 131 + 7) % M for i in range(64)}))
+        if family == "a8w8":
+            ref = O.run_torch(host["a_q"].view(torch.uint8).numpy()[rows], host["b_q"].view(torch.uint8).numpy(),
+                              host["sa"].numpy()[rows], host["sb"].numpy(), kind)
+        else:
+            ref = O.run_torch_w4(host["a_q"].numpy()[rows], host["b_q"].numpy(), host["sa"].numpy()[:M][rows], host["sb"].numpy())
+        bound_abs = 1e-2 * np.abs(ref) + 1e-2 * np.abs(ref).max()
+        ok = bool(np.all(np.abs(out[rows] - ref) <= bound_abs))
+
+    if bound == "hbm":
+        achieved, peak, unit = nbytes / kernel_s / 1e9, PEAK["hbm"], "GB/s"
+    else:
+        achieved, peak, unit = flops / kernel_s / 1e12, PEAK[kind], "TFLOP/s"
+    res = {
+        "workload": name, "dtype": kind, "M": M, "N": N, "K": K,
+        "tflops": flops / sec_per_step / 1e12, "gb_per_s": nbytes / sec_per_step / 1e9,
+        "us_per_step_wall": sec_per_step * 1e6, "us_per_launch_events": kernel_s * 1e6, "us_per_launch_hot_cache": hot_s * 1e6,
+        "operand_sets": n_sets, "parity_ok": ok,
+        "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+                     "traffic": None, "algorithmic_bytes": nbytes, "flops": flops},
+    }
+    del graph, ghot, sets
+    torch.cuda.empty_cache()
+    return res, host
+
+
+def cpu_baseline(name, host, budget_s=12.0):
+    """The reference's torch CPU path (dequantise to fp32 + torch.mm) on the same seeded operands,
+    timed on this box's host cores.  For workloads whose single pass exceeds the budget a row sample of
+    A is used (the weight side, which dominates the dequantisation cost, is always whole)."""
+    import torch
+
+    from oracle import psg_oracle as O
+
+    family, kind, M, N, K, _ = WORKLOADS[name]
+    cores = torch.get_num_threads()
+    # bound the work: ~2*m*N*K flop at a conservative 50 GFLOP/s per 8 cores
+    est = 2.0 * M * N * K / (6e9 * cores) + N * K / 2e8
+    m_s = M if est <= budget_s else max(16, int(M * budget_s / est))
+    if family == "a8w8":
+        a, b, sa, sb = host["a_q"][:m_s], host["b_q"], host["sa"][:m_s], host["sb"]
+        f = lambda: O.run_torch_cpu(a, b, sa, sb)  # noqa: E731
+    else:
+        a, b, sa, sb = host["a_q"][:m_s], host["b_q"], host["sa"], host["sb"]
+        f = lambda: O.run_torch_w4_cpu(a, b, sa, sb)  # noqa: E731
+    t0 = time.perf_counter()
+    f()
+    first = time.perf_counter() - t0
+    iters = max(1, min(10, int(budget_s / 2 / max(first, 1e-6))))
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        f()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": 2.0 * m_s * N * K / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"run_torch (fp32 dequant + torch.mm) on rows [0,{m_s}) of A x all {N} weight rows, K={K}; "
+                  f"median of {iters} runs, {med * 1e3:.1f} ms each",
+    }
+
+
+def load_traffic(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy
+    kernel of known size); kept as a small committed summary next to the profiles."""
+    path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name, {}).get("traffic_bytes")
+    except Exception:
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
+              "the GEMM shards over N with no exchange, see DESIGN.md", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the preshuffle GEMM has no CPU path", file=sys.stderr)
+        sys.exit(3)
+    from flydsl_amd import _lib
+
+    _lib.lib()  # fail loudly if the HIP library is missing
+
+    family, kind, M, N, K, bound = WORKLOADS[args.workload]
+    small = bound == "hbm"
+    steps = args.steps if args.steps is not None else (500 if small else 20)
+    warmup = args.warmup if args.warmup is not None else (50 if small else 3)
+
+    main_res, host = run_workload(args.workload, steps, warmup)
+    main_res["roofline"]["traffic"] = load_traffic(args.workload)
+    cpu = None if args.no_cpu else cpu_baseline(args.workload, host)
+    del host
+
+    others = []
+    if not args.no_others:
+        for name in ("fp8_decode_m1", "fp8_decode_m16", "fp8_decode_m32", "fp8_prefill_m8192", "int8_ffn_m4096", "mxfp4_m32",
+                     "mxfp4_m4096"):
+            if name == args.workload:
+                continue
+            b = WORKLOADS[name][5]
+            r, _ = run_workload(name, 300 if b == "hbm" else (5 if name == "int8_ffn_m4096" else 20), 20 if b == "hbm" else 2)
+            r["roofline"]["traffic"] = load_traffic(name)
+            others.append(r)
+
+    line = {
+        "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",
+        "value": main_res["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": main_res["us_per_step_wall"] / 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"fp8": "fp8_e4m3fn", "int8": "int8", "fp4": "mxfp4_e2m1"}[kind],
+        "data": "synthetic (seed 0; A~N(0,1) per-token quantised, W~N(0,0.02) per-channel quantised and preshuffled; "
+                f"{main_res['operand_sets']} rotating operand sets)",
+        "config": {"workload": f"{args.workload}: {kind} W8A8 preshuffle GEMM M={M} N={N} K={K}, bf16 out", "M": M, "N": N, "K": K,
+                   "timing": "K steps recorded into one HIP graph, replayed; wall clock between synchronizes"},
+        "gb_per_s": main_res["gb_per_s"],
+        "parity_ok": main_res["parity_ok"],
+        "us_per_launch_events": main_res["us_per_launch_events"],
+        "us_per_launch_hot_cache": main_res["us_per_launch_hot_cache"],
+        "roofline": main_res["roofline"],
+        "cpu_baseline": cpu,
+        "per_config": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

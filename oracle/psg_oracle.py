@@ -467,3 +467,41 @@ def xcd_remap_bx_by(bx: int, by: int, m: int, *, tile_m: int, tile_n: int, n: in
     size_m = min(gy - first_m, xcd_swizzle)
     in_group = wgid % per_group
     return first_m + in_group % size_m, in_group // size_m
+
+
+# ----------------------------------------------------------------------------------------------
+# The reference's CPU path, literally (torch ops), for the cpu_baseline timing
+# ----------------------------------------------------------------------------------------------
+
+
+def run_torch_cpu(a_q, b_q, scale_a, scale_b):
+    """``run_torch`` with torch CPU tensors exactly as the reference runs it on a CPU-only box
+    (tests/kernels/test_preshuffle_gemm.py:103-113): ``a.to(f32) * sa[:, None]``,
+    ``b.to(f32) * sb[:, None]``, ``torch.mm(a32, b32.T)``.  ``a_q`` / ``b_q`` are torch int8 or
+    float8_e4m3fn CPU tensors (``b_q`` un-shuffled)."""
+    import torch
+
+    a32 = a_q.to(torch.float32) * scale_a.view(-1, 1)
+    b32 = b_q.to(torch.float32) * scale_b.view(-1, 1)
+    return torch.mm(a32, b32.T)
+
+
+def run_torch_w4_cpu(a_packed, b_packed, scale_a, scale_b):
+    """``run_torch_w4`` with torch CPU tensors (tests/kernels/test_preshuffle_gemm.py:404-411)."""
+    import torch
+
+    lut = torch.from_numpy(E2M1_LUT.copy())
+
+    def dec(p):
+        b = p.view(torch.uint8)
+        codes = torch.stack([b & 0xF, b >> 4], dim=-1).reshape(b.shape[0], -1)
+        return lut[codes.long()]
+
+    def sc(s, rows):
+        b = s.view(torch.uint8)[:rows].to(torch.int32)
+        bits = torch.where(b == 0, torch.full_like(b, 0x00400000), b << 23)
+        return bits.view(torch.float32).repeat_interleave(32, dim=1)
+
+    x = dec(a_packed) * sc(scale_a, a_packed.shape[0])
+    w = dec(b_packed) * sc(scale_b, b_packed.shape[0])
+    return torch.mm(x, w.T)

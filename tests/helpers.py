@@ -1,73 +1,15 @@
-"""Shared input builders for the parity tests: seeded synthetic operands in the distributions the
-benchmark configs name (activations N(0,1), weights N(0,0.02)), quantised and laid out by the
-package's host helpers, with numpy views for the oracle."""
+"""Shared helpers of the parity tests."""
 
 from __future__ import annotations
 
 import numpy as np
 import torch
 
-from flydsl_amd import layout, quant
-
-FP8 = torch.float8_e4m3fn
-
-
-def gen(seed):
-    g = torch.Generator(device="cpu")
-    g.manual_seed(seed)
-    return g
-
-
-def make_a8w8(M, N, K, kind, seed=0, w_std=0.02):
-    """Returns dict with CPU tensors a_q [M,K], b_q [N,K] (un-shuffled), b_shuf, sa [M], sb [N]."""
-    g = gen(seed)
-    x = torch.randn(M, K, generator=g, dtype=torch.float32)
-    w = torch.randn(N, K, generator=g, dtype=torch.float32) * w_std
-    qd = torch.int8 if kind == "int8" else FP8
-    a_q, sa = quant.pertoken_quant(x, quant_dtype=qd)
-    b_q, sb = quant.pertoken_quant(w, quant_dtype=qd)
-    b_shuf = layout.shuffle_weight(b_q.contiguous(), layout=(16, 16))
-    return {
-        "kind": kind,
-        "a_q": a_q.contiguous(),
-        "b_q": b_q.contiguous(),
-        "b_shuf": b_shuf.contiguous(),
-        "sa": sa.reshape(-1).contiguous(),
-        "sb": sb.reshape(-1).contiguous(),
-    }
+from flydsl_amd.synthetic import make_a8w8, make_mxfp4  # noqa: F401
 
 
 def np_bytes(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.uint8).numpy()
-
-
-def make_mxfp4(M, N, K, seed=0, w_std=0.02):
-    """MXFP4 operands the way the reference's harness builds them
-    (tests/kernels/test_preshuffle_gemm.py:386-414): rows padded to 32 before quantisation."""
-    g = gen(seed)
-    x = torch.randn(M, K, generator=g, dtype=torch.float32)
-    w = torch.randn(N, K, generator=g, dtype=torch.float32) * w_std
-    m32 = (M + 31) // 32 * 32
-    n32 = (N + 31) // 32 * 32
-    xp = torch.zeros(m32, K)
-    xp[:M] = x
-    wp = torch.zeros(n32, K)
-    wp[:N] = w
-    a_q, sa, _ = quant.per_1x32_f4_quant(xp)
-    b_q, sb, _ = quant.per_1x32_f4_quant(wp)
-    a_q = a_q.view(torch.uint8)[:M].contiguous()
-    b_q = b_q.view(torch.uint8)[:N].contiguous()
-    sa = sa.view(torch.uint8).contiguous()
-    sb = sb.view(torch.uint8).contiguous()
-    return {
-        "a_q": a_q,
-        "b_q": b_q,
-        "sa": sa,
-        "sb": sb,
-        "b_shuf": layout.shuffle_weight_w4(b_q, 16, False, False).contiguous(),
-        "sa_shuf": layout.shuffle_scale_w4(sa, 1, False).contiguous(),
-        "sb_shuf": layout.shuffle_scale_w4(sb, 1, False).contiguous(),
-    }
 
 
 def bf16_bits(t: torch.Tensor) -> np.ndarray:
