@@ -121,9 +121,8 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
             } else {
                 const float sa = p.sa[m];
                 const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
-                float x[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) x[e] = ((float)sum[e] * sa) * sb[e];
+                const v4f x = {((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
+                               ((float)sum[3] * sa) * sb[3]};
                 store_c4(p, idx, n, x);
             }
         }

@@ -47,6 +47,8 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
     tn = in_g / size_m;
 }
 
+// STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
+// free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
 template <int KIND, int MR, int NR, int STORE>
 __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
@@ -94,16 +96,17 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
     v4i areg[A_LOADS];
     v4i blo[2][NR], bhi[2][NR];
 
+    // Loads never sit under control flow: a K step past the end (prefetch of the last iteration) and an A
+    // chunk past K (only when K % 128 == 64) are redirected past the descriptor bound, where the hardware
+    // returns zero without touching memory.  Selecting on the ADDRESS keeps the loaded registers untouched
+    // until they are used, so no wait is forced early.
     auto load_a = [&](int kt) {
         const uint32_t k0 = (uint32_t)kt * TK;
-        // a 16-byte chunk is either fully inside K or fully outside (K % 64 == 0)
         const bool in_k = (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
-            // the whole byte offset sits in the bounds-checked VGPR offset: rows >= M (and the tail of the
-            // last row when K % 128 == 64) come back as zero instead of touching memory past A
-            v4i v = buf_load16(ra, a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0, 0);
-            areg[j] = in_k ? v : (v4i){0, 0, 0, 0};
+            const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0;
+            areg[j] = buf_load16(ra, in_k ? off : 0xFFFFFFF0u, 0);
         }
     };
     auto store_a = [&](int stage) {
@@ -114,24 +117,34 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
         }
     };
     auto load_b = [&](int kt, v4i* lo, v4i* hi) {
+        const bool has_lo = (kt * TK) < K;
         const bool has_hi = (kt * TK + 64) < K;
+        const uint32_t koff = has_lo ? (uint32_t)kt * 2048u : 0u;
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
             // n-block select in the bounds-checked VGPR offset (blocks >= N/16 read as zero), K position in
-            // the scalar offset; a missing upper half re-reads the lower one instead of running past W
+            // the scalar offset
             const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
-            const uint32_t koff = (uint32_t)kt * 2048u;
-            lo[ni] = buf_load16(rb, voff, koff);
-            v4i h = buf_load16(rb, voff, has_hi ? koff + 1024u : koff);
-            hi[ni] = has_hi ? h : (v4i){0, 0, 0, 0};
+            lo[ni] = buf_load16(rb, has_lo ? voff : 0xFFFFFFF0u, koff);
+            hi[ni] = buf_load16(rb, has_hi ? voff : 0xFFFFFFF0u, has_hi ? koff + 1024u : 0u);
         }
     };
+    // A fragments are read one m-block ahead of the MFMAs that use them (register double buffer), so the
+    // LDS latency of block mi+1 hides behind the MFMAs of block mi.
+    auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {
+        const int row = mi * 16 + li;
+        flo = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
+        fhi = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
+    };
     auto compute = [&](int stage, const v4i* lo, const v4i* hi) {
+        v4i flo[2], fhi[2];
+        read_frag(stage, 0, flo[0], fhi[0]);
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) {
-            const int row = mi * 16 + li;
-            const v4i alo = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
-            const v4i ahi = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
+            if (mi + 1 < MR) read_frag(stage, mi + 1, flo[(mi + 1) & 1], fhi[(mi + 1) & 1]);
+            // keep the prefetch ahead of this block's MFMAs (the machine scheduler would otherwise sink it)
+            __builtin_amdgcn_sched_barrier(0);
+            const v4i alo = flo[mi & 1], ahi = fhi[mi & 1];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
@@ -146,6 +159,7 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
                     acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[mi][ni], 0, 0, 0, 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -155,52 +169,53 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
     store_a(0);
     __syncthreads();
 
+    // Two K steps per iteration (LDS / register ping-pong).  When the step count is odd the last "odd" step
+    // multiplies zero operands (its loads were redirected past the bounds): harmless, and the loop body stays
+    // free of control flow, which the software pipeline needs.
     for (int kt = 0; kt < KT; kt += 2) {
-        {  // even step: compute stage 0, prefetch stage 1
-            const bool next = (kt + 1) < KT;
-            if (next) {
-                load_a(kt + 1);
-                load_b(kt + 1, blo[1], bhi[1]);
-            }
-            compute(0, blo[0], bhi[0]);
-            if (next) store_a(1);
-            __syncthreads();
-        }
-        if (kt + 1 < KT) {  // odd step: compute stage 1, prefetch stage 0
-            const bool next = (kt + 2) < KT;
-            if (next) {
-                load_a(kt + 2);
-                load_b(kt + 2, blo[0], bhi[0]);
-            }
-            compute(1, blo[1], bhi[1]);
-            if (next) store_a(0);
-            __syncthreads();
-        }
+        load_a(kt + 1);
+        load_b(kt + 1, blo[1], bhi[1]);
+        compute(0, blo[0], bhi[0]);
+        store_a(1);
+        __syncthreads();
+
+        load_a(kt + 2);
+        load_b(kt + 2, blo[0], bhi[0]);
+        compute(1, blo[1], bhi[1]);
+        store_a(0);
+        __syncthreads();
     }
 
-    // epilogue: lane owns C[m0 + mi*16 + li][n0 + (wave*NR + ni)*16 + lg*4 + 0..3]
-#pragma unroll
-    for (int mi = 0; mi < MR; mi++) {
+    // epilogue: lane owns C[m0 + mi*16 + li][n0 + (wave*NR + ni)*16 + lg*4 + 0..3].  Compile-time indices only,
+    // so the accumulators are never addressed dynamically.
+    static_for<MR>([&](auto MI) {
+        constexpr int mi = decltype(MI)::value;
         const int m = m0 + mi * 16 + li;
-        if (m >= p.M) continue;
-        float sa = 0.f;
-        if constexpr (STORE == STORE_C) sa = p.sa[m];
-#pragma unroll
-        for (int ni = 0; ni < NR; ni++) {
-            const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-            if (n >= p.N) continue;
-            const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
-            if constexpr (STORE == STORE_ACC) {
-                *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = acc[mi][ni];
-            } else {
-                const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
-                float x[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) x[e] = ((float)acc[mi][ni][e] * sa) * sb[e];
-                store_c4(p, idx, n, x);
-            }
+        if (m < p.M) {
+            float sa = 0.f;
+            if constexpr (STORE != STORE_ACC) sa = p.sa[m];
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                if (n < p.N) {
+                    const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
+                    const acc_t r = acc[mi][ni];
+                    if constexpr (STORE == STORE_ACC) {
+                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = r;
+                    } else {
+                        const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
+                        const v4f x = {((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2],
+                                       ((float)r[3] * sa) * sb[3]};
+                        if constexpr (STORE == STORE_C) {
+                            *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(p.c) + idx) = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
+                        } else {
+                            store_c4(p, idx, n, x);
+                        }
+                    }
+                }
+            });
         }
-    }
+    });
 }
 
 template <int KIND, int MR, int NR, int STORE>
@@ -230,12 +245,15 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
 // Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8.  tile_m x tile_n must be one of the
 // instantiated shapes: 256x256, 128x256, 64x256, 32x256, 128x128, 64x64.
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
+    if (store == STORE_C && (p.epi != EPI_NONE || p.out != OUT_BF16)) store = STORE_C_GENERIC;
     if (kind == KIND_INT8) {
         if (store == STORE_ACC) return launch_shape<KIND_INT8, STORE_ACC>(p, tile_m, tile_n, stream);
+        if (store == STORE_C_GENERIC) return launch_shape<KIND_INT8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
         return launch_shape<KIND_INT8, STORE_C>(p, tile_m, tile_n, stream);
     }
     if (kind == KIND_FP8) {
         if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);
+        if (store == STORE_C_GENERIC) return launch_shape<KIND_FP8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
         return launch_shape<KIND_FP8, STORE_C>(p, tile_m, tile_n, stream);
     }
     return hipErrorInvalidValue;

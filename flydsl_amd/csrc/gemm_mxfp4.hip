@@ -107,85 +107,94 @@ __global__ void __launch_bounds__(256) k_mxfp4_tiled(MxParams p) {
     v4i bq[2][NR][2];
     int sav[2][MP], sbv[2][NP];
 
+    // Loads never sit under control flow: a K step past the end (prefetch of the last iteration) is
+    // redirected past the descriptor bounds, where the hardware returns zero without touching memory.
     auto load_a = [&](int kt) {
+        const bool valid = kt < KT;
 #pragma unroll
-        for (int j = 0; j < A_LOADS; j++)
-            areg[j] = buf_load16(ra, a_goff0 + (uint32_t)j * 32u * (uint32_t)KP + (uint32_t)kt * TKB, 0);
+        for (int j = 0; j < A_LOADS; j++) {
+            const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)KP + (uint32_t)kt * TKB;
+            areg[j] = buf_load16(ra, valid ? off : 0xFFFFFFF0u, 0);
+        }
     };
     auto store_a = [&](int stage) {
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++)
             *reinterpret_cast<v4i*>(&lds[stage][lds_off(a_row0 + 32 * j, a_kc)]) = areg[j];
     };
-    auto load_b = [&](int kt, int st) {
+    auto load_b = [&](int kt, auto ST) {
+        constexpr int st = decltype(ST)::value;
+        const bool valid = kt < KT;
+        const uint32_t koff = valid ? (uint32_t)kt * 2048u : 0u;
+        const uint32_t soff = valid ? (uint32_t)kt * 256u : 0u;
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
-            const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)KP;
-            bq[st][ni][0] = buf_load16(rb, voff, (uint32_t)kt * 2048u);
-            bq[st][ni][1] = buf_load16(rb, voff, (uint32_t)kt * 2048u + 1024u);
+            const uint32_t voff = valid ? (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)KP : 0xFFFFFFF0u;
+            bq[st][ni][0] = buf_load16(rb, voff, koff);
+            bq[st][ni][1] = buf_load16(rb, voff, valid ? koff + 1024u : 0u);
         }
 #pragma unroll
         for (int mp = 0; mp < MP; mp++)
-            sav[st][mp] = buf_load4(rsa, (uint32_t)mp * (uint32_t)chunk_bytes + (uint32_t)lane * 4u, (uint32_t)kt * 256u);
+            sav[st][mp] = buf_load4(rsa, valid ? (uint32_t)mp * (uint32_t)chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
 #pragma unroll
         for (int np = 0; np < NP; np++)
-            sbv[st][np] = buf_load4(rsb, (uint32_t)np * (uint32_t)chunk_bytes + (uint32_t)lane * 4u, (uint32_t)kt * 256u);
+            sbv[st][np] = buf_load4(rsb, valid ? (uint32_t)np * (uint32_t)chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
     };
+    // A fragments (m-block, 128-K half) are read one step ahead of the MFMAs that use them
     auto compute = [&](auto ST) {
         constexpr int st = decltype(ST)::value;
-        static_for<MR>([&](auto MI) {
-            constexpr int mi = decltype(MI)::value;
-            static_for<2>([&](auto KH) {
-                constexpr int kh = decltype(KH)::value;
-                const v4i af = *reinterpret_cast<const v4i*>(&lds[st][lds_off(mi * 16 + li, kh * 4 + lg)]);
-                static_for<NR>([&](auto NI) {
-                    constexpr int ni = decltype(NI)::value;
-                    acc[mi][ni] = mx_mfma<kh * 2 + (ni & 1), kh * 2 + (mi & 1)>(bq[st][ni][kh], af, acc[mi][ni],
-                                                                                   sbv[st][ni / 2], sav[st][mi / 2]);
-                });
+        v4i af[2];
+        af[0] = *reinterpret_cast<const v4i*>(&lds[st][lds_off(li, lg)]);
+        static_for<MR * 2>([&](auto IDX) {
+            constexpr int idx = decltype(IDX)::value;
+            constexpr int mi = idx / 2, kh = idx % 2;
+            if constexpr (idx + 1 < MR * 2) {
+                constexpr int mi1 = (idx + 1) / 2, kh1 = (idx + 1) % 2;
+                af[(idx + 1) & 1] = *reinterpret_cast<const v4i*>(&lds[st][lds_off(mi1 * 16 + li, kh1 * 4 + lg)]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                acc[mi][ni] = mx_mfma<kh * 2 + (ni & 1), kh * 2 + (mi & 1)>(bq[st][ni][kh], af[idx & 1], acc[mi][ni],
+                                                                               sbv[st][ni / 2], sav[st][mi / 2]);
             });
+            __builtin_amdgcn_sched_barrier(0);
         });
     };
 
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
     load_a(0);
-    load_b(0, 0);
+    load_b(0, S0{});
     store_a(0);
     __syncthreads();
 
+    // two K steps per iteration (ping-pong); an odd step count ends with one step on zero operands
     for (int kt = 0; kt < KT; kt += 2) {
-        {
-            const bool next = (kt + 1) < KT;
-            if (next) {
-                load_a(kt + 1);
-                load_b(kt + 1, 1);
-            }
-            compute(std::integral_constant<int, 0>{});
-            if (next) store_a(1);
-            __syncthreads();
-        }
-        if (kt + 1 < KT) {
-            const bool next = (kt + 2) < KT;
-            if (next) {
-                load_a(kt + 2);
-                load_b(kt + 2, 0);
-            }
-            compute(std::integral_constant<int, 1>{});
-            if (next) store_a(0);
-            __syncthreads();
-        }
+        load_a(kt + 1);
+        load_b(kt + 1, S1{});
+        compute(S0{});
+        store_a(1);
+        __syncthreads();
+
+        load_a(kt + 2);
+        load_b(kt + 2, S0{});
+        compute(S1{});
+        store_a(0);
+        __syncthreads();
     }
 
-#pragma unroll
-    for (int mi = 0; mi < MR; mi++) {
+    static_for<MR>([&](auto MI) {
+        constexpr int mi = decltype(MI)::value;
         const int m = m0 + mi * 16 + li;
-        if (m >= p.M) continue;
-#pragma unroll
-        for (int ni = 0; ni < NR; ni++) {
-            const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-            if (n >= p.N) continue;
-            store_mx4(p, STORE, (size_t)m * (size_t)p.N + (size_t)n, acc[mi][ni]);
+        if (m < p.M) {
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                if (n < p.N) store_mx4(p, STORE, (size_t)m * (size_t)p.N + (size_t)n, acc[mi][ni]);
+            });
         }
-    }
+    });
 }
 
 // ------------------------------------------------------------------------------------------------

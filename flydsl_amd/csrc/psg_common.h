@@ -16,7 +16,7 @@ enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3 };
 enum { OUT_BF16 = 0, OUT_FP16 = 1 };
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_RELU = 2, EPI_BIAS_SILU = 3, EPI_BIAS_GELU = 4 };
 // what a kernel writes: the scaled/activated C, or the raw accumulators
-enum { STORE_C = 0, STORE_ACC = 1 };
+enum { STORE_C = 0, STORE_ACC = 1, STORE_C_GENERIC = 2 };
 
 // Raw buffer resource over [base, base+bytes): loads past the end return 0, stores past it are dropped.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint64_t bytes) {
@@ -122,35 +122,35 @@ struct MxParams {
     int out;  // OUT_*
 };
 
-// bias + activation + 16-bit conversion of four consecutive columns, chosen at run time (the epilogue is
-// a vanishing part of any launch, so it is not worth a kernel instantiation per variant)
-template <int OUT>
-__device__ __forceinline__ v2i finish4(const float* x, const uint16_t* bias_n, int epi) {
-    float b[4] = {0.f, 0.f, 0.f, 0.f};
-    if (epi != EPI_NONE) {
+// bias + activation + 16-bit conversion of four consecutive columns.  The variant is chosen at run time
+// (the epilogue is a vanishing part of any launch, so it is not worth a kernel instantiation per variant).
+template <int OUT, int EPI>
+__device__ __forceinline__ v2i finish4(v4f x, const uint16_t* bias_n) {
+    float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+    if constexpr (EPI != EPI_NONE) {
         const v2i braw = *reinterpret_cast<const v2i*>(bias_n);
-        b[0] = from_out16<OUT>((uint16_t)(braw[0] & 0xFFFF));
-        b[1] = from_out16<OUT>((uint16_t)((uint32_t)braw[0] >> 16));
-        b[2] = from_out16<OUT>((uint16_t)(braw[1] & 0xFFFF));
-        b[3] = from_out16<OUT>((uint16_t)((uint32_t)braw[1] >> 16));
+        b0 = from_out16<OUT>((uint16_t)(braw[0] & 0xFFFF));
+        b1 = from_out16<OUT>((uint16_t)((uint32_t)braw[0] >> 16));
+        b2 = from_out16<OUT>((uint16_t)(braw[1] & 0xFFFF));
+        b3 = from_out16<OUT>((uint16_t)((uint32_t)braw[1] >> 16));
     }
-    float v[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        switch (epi) {
-            case EPI_BIAS: v[e] = epi_act<EPI_BIAS>(x[e], b[e]); break;
-            case EPI_BIAS_RELU: v[e] = epi_act<EPI_BIAS_RELU>(x[e], b[e]); break;
-            case EPI_BIAS_SILU: v[e] = epi_act<EPI_BIAS_SILU>(x[e], b[e]); break;
-            case EPI_BIAS_GELU: v[e] = epi_act<EPI_BIAS_GELU>(x[e], b[e]); break;
-            default: v[e] = x[e]; break;
-        }
+    return pack4_out16<OUT>(epi_act<EPI>(x[0], b0), epi_act<EPI>(x[1], b1), epi_act<EPI>(x[2], b2), epi_act<EPI>(x[3], b3));
+}
+
+template <int OUT>
+__device__ __forceinline__ v2i finish4_rt(v4f x, const uint16_t* bias_n, int epi) {
+    switch (epi) {
+        case EPI_BIAS: return finish4<OUT, EPI_BIAS>(x, bias_n);
+        case EPI_BIAS_RELU: return finish4<OUT, EPI_BIAS_RELU>(x, bias_n);
+        case EPI_BIAS_SILU: return finish4<OUT, EPI_BIAS_SILU>(x, bias_n);
+        case EPI_BIAS_GELU: return finish4<OUT, EPI_BIAS_GELU>(x, bias_n);
+        default: return finish4<OUT, EPI_NONE>(x, bias_n);
     }
-    return pack4_out16<OUT>(v[0], v[1], v[2], v[3]);
 }
 
 // store four consecutive columns of row-major 16-bit C starting at element index idx (column n)
 template <class P>
-__device__ __forceinline__ void store_c4(const P& p, size_t idx, int n, const float* x) {
-    v2i r = p.out == OUT_BF16 ? finish4<OUT_BF16>(x, p.bias + n, p.epi) : finish4<OUT_FP16>(x, p.bias + n, p.epi);
+__device__ __forceinline__ void store_c4(const P& p, size_t idx, int n, v4f x) {
+    const v2i r = p.out == OUT_BF16 ? finish4_rt<OUT_BF16>(x, p.bias + n, p.epi) : finish4_rt<OUT_FP16>(x, p.bias + n, p.epi);
     *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(p.c) + idx) = r;
 }
