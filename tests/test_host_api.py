@@ -1,0 +1,218 @@
+"""Host-side tests that need no GPU: the package's quantisers / layouts against the oracle, the validation
+rules of the entry points (the cases the reference's own tests hold,
+tests/kernels/test_preshuffle_gemm.py:983-1039), and the C ABI (library loads, exports every declared
+symbol, struct layouts match the header)."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+from flydsl_amd import _lib, layout, quant
+from kernels.gemm.mxfp4_preshuffle import launch_gemm
+from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
+from oracle import psg_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "psgemm.h")
+
+
+# ---- package helpers == oracle --------------------------------------------------------------------
+def test_package_layouts_equal_oracle():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randint(0, 255, (64, 256), generator=g, dtype=torch.uint8)
+    assert np.array_equal(layout.shuffle_weight(x).numpy(), O.shuffle_weight(x.numpy()))
+    h = torch.randn(64, 256, generator=g).to(torch.bfloat16)
+    assert np.array_equal(layout.shuffle_weight(h).view(torch.int16).numpy(), O.shuffle_weight(h.view(torch.int16).numpy()))
+    assert np.array_equal(layout.shuffle_weight_w4(x, 16, False, False).numpy(), O.shuffle_weight_w4(x.numpy()))
+    s = torch.randint(0, 255, (64, 16), generator=g, dtype=torch.uint8)
+    assert np.array_equal(layout.shuffle_scale_w4(s, 1, False).numpy(), O.shuffle_scale_w4(s.numpy()))
+    assert getattr(layout.shuffle_weight(x), "is_shuffled", False)
+    with pytest.raises(AssertionError):
+        layout.shuffle_weight(torch.zeros(20, 64, dtype=torch.int8))
+    with pytest.raises(AssertionError):
+        layout.shuffle_weight(torch.zeros(32, 48, dtype=torch.int8))
+    # leading batch dimension, as the reference's view(-1, ...) allows
+    xb = torch.randint(0, 255, (3, 32, 64), generator=g, dtype=torch.uint8)
+    got = layout.shuffle_weight(xb)
+    for i in range(3):
+        assert np.array_equal(got[i].numpy(), O.shuffle_weight(xb[i].numpy()))
+
+
+def test_package_quantisers_equal_oracle():
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(64, 512, generator=g) * torch.logspace(-3, 3, 64).view(-1, 1)
+    w[7] = 0
+    for qd, kind in ((torch.int8, "int8"), (torch.float8_e4m3fn, "fp8")):
+        y, sc = quant.pertoken_quant(w, quant_dtype=qd)
+        yo, so = O.pertoken_quant(w.numpy(), kind)
+        assert sc.shape == (64, 1) and sc.dtype == torch.float32
+        assert np.array_equal(y.view(torch.uint8).numpy(), yo.view(np.uint8))
+        assert np.array_equal(sc.numpy(), so)
+    p, sc, _ = quant.per_1x32_f4_quant(w)
+    po, so = O.per_1x32_f4_quant(w.numpy())
+    assert np.array_equal(p.view(torch.uint8).numpy(), po) and np.array_equal(sc.view(torch.uint8).numpy(), so)
+    assert np.array_equal(quant.mxfp4_to_f32(p).numpy(), O.mxfp4_to_f32(po))
+    b = torch.arange(256, dtype=torch.uint8)
+    got, want = quant.e8m0_to_f32(b).numpy(), O.e8m0_to_f32(b.numpy())
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    v = torch.cat([torch.linspace(-8, 8, 20001), torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.0, 6.0, 1e-9])])
+    assert np.array_equal(quant.f32_to_e2m1_codes(v).numpy(), O.f32_to_e2m1(v.numpy()))
+    e = torch.tensor([1.0, 1.5, 2.0**-127, 0.0, float("nan"), 3e38, 1.4999999])
+    assert np.array_equal(quant.f32_to_e8m0(e).view(torch.uint8).numpy(), O.f32_to_e8m0(e.numpy()))
+
+
+# ---- validation rules of compile_preshuffle_gemm ---------------------------------------------------
+@pytest.mark.parametrize("tile_m", [48, 80, 112, 144])
+def test_rejects_partial_a_tile(tile_m):
+    with pytest.raises(ValueError, match=r"must be a multiple of"):
+        compile_preshuffle_gemm(N=1024, K=2048, tile_m=tile_m, tile_n=256, tile_k=64, in_dtype="bf16", out_dtype="bf16")
+
+
+@pytest.mark.parametrize("tile_m", [64, 96, 128, 160])
+def test_accepts_whole_a_tile(tile_m):
+    # the reference's case is bf16 with tile_k=64 (2 bytes/element); same byte count with 1-byte elements
+    compile_preshuffle_gemm(N=1024, K=2048, tile_m=tile_m, tile_n=256, tile_k=128, in_dtype="int8", out_dtype="bf16")
+
+
+@pytest.mark.parametrize("bad", [(1,), (1, 2, 3), (-1, 0), (0, -1), 4])
+def test_preload_validation(bad):
+    with pytest.raises((ValueError, TypeError)):
+        compile_preshuffle_gemm(N=1024, K=2048, tile_m=128, tile_n=256, tile_k=64, in_dtype="int8", out_dtype="bf16", preload=bad)
+
+
+def test_other_validation_errors():
+    ok = dict(N=1024, K=2048, tile_m=128, tile_n=256, tile_k=128)
+    with pytest.raises(ValueError, match="in_dtype"):
+        compile_preshuffle_gemm(**ok, in_dtype="fp4")
+    with pytest.raises(ValueError, match="tile_k"):
+        compile_preshuffle_gemm(**{**ok, "tile_k": 96})
+    with pytest.raises(ValueError, match="tile_k"):
+        compile_preshuffle_gemm(**{**ok, "tile_k": 0})
+    with pytest.raises(ValueError, match="epilogue"):
+        compile_preshuffle_gemm(**ok, epilogue="bias_tanh")
+    with pytest.raises(ValueError, match="lds_stage"):
+        compile_preshuffle_gemm(**ok, lds_stage=3)
+    with pytest.raises(ValueError, match="LDS swizzle"):
+        compile_preshuffle_gemm(N=1024, K=768, tile_m=256, tile_n=256, tile_k=384, in_dtype="int8")
+    with pytest.raises(ValueError, match="multiple of 16"):
+        compile_preshuffle_gemm(**{**ok, "N": 1000})
+    with pytest.raises(TypeError):
+        compile_preshuffle_gemm(1024, 2048, 128, 256, 128)  # keyword-only, like the reference
+    fn = compile_preshuffle_gemm(**ok, in_dtype="fp8", waves_per_eu=2, use_async_copy=True, xcd_swizzle=4, preload=(2, 2))
+    assert fn.N == 1024 and fn.K == 2048
+
+
+def test_mxfp4_entry_rejects_what_is_not_built():
+    base = [0, 0, 0, 0, 0, 32, 128, None, 128, 256, 32, 128, 256, "fp4", "bf16", "fp4", 1, -1, -1, -1, -1, -1, -1, 0]
+    for idx, val, exc in ((13, "fp8", NotImplementedError), (15, "fp8", NotImplementedError), (16, 2, NotImplementedError),
+                          (17, 64, NotImplementedError), (12, 64, ValueError), (11, 64, ValueError), (14, "fp32", ValueError),
+                          (6, 256, ValueError)):
+        args = list(base)
+        args[idx] = val
+        with pytest.raises(exc):
+            launch_gemm(*args)
+
+
+# ---- the C ABI -------------------------------------------------------------------------------------
+def _declared_functions():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"^\s*(?:int|uint64_t|const char \*)\s*\**\s*(psg_\w+)\s*\(", text, flags=re.M)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS), names
+    handle = _lib.lib()
+    for n in names:
+        assert getattr(handle, n) is not None
+    assert handle.psg_abi_version() == _lib.ABI_VERSION
+    assert handle.psg_workspace_bytes(16, 6144, 4096, 1) == 0
+
+
+def test_struct_layouts_match_header():
+    src = r'''
+    #include <stdio.h>
+    #include <stddef.h>
+    #include "psgemm.h"
+    int main(void) {
+        printf("%zu %zu %zu %zu %zu %zu\n", sizeof(psg_a8w8_args), offsetof(psg_a8w8_args, workspace_bytes),
+               offsetof(psg_a8w8_args, M), offsetof(psg_a8w8_args, epilogue), offsetof(psg_a8w8_args, force_path),
+               offsetof(psg_a8w8_args, bias));
+        printf("%zu %zu %zu %zu\n", sizeof(psg_mxfp4_args), offsetof(psg_mxfp4_args, M), offsetof(psg_mxfp4_args, out_dtype),
+               offsetof(psg_mxfp4_args, force_path));
+        return 0;
+    }'''
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.run(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
+    a, m = _lib.A8W8Args, _lib.MxArgs
+    want = [ctypes.sizeof(a), a.workspace_bytes.offset, a.M.offset, a.epilogue.offset, a.force_path.offset, a.bias.offset,
+            ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset]
+    assert [int(v) for v in out] == want
+
+
+def test_validation_errors_come_back_as_codes_without_a_gpu():
+    handle = _lib.lib()
+    args = _lib.A8W8Args()
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -1  # PSG_E_NULL
+    assert b"non-NULL" in handle.psg_last_error()
+    args.a = args.b = args.c = args.scale_a = args.scale_b = 0x1000
+    args.M, args.N, args.K = 4, 30, 64
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -2  # PSG_E_SHAPE
+    args.N, args.K = 32, 100
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -2
+    args.K, args.M = 64, 0
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -2
+    args.M, args.in_dtype = 4, 7
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -3  # PSG_E_DTYPE
+    args.in_dtype, args.a = 1, 0x1001
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -6  # PSG_E_ALIGN
+    args.a, args.in_dtype = 0x1000, 3
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -5  # PSG_E_UNSUPPORTED (bf16 inputs)
+    with pytest.raises(ValueError):
+        _lib.check(-2, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(1, "x")
+
+
+def test_stream_argument_forms():
+    assert _lib.stream_handle(0) == 0 and _lib.stream_handle(1234) == 1234
+
+    class S:
+        cuda_stream = 77
+
+    assert _lib.stream_handle(S()) == 77
+    from flydsl_amd import compiler as flyc
+    from flydsl_amd import expr as fx
+
+    assert _lib.stream_handle(fx.Stream(5)) == 5
+    p = flyc.from_c_void_p(fx.Uint8, 0xABC0)
+    assert p.value == 0xABC0 and int(p) == 0xABC0
+    with pytest.raises(TypeError):
+        _lib.stream_handle("stream")
+    calls = []
+    cf = flyc.compile(lambda *a: calls.append(a), 1, 2)
+    cf(3, 4)
+    assert calls == [(1, 2), (3, 4)]
+
+
+def test_product_code_does_not_touch_the_oracle():
+    bad = []
+    for base in ("flydsl_amd", "kernels"):
+        for dirpath, _, files in os.walk(os.path.join(ROOT, base)):
+            for f in files:
+                if f.endswith((".py", ".hip", ".h", ".cpp")):
+                    text = open(os.path.join(dirpath, f)).read()
+                    if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "psg_oracle" in text:
+                        bad.append(os.path.join(dirpath, f))
+    assert not bad, bad
