@@ -1,15 +1,19 @@
 // Memory-bound small-M (M <= 32) path of the 8-bit preshuffle GEMM for gfx950.
 //
 // The whole cost is streaming W once (N*K bytes), so the kernel is organised around the 1 KB preshuffled
-// blocks [N/16][K/64]: a wavefront owns one 16-column n-block and a contiguous slice of K, issues every
-// block load of its slice up front (one fully coalesced 1 KB load per block, 16 bytes per lane, marked
-// non-temporal), and feeds the registers straight into MFMA.  A workgroup is 8 wavefronts =
-// (8/ksplit) n-blocks x ksplit K-slices; the K-slices of one n-block always sit in one workgroup, so the
-// split-K reduction happens in LDS in a fixed order (deterministic, single launch, no workspace).
+// blocks [N/16][K/64]: a wavefront owns one 16-column n-block and a contiguous slice of K, issues the block
+// loads of a chunk of K steps up front (one fully coalesced 1 KB load per block, 16 bytes per lane) and
+// feeds the registers straight into MFMA.  A workgroup is 8 wavefronts = (8/ksplit) n-blocks x ksplit
+// K-slices; the K-slices of one n-block always sit in one workgroup, so the split-K reduction happens in LDS
+// in a fixed order (deterministic, single launch, no workspace).
 //
-// A (at most 32 x K bytes, L2 resident after first touch) is read directly in fragment order:
-// lane (i = lane%16, g = lane/16) needs bytes [16g,16g+16) and [64+16g, 64+16g+16) of row i per 128-byte K step.
-// Rows >= M read as zero through the buffer descriptor bound.
+// A (at most 32 x K bytes, L2 resident after first touch) is needed in fragment order: lane
+// (i = lane%16, g = lane/16) wants bytes [16g,16g+16) and [64+16g, 64+16g+16) of row i per K step, i.e. 16
+// different rows per load instruction.  Reading it that way from global memory costs more address
+// processing than the whole W stream, so each wavefront instead reads its slice of A with row-contiguous
+// loads (32 or 16 lanes per row) into a private 8 KB LDS patch (XOR-swizzled 16-byte chunks) and picks the
+// fragments up from there.  The patch is private to the wavefront: no barrier is involved.
+// Rows >= M and bytes >= K read as zero through the buffer descriptor bound.
 //
 // Operands are swapped like in the tiled kernel (src0 = W fragment, src1 = A fragment): a lane holds
 // C[m = i][n = nblk*16 + g*4 + 0..3].
@@ -18,7 +22,7 @@
 namespace {
 
 constexpr int NW = 8;       // wavefronts per workgroup
-constexpr int UNROLL = 4;   // 128-byte K steps in flight per wavefront
+constexpr int UNROLL = 4;   // 128-byte K steps per chunk when 16 rows of A are staged (2 when 32 rows are)
 
 template <int KIND>
 struct Acc {
@@ -29,10 +33,15 @@ struct Acc<KIND_INT8> {
     using type = v4i;
 };
 
-template <int KIND, int MB, int STORE>
+// NB = n-blocks per wavefront: with two, the A slice a wavefront stages is shared by twice as much of W.
+template <int KIND, int MB, int NB, int STORE>
 __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
-    __shared__ __attribute__((aligned(16))) acc_t red[NW][MB][64];
+    constexpr int ROWS = 16 * MB;          // A rows staged
+    constexpr int SPS = UNROLL / MB;       // K steps per staging pass (patch = ROWS x SPS*128 bytes = 8 KB)
+    constexpr int CPR = SPS * 8;           // 16-byte chunks per staged row (32 or 16)
+    __shared__ __attribute__((aligned(16))) v4i patch[NW][512];
+    __shared__ __attribute__((aligned(16))) acc_t red[NW][NB * MB][64];
 
     const int tid = threadIdx.x;
     const int wave = wave_id();
@@ -41,116 +50,169 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     const int lg = lane >> 4;
     const int K = p.K;
     const int ks = p.ksplit;           // 1, 2, 4 or 8
-    const int nbw = NW / ks;           // n-blocks per workgroup
+    const int nbw = NW / ks;           // wavefront groups (K-slice sets) per workgroup, NB n-blocks each
     const int my_ks = wave % ks;
-    const int my_nb = (int)blockIdx.x * nbw + wave / ks;
+    const int my_nb = ((int)blockIdx.x * nbw + wave / ks) * NB;
     const int n_blocks = p.N >> 4;
     const int steps = (K + 127) >> 7;                    // 128-byte K steps
     const int per = (steps + ks - 1) / ks;               // steps per K-slice
     const int s_begin = my_ks * per;
     const int s_end = (s_begin + per) < steps ? (s_begin + per) : steps;
 
-    acc_t acc[MB];
+    acc_t acc[NB][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) acc[mb] = (acc_t){0, 0, 0, 0};
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) acc[nb][mb] = (acc_t){0, 0, 0, 0};
+
+    // The scales of the outputs this thread will finish are fetched now, so that their latency does not sit
+    // behind the reduction barrier at the very end of the kernel.  Finishing work item t = tid (+ NW*64):
+    // (n-block t/(MB*64) of the workgroup, m-block, lane).
+    constexpr int FIN = (NB * MB * NW * 64 + NW * 64 - 1) / (NW * 64);  // items per thread at ksplit 1
+    float fin_sa[FIN];
+    v4f fin_sb[FIN];
+    if constexpr (STORE != STORE_ACC) {
+#pragma unroll
+        for (int f = 0; f < FIN; f++) {
+            const int t = tid + f * NW * 64;
+            const int nbq = (int)blockIdx.x * nbw * NB + t / (MB * 64);
+            const int m = ((t / 64) % MB) * 16 + li;
+            const bool live = t < nbw * NB * MB * 64 && nbq < n_blocks && m < p.M;
+            fin_sa[f] = live ? p.sa[m] : 0.f;
+            fin_sb[f] = live ? *reinterpret_cast<const v4f*>(p.sb + nbq * 16 + lg * 4) : (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+    }
 
     if (my_nb < n_blocks) {
-        __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (uint64_t)my_nb * 16ull * (uint64_t)K, 16ull * (uint64_t)K);
+        // this wavefront's NB n-blocks; a block past N/16 (odd block count) reads as zero
+        const uint64_t b_left = (uint64_t)(n_blocks - my_nb) * 16ull * (uint64_t)K;
+        const uint64_t b_mine = (uint64_t)NB * 16ull * (uint64_t)K;
+        __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (uint64_t)my_nb * 16ull * (uint64_t)K, b_left < b_mine ? b_left : b_mine);
         __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)p.M * (uint64_t)K);
-        const uint32_t a_voff = (uint32_t)li * (uint32_t)K + (uint32_t)lg * 16u;
+        v4i* my_patch = patch[wave];
+        // staging geometry: item = pass*64 + lane -> (row = item / CPR, chunk = item % CPR)
+        const int st_c = lane % CPR;
+        const int st_r0 = lane / CPR;                   // + pass * (64 / CPR)
+        const uint32_t slice_end = (uint32_t)(s_end * 128 < K ? s_end * 128 : K);
 
-        for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
-            v4i blo[UNROLL], bhi[UNROLL], alo[UNROLL][MB], ahi[UNROLL][MB];
+        for (int s0 = s_begin; s0 < s_end; s0 += SPS) {
+            // 1. A first: it comes from L2 and must not queue behind the W stream (loads return in order)
+            const uint32_t kbase = (uint32_t)s0 * 128u;
+            v4i tmp[8];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const int s = s0 + u;
-                blo[u] = bhi[u] = (v4i){0, 0, 0, 0};
-#pragma unroll
-                for (int mb = 0; mb < MB; mb++) alo[u][mb] = ahi[u][mb] = (v4i){0, 0, 0, 0};
-                if (s < s_end) {  // wave-uniform
-                    const bool has_hi = (s * 128 + 64) < K;
-                    const uint32_t kb = (uint32_t)s * 128u;
-                    const uint32_t boff = (uint32_t)s * 2048u;
-                    blo[u] = buf_load16_nt(rb, (uint32_t)lane * 16u, boff);
-                    if (has_hi) bhi[u] = buf_load16_nt(rb, (uint32_t)lane * 16u, boff + 1024u);
-#pragma unroll
-                    for (int mb = 0; mb < MB; mb++) {
-                        // row select in the bounds-checked VGPR offset: rows >= M read as zero
-                        const uint32_t voff = a_voff + (uint32_t)mb * 16u * (uint32_t)K;
-                        alo[u][mb] = buf_load16(ra, voff, kb);
-                        if (has_hi) ahi[u][mb] = buf_load16(ra, voff, kb + 64u);
-                    }
-                }
+            for (int ps = 0; ps < 8; ps++) {
+                const int r = st_r0 + ps * (64 / CPR);
+                const uint32_t kbyte = kbase + (uint32_t)st_c * 16u;
+                tmp[ps] = buf_load16(ra, kbyte < slice_end ? (uint32_t)r * (uint32_t)K + kbyte : 0xFFFFFFF0u, 0);
             }
+            // 2. the W blocks of this chunk, all in flight at once
+            v4i blo[NB][SPS], bhi[NB][SPS];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int u = 0; u < SPS; u++) {
+                    const int s = s0 + u;
+                    const bool has_lo = s < s_end;                       // wave-uniform
+                    const bool has_hi = has_lo && (s * 128 + 64) < K;    // K % 128 == 64: last step has no upper half
+                    const uint32_t boff = has_lo ? (uint32_t)s * 2048u : 0u;
+                    const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)nb * 16u * (uint32_t)K;
+                    blo[nb][u] = buf_load16_nt(rb, has_lo ? voff : 0xFFFFFFF0u, boff);
+                    bhi[nb][u] = buf_load16_nt(rb, has_hi ? voff : 0xFFFFFFF0u, has_hi ? boff + 1024u : 0u);
+                }
+            // 3. A through the private LDS patch into fragment order while W is still on its way
+#pragma unroll
+            for (int ps = 0; ps < 8; ps++) {
+                const int r = st_r0 + ps * (64 / CPR);
+                my_patch[r * CPR + (st_c ^ (r & 15))] = tmp[ps];
+            }
+            v4i alo[SPS][MB], ahi[SPS][MB];
+#pragma unroll
+            for (int t = 0; t < SPS; t++)
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++) {
-                    if constexpr (KIND == KIND_INT8) {
-                        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[u], alo[u][mb], acc[mb], 0, 0, 0);
-                        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[u], ahi[u][mb], acc[mb], 0, 0, 0);
-                    } else {
-                        const v8i bf = {blo[u][0], blo[u][1], blo[u][2], blo[u][3], bhi[u][0], bhi[u][1], bhi[u][2], bhi[u][3]};
-                        const v8i af = {alo[u][mb][0], alo[u][mb][1], alo[u][mb][2], alo[u][mb][3],
-                                        ahi[u][mb][0], ahi[u][mb][1], ahi[u][mb][2], ahi[u][mb][3]};
-                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[mb], 0, 0, 0, 0, 0, 0);
-                    }
+                    const int r = mb * 16 + li;
+                    alo[t][mb] = my_patch[r * CPR + ((t * 8 + lg) ^ (r & 15))];
+                    ahi[t][mb] = my_patch[r * CPR + ((t * 8 + 4 + lg) ^ (r & 15))];
                 }
-            }
+            // 4. MFMA as W arrives
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int t = 0; t < SPS; t++)
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++) {
+                        if constexpr (KIND == KIND_INT8) {
+                            acc[nb][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[nb][t], alo[t][mb], acc[nb][mb], 0, 0, 0);
+                            acc[nb][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[nb][t], ahi[t][mb], acc[nb][mb], 0, 0, 0);
+                        } else {
+                            const v8i bf = {blo[nb][t][0], blo[nb][t][1], blo[nb][t][2], blo[nb][t][3],
+                                            bhi[nb][t][0], bhi[nb][t][1], bhi[nb][t][2], bhi[nb][t][3]};
+                            const v8i af = {alo[t][mb][0], alo[t][mb][1], alo[t][mb][2], alo[t][mb][3],
+                                            ahi[t][mb][0], ahi[t][mb][1], ahi[t][mb][2], ahi[t][mb][3]};
+                            acc[nb][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[nb][mb], 0, 0, 0, 0, 0, 0);
+                        }
+                    }
         }
     }
 
     // split-K reduction through LDS, fixed order
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) red[wave][mb][lane] = acc[mb];
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) red[wave][nb * MB + mb][lane] = acc[nb][mb];
     __syncthreads();
 
-    // work item t < nbw*MB*64 finishes (n-block t/(MB*64), m-block, lane); up to 1024 items for 512 threads
-    for (int t = tid; t < nbw * MB * 64; t += NW * 64) {
-        const int nbi = t / (MB * 64);
-        const int mb = (t / 64) % MB;
-        const int nb = (int)blockIdx.x * nbw + nbi;
-        acc_t sum = red[nbi * ks][mb][lane];
-        for (int j = 1; j < ks; j++) sum += red[nbi * ks + j][mb][lane];
-        const int m = mb * 16 + li;
-        const int n = nb * 16 + lg * 4;
-        if (nb < n_blocks && m < p.M) {
-            const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
-            if constexpr (STORE == STORE_ACC) {
-                *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = sum;
-            } else {
-                const float sa = p.sa[m];
-                const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
-                const v4f x = {((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
-                               ((float)sum[3] * sa) * sb[3]};
-                store_c4(p, idx, n, x);
+#pragma unroll
+    for (int f = 0; f < FIN; f++) {
+        const int t = tid + f * NW * 64;
+        if (t < nbw * NB * MB * 64) {
+            const int nbi = t / (MB * 64);  // n-block of the workgroup: wavefront group nbi / NB, its block nbi % NB
+            const int mb = (t / 64) % MB;
+            const int grp = nbi / NB, frag = (nbi % NB) * MB + mb;
+            const int nbq = (int)blockIdx.x * nbw * NB + nbi;
+            acc_t sum = red[grp * ks][frag][lane];
+            for (int j = 1; j < ks; j++) sum += red[grp * ks + j][frag][lane];
+            const int m = mb * 16 + li;
+            const int n = nbq * 16 + lg * 4;
+            if (nbq < n_blocks && m < p.M) {
+                const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
+                if constexpr (STORE == STORE_ACC) {
+                    *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = sum;
+                } else {
+                    const float sa = fin_sa[f];
+                    const v4f sb = fin_sb[f];
+                    const v4f x = {((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
+                                   ((float)sum[3] * sa) * sb[3]};
+                    store_c4(p, idx, n, x);
+                }
             }
         }
     }
 }
 
-template <int KIND, int MB, int STORE>
+template <int KIND, int MB, int NB, int STORE>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
-    const int nbw = NW / p.ksplit;
+    const int per_wg = (NW / p.ksplit) * NB;  // n-blocks per workgroup
     const int n_blocks = p.N / 16;
-    const int grid = (n_blocks + nbw - 1) / nbw;
-    hipLaunchKernelGGL((k_a8w8_smallm<KIND, MB, STORE>), dim3(grid), dim3(NW * 64), 0, stream, p);
+    const int grid = (n_blocks + per_wg - 1) / per_wg;
+    hipLaunchKernelGGL((k_a8w8_smallm<KIND, MB, NB, STORE>), dim3(grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
+}
+
+template <int KIND, int STORE>
+hipError_t launch_kind(const A8W8Params& p, int nb, hipStream_t stream) {
+    const int mb = p.M <= 16 ? 1 : 2;
+    if (mb == 1) return nb == 2 ? launch_one<KIND, 1, 2, STORE>(p, stream) : launch_one<KIND, 1, 1, STORE>(p, stream);
+    return nb == 2 ? launch_one<KIND, 2, 2, STORE>(p, stream) : launch_one<KIND, 2, 1, STORE>(p, stream);
 }
 
 }  // namespace
 
-// Host entry used by the C-ABI layer.  Requires 1 <= M <= 32 and p.ksplit in {1,2,4,8}.
-hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, hipStream_t stream) {
-    const int mb = p.M <= 16 ? 1 : 2;
-#define PSG_GO(KIND_, MB_)                                                                    \
-    return store == STORE_ACC ? launch_one<KIND_, MB_, STORE_ACC>(p, stream) : launch_one<KIND_, MB_, STORE_C>(p, stream);
-    if (kind == KIND_INT8) {
-        if (mb == 1) { PSG_GO(KIND_INT8, 1) } else { PSG_GO(KIND_INT8, 2) }
-    }
-    if (kind == KIND_FP8) {
-        if (mb == 1) { PSG_GO(KIND_FP8, 1) } else { PSG_GO(KIND_FP8, 2) }
-    }
-#undef PSG_GO
+// Host entry used by the C-ABI layer.  Requires 1 <= M <= 32, p.ksplit in {1,2,4,8}, nb (n-blocks per wavefront) in {1,2}.
+hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream) {
+    if (kind == KIND_INT8)
+        return store == STORE_ACC ? launch_kind<KIND_INT8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_INT8, STORE_C>(p, nb, stream);
+    if (kind == KIND_FP8)
+        return store == STORE_ACC ? launch_kind<KIND_FP8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_FP8, STORE_C>(p, nb, stream);
     return hipErrorInvalidValue;
 }

@@ -9,7 +9,7 @@
 #include "psg_common.h"
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
-hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, hipStream_t stream);
+hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream);
 hipError_t psg_launch_mxfp4_tiled(const MxParams& p, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
 
@@ -33,7 +33,7 @@ int hip_fail(hipError_t e, const char* what) {
 bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int kSmallM = 32;      // rows the split-K path covers
-constexpr int kTargetWaves = 2048;  // wavefronts wanted in flight for the streaming path (8 per CU)
+constexpr int kTargetWaves = 1536;  // wavefronts wanted in flight for the streaming path (6 per CU)
 
 int pick_ksplit(int units, int steps) {
     int ks = 1;
@@ -124,8 +124,12 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
     if (small) {
-        p.ksplit = pick_ksplit(a->N / 16, (a->K + 127) / 128);
-        e = psg_launch_a8w8_smallm(p, kind, store, static_cast<hipStream_t>(stream));
+        // two n-blocks per wavefront halve the A traffic per byte of W; keep one when that would leave too few
+        // wavefronts to cover the memory latency
+        const int steps = (a->K + 127) / 128;
+        const int nb = (a->N / 16) >= 256 ? 2 : 1;
+        p.ksplit = pick_ksplit((a->N / 16 + nb - 1) / nb, steps);
+        e = psg_launch_a8w8_smallm(p, kind, store, nb, static_cast<hipStream_t>(stream));
     } else {
         const Tile t = pick_tile(a->M, a->N, false, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
         p.ksplit = 1;
