@@ -30,6 +30,18 @@ struct Acc<KIND_INT8> {
     using type = v4i;
 };
 
+// MFMA through inline assembly with the accumulator constrained to the AGPR file ("+a").  With the builtin
+// the register allocator is free to place accumulators in either file; at 256 accumulator registers per lane
+// it then shuffles them between the files inside the main loop.  The accumulator of each call is both vDst
+// and SrcC (in-place accumulate); the compiler does not know these are MFMAs, so the kernel never reads an
+// accumulator with a non-MFMA instruction without a barrier and explicit wait states in between.
+__device__ __forceinline__ void mfma_f8(v4f& c, const v8i& a, const v8i& b) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_i8(v4i& c, const v4i& a, const v4i& b) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 // LDS byte offset of 16-byte chunk `kc` (0..7) of row `row` inside one A stage
 __device__ __forceinline__ int lds_off(int row, int kc) { return row * TK + ((kc ^ ((row >> 1) & 7)) << 4); }
 
@@ -50,7 +62,7 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
 template <int KIND, int MR, int NR, int STORE>
-__global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
+__global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr int TM = 16 * MR;
     constexpr int TN = 64 * NR;
@@ -93,97 +105,128 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (acc_t){0, 0, 0, 0};
 
+    // Register sets: areg holds the A tile of the next K step on its way to LDS (each register is written to
+    // LDS and immediately reloaded for the step after); blo/bhi[q] hold the W fragments of a step with parity q.
     v4i areg[A_LOADS];
     v4i blo[2][NR], bhi[2][NR];
 
-    // Loads never sit under control flow: a K step past the end (prefetch of the last iteration) and an A
+    // Loads never sit under control flow: a K step past the end (prefetch of the last iterations) and an A
     // chunk past K (only when K % 128 == 64) are redirected past the descriptor bound, where the hardware
     // returns zero without touching memory.  Selecting on the ADDRESS keeps the loaded registers untouched
     // until they are used, so no wait is forced early.
-    auto load_a = [&](int kt) {
+    auto load_a1 = [&](int kt, int j, v4i& dst) {
         const uint32_t k0 = (uint32_t)kt * TK;
         const bool in_k = (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
-#pragma unroll
-        for (int j = 0; j < A_LOADS; j++) {
-            const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0;
-            areg[j] = buf_load16(ra, in_k ? off : 0xFFFFFFF0u, 0);
-        }
+        const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0;
+        dst = buf_load16(ra, in_k ? off : 0xFFFFFFF0u, 0);
     };
-    auto store_a = [&](int stage) {
-#pragma unroll
-        for (int j = 0; j < A_LOADS; j++) {
-            const int row = a_row0 + 32 * j;
-            *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, a_kc)]) = areg[j];
-        }
+    auto store_a1 = [&](int stage, int j, const v4i& src) {
+        *reinterpret_cast<v4i*>(&lds[stage][lds_off(a_row0 + 32 * j, a_kc)]) = src;
     };
-    auto load_b = [&](int kt, v4i* lo, v4i* hi) {
-        const bool has_lo = (kt * TK) < K;
-        const bool has_hi = (kt * TK + 64) < K;
-        const uint32_t koff = has_lo ? (uint32_t)kt * 2048u : 0u;
-#pragma unroll
-        for (int ni = 0; ni < NR; ni++) {
-            // n-block select in the bounds-checked VGPR offset (blocks >= N/16 read as zero), K position in
-            // the scalar offset
-            const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
-            lo[ni] = buf_load16(rb, has_lo ? voff : 0xFFFFFFF0u, koff);
-            hi[ni] = buf_load16(rb, has_hi ? voff : 0xFFFFFFF0u, has_hi ? koff + 1024u : 0u);
-        }
+    // W fragment load number idx of a K step: n-block idx/2, 64-byte half idx%2.  The n-block select sits in
+    // the bounds-checked VGPR offset (blocks >= N/16 read as zero), the K position in the scalar offset.
+    auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi) {
+        const int ni = idx >> 1;
+        const bool has = (kt * TK + (idx & 1) * 64) < K;
+        const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
+        const v4i v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, has ? (uint32_t)kt * 2048u + (uint32_t)(idx & 1) * 1024u : 0u);
+        if (idx & 1) hi[ni] = v; else lo[ni] = v;
     };
-    // A fragments are read one m-block ahead of the MFMAs that use them (register double buffer), so the
-    // LDS latency of block mi+1 hides behind the MFMAs of block mi.
     auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {
         const int row = mi * 16 + li;
         flo = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
         fhi = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
     };
-    auto compute = [&](int stage, const v4i* lo, const v4i* hi) {
+
+    // One K step (tile kt, parity S): MFMAs on LDS stage S and W set S, with the memory work of the next
+    // steps dealt out between the m-blocks so that no instruction queue (texture addresser, LDS) ever holds
+    // up MFMA issue:
+    //   first half of the m-blocks : the W fragment loads of step kt+1 -> W set S^1
+    //   second half                : A tile of step kt+1 (in registers, loaded one step ago) -> LDS stage S^1,
+    //                                each register reloaded at once with its part of the A tile of step kt+2
+    //   every m-block              : LDS read of the next m-block's A fragment (register double buffer)
+    auto step = [&](int kt, auto SP) {
+        constexpr int S = decltype(SP)::value;
+        constexpr int HALF = MR / 2;
+        constexpr int B_PER = (2 * NR + HALF - 1) / HALF;
         v4i flo[2], fhi[2];
-        read_frag(stage, 0, flo[0], fhi[0]);
-#pragma unroll
-        for (int mi = 0; mi < MR; mi++) {
-            if (mi + 1 < MR) read_frag(stage, mi + 1, flo[(mi + 1) & 1], fhi[(mi + 1) & 1]);
-            // keep the prefetch ahead of this block's MFMAs (the machine scheduler would otherwise sink it)
+        read_frag(S, 0, flo[0], fhi[0]);
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            if constexpr (mi + 1 < MR) read_frag(S, mi + 1, flo[(mi + 1) & 1], fhi[(mi + 1) & 1]);
+            if constexpr (mi < HALF) {
+                static_for<B_PER>([&](auto Q) {
+                    constexpr int idx = mi * B_PER + decltype(Q)::value;
+                    if constexpr (idx < 2 * NR) load_b1(kt + 1, idx, blo[S ^ 1], bhi[S ^ 1]);
+                });
+            } else {
+                constexpr int j = mi - HALF;
+                if constexpr (j < A_LOADS) {
+                    store_a1(S ^ 1, j, areg[j]);
+                    load_a1(kt + 2, j, areg[j]);
+                }
+            }
+            // keep the memory instructions above ahead of this block's MFMAs (the machine scheduler would
+            // otherwise cluster them at the top of the step)
             __builtin_amdgcn_sched_barrier(0);
             const v4i alo = flo[mi & 1], ahi = fhi[mi & 1];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
-                for (int ni = 0; ni < NR; ni++) {
-                    acc[mi][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo[ni], alo, acc[mi][ni], 0, 0, 0);
-                    acc[mi][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi[ni], ahi, acc[mi][ni], 0, 0, 0);
-                }
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[S][ni], alo);
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[S][ni], ahi);
             } else {
                 const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
-                    const v8i bf = {lo[ni][0], lo[ni][1], lo[ni][2], lo[ni][3], hi[ni][0], hi[ni][1], hi[ni][2], hi[ni][3]};
-                    acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[mi][ni], 0, 0, 0, 0, 0, 0);
+                    const v8i bf = {blo[S][ni][0], blo[S][ni][1], blo[S][ni][2], blo[S][ni][3],
+                                    bhi[S][ni][0], bhi[S][ni][1], bhi[S][ni][2], bhi[S][ni][3]};
+                    mfma_f8(acc[mi][ni], bf, af);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-        }
+        });
+        __syncthreads();
     };
 
-    // prologue: stage 0
-    load_a(0);
-    load_b(0, blo[0], bhi[0]);
-    store_a(0);
+    // prologue: A(0) -> LDS stage 0, A(1) -> registers, W(0) -> set 0
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) load_a1(0, j, areg[j]);
+#pragma unroll
+    for (int idx = 0; idx < 2 * NR; idx++) load_b1(0, idx, blo[0], bhi[0]);
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) {
+        store_a1(0, j, areg[j]);
+        load_a1(1, j, areg[j]);
+    }
     __syncthreads();
 
     // Two K steps per iteration (LDS / register ping-pong).  When the step count is odd the last "odd" step
     // multiplies zero operands (its loads were redirected past the bounds): harmless, and the loop body stays
     // free of control flow, which the software pipeline needs.
     for (int kt = 0; kt < KT; kt += 2) {
-        load_a(kt + 1);
-        load_b(kt + 1, blo[1], bhi[1]);
-        compute(0, blo[0], bhi[0]);
-        store_a(1);
-        __syncthreads();
+        step(kt, std::integral_constant<int, 0>{});
+        step(kt + 1, std::integral_constant<int, 1>{});
+    }
 
-        load_a(kt + 2);
-        load_b(kt + 2, blo[0], bhi[0]);
-        compute(1, blo[1], bhi[1]);
-        store_a(0);
-        __syncthreads();
+    // the last MFMAs (up to 8 passes of 4 cycles each) must have left the pipeline before anything else reads
+    // an accumulator: the loop's final barrier is followed by explicit wait states
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // epilogue operands, fetched in one batch (one memory latency for the whole tile, not one per fragment)
+    float sa_v[MR];
+    v4f sb_v[NR];
+    if constexpr (STORE != STORE_ACC) {
+#pragma unroll
+        for (int mi = 0; mi < MR; mi++) {
+            const int m = m0 + mi * 16 + li;
+            sa_v[mi] = p.sa[m < p.M ? m : p.M - 1];
+        }
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) {
+            const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+            sb_v[ni] = *reinterpret_cast<const v4f*>(p.sb + (n < p.N ? n : 0));
+        }
     }
 
     // epilogue: lane owns C[m0 + mi*16 + li][n0 + (wave*NR + ni)*16 + lg*4 + 0..3].  Compile-time indices only,
@@ -193,7 +236,7 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
         const int m = m0 + mi * 16 + li;
         if (m < p.M) {
             float sa = 0.f;
-            if constexpr (STORE != STORE_ACC) sa = p.sa[m];
+            if constexpr (STORE != STORE_ACC) sa = sa_v[mi];
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
                 const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
@@ -203,7 +246,7 @@ __global__ void __launch_bounds__(256) k_a8w8_tiled(A8W8Params p) {
                     if constexpr (STORE == STORE_ACC) {
                         *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = r;
                     } else {
-                        const v4f sb = *reinterpret_cast<const v4f*>(p.sb + n);
+                        const v4f sb = sb_v[ni];
                         const v4f x = {((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2],
                                        ((float)r[3] * sa) * sb[3]};
                         if constexpr (STORE == STORE_C) {

@@ -45,26 +45,35 @@ struct Tile {
     int m, n;
 };
 
-// Tile choice for the MFMA mainloop: widest N tile that N supports, then the M tile with the best
-// product of CU fill, padding efficiency and per-tile efficiency (bigger tiles reuse operands more).
+// Tile choice for the MFMA mainloop.  Each shape has a measured relative efficiency at full occupancy (the
+// 128-row tiles run two workgroups per CU, so one workgroup's epilogue overlaps the other's mainloop; the 256-row
+// tile has the highest operand reuse but runs alone).  The score multiplies that by how evenly the tiles fill the
+// CUs' workgroup slots and by the fraction of each tile that is not padding.
 Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
-    static const int shapes8[][2] = {{256, 256}, {128, 256}, {64, 256}, {32, 256}, {128, 128}, {64, 64}};
-    static const int shapesx[][2] = {{256, 256}, {128, 256}, {64, 256}, {32, 256}, {64, 128}, {32, 128}};
-    const int(*shapes)[2] = mx ? shapesx : shapes8;
+    struct Shape {
+        int m, n, per_cu;
+        double eff;
+    };
+    static const Shape shapes8[] = {{128, 256, 2, 1.00}, {256, 256, 1, 0.95}, {64, 256, 2, 0.62}, {32, 256, 3, 0.36},
+                                    {128, 128, 2, 0.70}, {64, 64, 5, 0.25}};
+    static const Shape shapesx[] = {{128, 256, 2, 1.00}, {256, 256, 1, 0.95}, {64, 256, 2, 0.62}, {32, 256, 3, 0.36},
+                                    {64, 128, 3, 0.40}, {32, 128, 4, 0.25}};
+    const Shape* shapes = mx ? shapesx : shapes8;
     for (int i = 0; i < 6; i++)
-        if (shapes[i][0] == hint_m && shapes[i][1] == hint_n) return {hint_m, hint_n};
+        if (shapes[i].m == hint_m && shapes[i].n == hint_n) return {hint_m, hint_n};
     double best = -1.0;
-    Tile t = {shapes[0][0], shapes[0][1]};
+    Tile t = {shapes[0].m, shapes[0].n};
     for (int i = 0; i < 6; i++) {
-        const int tm = shapes[i][0], tn = shapes[i][1];
+        const int tm = shapes[i].m, tn = shapes[i].n;
         const long tiles_m = (M + tm - 1) / tm, tiles_n = (N + tn - 1) / tn;
         const long tiles = tiles_m * tiles_n;
-        const long rounds = (tiles + 255) / 256;
-        const double fill = (double)tiles / (double)(rounds * 256);
+        const long slots = 256L * shapes[i].per_cu;
+        const long rounds = (tiles + slots - 1) / slots;
+        // a partly filled last round still costs a full tile time on the CUs it touches
+        const double fill = (double)tiles / (double)(rounds * slots);
+        const double busy = tiles >= slots ? fill : (double)(tiles < 256 ? tiles : 256) / 256.0;
         const double pad = ((double)M / (double)(tiles_m * tm)) * ((double)N / (double)(tiles_n * tn));
-        // operand bytes fetched per MFMA: (tm + tn) / (tm * tn), relative to the 256x256 tile
-        const double reuse = (2.0 / 256.0) / ((double)(tm + tn) / ((double)tm * tn));
-        const double score = fill * pad * (0.35 + 0.65 * reuse);
+        const double score = busy * pad * shapes[i].eff;
         if (score > best) {
             best = score;
             t = {tm, tn};
