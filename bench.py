@@ -221,6 +221,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device-to-device copy a few times (the known-size kernel that the "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -235,6 +238,15 @@ def main():
     from flydsl_amd import _lib
 
     _lib.lib()  # fail loudly if the HIP library is missing
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": 5}))
+        return
 
     family, kind, M, N, K, bound = WORKLOADS[args.workload]
     small = bound == "hbm"

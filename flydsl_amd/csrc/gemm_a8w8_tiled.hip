@@ -1,4 +1,4 @@
-// Compute-bound mainloop of the 8-bit preshuffle GEMM for gfx950.
+// Compute-bound mainloop of the preshuffle GEMM for gfx950: int8, OCP fp8 and MXFP4 operands.
 //
 //   C[M,N] = A[M,K] * W[N,K]^T, W preshuffled into 1 KB fragment blocks [N/16][K/64][klane 4][nlane 16][16 B].
 //
@@ -13,6 +13,10 @@
 //             bytes [16g,16g+16) and [64+16g, 64+16g+16) of the 128-byte K step (g = lane/16) so that
 //             each half is exactly one preshuffled block; A uses the same K order.
 //       int8: two v_mfma_i32_16x16x64_i8 per K step (one per 64-byte half), int32 accumulate (exact).
+//       mxfp4: K is packed two elements per byte, so a 128-byte K step is 256 elements = one chunk of the
+//             shuffled e8m0 scale layout; two v_mfma_scale_f32_16x16x128_f8f6f4 per step (one per 64-byte
+//             half = one preshuffled block), each lane's 16 bytes are 32 consecutive K elements sharing one
+//             scale byte, selected from the lane's scale dword with op_sel (byte = 2*half + 16-row half).
 //   * Workgroup ids are remapped so that the ids the hardware deals to one XCD cover a compact
 //     group_m x tiles_n patch of tiles (A and B panels stay in that XCD's L2).
 #include "psg_common.h"
@@ -40,6 +44,13 @@ __device__ __forceinline__ void mfma_f8(v4f& c, const v8i& a, const v8i& b) {
 }
 __device__ __forceinline__ void mfma_i8(v4i& c, const v4i& a, const v4i& b) {
     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+// fp4 x fp4 with per-lane e8m0 scales: scale byte of src0 = 2*HI + LO0 of dword s0, of src1 = 2*HI + LO1 of s1
+template <int HI, int LO0, int LO1>
+__device__ __forceinline__ void mfma_mx(v4f& c, const v4i& a, const v4i& b, int s0, int s1) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%7,0] cbsz:4 blgp:4"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "v"(s0), "v"(s1), "n"(LO0), "n"(LO1), "n"(HI));
 }
 
 // LDS byte offset of 16-byte chunk `kc` (0..7) of row `row` inside one A stage
@@ -82,7 +93,8 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     tile_coords((int)blockIdx.x, tiles_m, tiles_n, p.group_m, tm, tn);
     const int m0 = tm * TM;
     const int n0 = tn * TN;
-    const int K = p.K;
+    // K counts BYTES of one operand row from here on (two fp4 elements per byte)
+    const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : p.K;
     const int KT = (K + TK - 1) / TK;
 
     // A: this tile's rows; rows >= M read as zero through the descriptor bound
@@ -93,6 +105,22 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)K;
     const uint64_t b_total = (uint64_t)p.N * (uint64_t)K;
     __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
+
+    // MXFP4 scales: 256 bytes per (32-row chunk, 256-K chunk); this tile's / this wave's chunks; chunks past the
+    // end read as zero (scale byte 0 = 2^-127, multiplied by operands that are zero too)
+    constexpr int MP = MR / 2 > 0 ? MR / 2 : 1, NP = NR / 2 > 0 ? NR / 2 : 1;
+    __amdgpu_buffer_rsrc_t rsa = ra, rsb = ra;
+    uint32_t chunk_bytes = 0;
+    if constexpr (KIND == KIND_MXFP4) {
+        static_assert(KIND != KIND_MXFP4 || (MR % 2 == 0 && NR % 2 == 0), "scale chunks cover 32 rows");
+        chunk_bytes = (uint32_t)KT * 256u;
+        const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5), sa_first = (uint64_t)(m0 >> 5);
+        rsa = make_rsrc(p.mx_sa + sa_first * chunk_bytes, (sa_chunks - sa_first) * chunk_bytes);
+        const uint64_t sb_chunks = (uint64_t)(p.N >> 5), sb_first = (uint64_t)((n0 >> 5) + wave * NP);
+        rsb = make_rsrc(p.mx_sb + (sb_first < sb_chunks ? sb_first : sb_chunks) * chunk_bytes,
+                        sb_first < sb_chunks ? (sb_chunks - sb_first) * chunk_bytes : 0);
+    }
+    int sav[2][MP], sbv[2][NP];
 
     // per-thread A copy geometry: chunk c = tid + 256*j -> (row = c/8, kc = c%8)
     const int a_row0 = tid >> 3;
@@ -125,6 +153,16 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     };
     // W fragment load number idx of a K step: n-block idx/2, 64-byte half idx%2.  The n-block select sits in
     // the bounds-checked VGPR offset (blocks >= N/16 read as zero), the K position in the scalar offset.
+    // MXFP4: load number 2*NR + q fetches scale dword q of the step (A-side chunks first, then W-side)
+    auto load_sc1 = [&](int kt, int q, int* sa_dst, int* sb_dst) {
+        const bool has = kt < KT;
+        const uint32_t soff = has ? (uint32_t)kt * 256u : 0u;
+        if (q < MP) {
+            sa_dst[q] = buf_load4(rsa, has ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
+        } else {
+            sb_dst[q - MP] = buf_load4(rsb, has ? (uint32_t)(q - MP) * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
+        }
+    };
     auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi) {
         const int ni = idx >> 1;
         const bool has = (kt * TK + (idx & 1) * 64) < K;
@@ -148,7 +186,8 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     auto step = [&](int kt, auto SP) {
         constexpr int S = decltype(SP)::value;
         constexpr int HALF = MR / 2;
-        constexpr int B_PER = (2 * NR + HALF - 1) / HALF;
+        constexpr int N_LOADS = 2 * NR + (KIND == KIND_MXFP4 ? MP + NP : 0);  // W fragments (+ scale dwords)
+        constexpr int B_PER = (N_LOADS + HALF - 1) / HALF;
         v4i flo[2], fhi[2];
         read_frag(S, 0, flo[0], fhi[0]);
         static_for<MR>([&](auto MI) {
@@ -158,6 +197,7 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
                 static_for<B_PER>([&](auto Q) {
                     constexpr int idx = mi * B_PER + decltype(Q)::value;
                     if constexpr (idx < 2 * NR) load_b1(kt + 1, idx, blo[S ^ 1], bhi[S ^ 1]);
+                    else if constexpr (idx < N_LOADS) load_sc1(kt + 1, idx - 2 * NR, sav[S ^ 1], sbv[S ^ 1]);
                 });
             } else {
                 constexpr int j = mi - HALF;
@@ -175,6 +215,15 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
                 for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[S][ni], alo);
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[S][ni], ahi);
+            } else if constexpr (KIND == KIND_MXFP4) {
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    mfma_mx<0, ni & 1, mi & 1>(acc[mi][ni], blo[S][ni], alo, sbv[S][ni / 2], sav[S][mi / 2]);
+                });
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    mfma_mx<1, ni & 1, mi & 1>(acc[mi][ni], bhi[S][ni], ahi, sbv[S][ni / 2], sav[S][mi / 2]);
+                });
             } else {
                 const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
 #pragma unroll
@@ -194,6 +243,10 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     for (int j = 0; j < A_LOADS; j++) load_a1(0, j, areg[j]);
 #pragma unroll
     for (int idx = 0; idx < 2 * NR; idx++) load_b1(0, idx, blo[0], bhi[0]);
+    if constexpr (KIND == KIND_MXFP4) {
+#pragma unroll
+        for (int q = 0; q < MP + NP; q++) load_sc1(0, q, sav[0], sbv[0]);
+    }
 #pragma unroll
     for (int j = 0; j < A_LOADS; j++) {
         store_a1(0, j, areg[j]);
@@ -216,7 +269,7 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
     // epilogue operands, fetched in one batch (one memory latency for the whole tile, not one per fragment)
     float sa_v[MR];
     v4f sb_v[NR];
-    if constexpr (STORE != STORE_ACC) {
+    if constexpr (STORE != STORE_ACC && KIND != KIND_MXFP4) {
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) {
             const int m = m0 + mi * 16 + li;
@@ -236,7 +289,7 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
         const int m = m0 + mi * 16 + li;
         if (m < p.M) {
             float sa = 0.f;
-            if constexpr (STORE != STORE_ACC) sa = sa_v[mi];
+            if constexpr (STORE != STORE_ACC && KIND != KIND_MXFP4) sa = sa_v[mi];
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
                 const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
@@ -246,9 +299,14 @@ __global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Param
                     if constexpr (STORE == STORE_ACC) {
                         *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = r;
                     } else {
-                        const v4f sb = sb_v[ni];
-                        const v4f x = {((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2],
-                                       ((float)r[3] * sa) * sb[3]};
+                        v4f x;
+                        if constexpr (KIND == KIND_MXFP4) {
+                            x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};  // scales were applied by the MFMA
+                        } else {
+                            const v4f sb = sb_v[ni];
+                            x = (v4f){((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2],
+                                      ((float)r[3] * sa) * sb[3]};
+                        }
                         if constexpr (STORE == STORE_C) {
                             *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(p.c) + idx) = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
                         } else {
@@ -277,16 +335,21 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
     PSG_CASE(8, 4)
     PSG_CASE(4, 4)
     PSG_CASE(2, 4)
-    PSG_CASE(8, 2)
-    PSG_CASE(4, 1)
+    if constexpr (KIND == KIND_MXFP4) {
+        PSG_CASE(4, 2)
+        PSG_CASE(2, 2)
+    } else {
+        PSG_CASE(8, 2)
+        PSG_CASE(4, 1)
+    }
 #undef PSG_CASE
     return hipErrorInvalidConfiguration;
 }
 
 }  // namespace
 
-// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8.  tile_m x tile_n must be one of the
-// instantiated shapes: 256x256, 128x256, 64x256, 32x256, 128x128, 64x64.
+// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8 / KIND_MXFP4.  tile_m x tile_n must be one of the
+// instantiated shapes: 256x256, 128x256, 64x256, 32x256, then 128x128 and 64x64 (8-bit) or 64x128 and 32x128 (MXFP4).
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
     if (store == STORE_C && (p.epi != EPI_NONE || p.out != OUT_BF16)) store = STORE_C_GENERIC;
     if (kind == KIND_INT8) {
@@ -298,6 +361,11 @@ hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int t
         if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);
         if (store == STORE_C_GENERIC) return launch_shape<KIND_FP8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
         return launch_shape<KIND_FP8, STORE_C>(p, tile_m, tile_n, stream);
+    }
+    if (kind == KIND_MXFP4) {
+        if (store == STORE_ACC) return launch_shape<KIND_MXFP4, STORE_ACC>(p, tile_m, tile_n, stream);
+        if (store == STORE_C_GENERIC) return launch_shape<KIND_MXFP4, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
+        return launch_shape<KIND_MXFP4, STORE_C>(p, tile_m, tile_n, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -8,29 +8,13 @@
 //     the four bytes (128-K half kh, 16-row half h) -> byte kh*2 + h, selected with the MFMA's opsel.
 //   * Operands are swapped (src0 = W, src1 = A) so a lane ends up with 4 consecutive N columns.
 //
-// Two kernels: a tiled one (A staged through swizzled LDS, 4 wavefronts along N) and a small-M one
-// (M <= 32, wavefront = one 32-column n-pair x a K slice, LDS split-K reduction in a fixed order).
+// This file holds the small-M kernel (M <= 32, wavefront = one 32-column n-pair x a K slice, LDS split-K
+// reduction in a fixed order); the tiled MFMA mainloop shares its source with the 8-bit kernels.
 #include "psg_common.h"
 
 namespace {
 
 constexpr int TKB = 128;  // bytes of packed K per mainloop step (= 256 K elements = one scale chunk)
-
-__device__ __forceinline__ int lds_off(int row, int kc) { return row * TKB + ((kc ^ ((row >> 1) & 7)) << 4); }
-
-__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
-    const int num = tiles_m * tiles_n;
-    const int q = num >> 3, r = num & 7;
-    const int xcd = id & 7, in_xcd = id >> 3;
-    const int wg = xcd * q + (xcd < r ? xcd : r) + in_xcd;
-    const int per_group = group_m * tiles_n;
-    const int g = wg / per_group;
-    const int first_m = g * group_m;
-    const int size_m = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-    const int in_g = wg - g * per_group;
-    tm = first_m + in_g % size_m;
-    tn = in_g / size_m;
-}
 
 // fp4 operands occupy the low four dwords of the eight-dword MFMA operand
 __device__ __forceinline__ v8i widen(v4i x) { return __builtin_shufflevector(x, x, 0, 1, 2, 3, -1, -1, -1, -1); }
@@ -48,153 +32,6 @@ __device__ __forceinline__ void store_mx4(const P& p, int store, size_t idx, v4f
         v2i r = p.out == OUT_BF16 ? pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]) : pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
         *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(p.c) + idx) = r;
     }
-}
-
-// ------------------------------------------------------------------------------------------------
-// tiled kernel: tile (16*MR) x (64*NR) x 256 K; MR and NR even (scale chunks cover 32 rows)
-// ------------------------------------------------------------------------------------------------
-template <int MR, int NR, int STORE>
-__global__ void __launch_bounds__(256) k_mxfp4_tiled(MxParams p) {
-    constexpr int TM = 16 * MR;
-    constexpr int TN = 64 * NR;
-    constexpr int A_LOADS = TM / 32;
-    constexpr int MP = MR / 2, NP = NR / 2;
-    static_assert(MR % 2 == 0 && NR % 2 == 0, "scale chunks cover 32 rows");
-
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * TKB];
-
-    const int tid = threadIdx.x;
-    const int wave = wave_id();
-    const int lane = tid & 63;
-    const int li = lane & 15;
-    const int lg = lane >> 4;
-
-    const int tiles_m = (p.M + TM - 1) / TM;
-    const int tiles_n = (p.N + TN - 1) / TN;
-    int tm, tn;
-    tile_coords((int)blockIdx.x, tiles_m, tiles_n, p.group_m, tm, tn);
-    const int m0 = tm * TM;
-    const int n0 = tn * TN;
-    const int KP = p.K >> 1;   // packed bytes per row
-    const int KT = p.K >> 8;   // 256-K steps
-
-    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a + (uint64_t)m0 * KP, (uint64_t)(p.M - m0) * (uint64_t)KP);
-    const int nb0 = (n0 >> 4) + wave * NR;
-    const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)KP;
-    const uint64_t b_total = (uint64_t)p.N * (uint64_t)KP;
-    __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
-    // scales: 256 bytes per (32-row chunk, 256-K chunk)
-    const uint64_t chunk_bytes = (uint64_t)KT * 256ull;
-    const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5);
-    const uint64_t sa_first = (uint64_t)(m0 >> 5);
-    __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.sa + sa_first * chunk_bytes, (sa_chunks - sa_first) * chunk_bytes);
-    const uint64_t sb_chunks = (uint64_t)(p.N >> 5);
-    const uint64_t sb_first = (uint64_t)((n0 >> 5) + wave * NP);
-    __amdgpu_buffer_rsrc_t rsb = make_rsrc(p.sb + (sb_first < sb_chunks ? sb_first : sb_chunks) * chunk_bytes,
-                                           sb_first < sb_chunks ? (sb_chunks - sb_first) * chunk_bytes : 0);
-
-    const int a_row0 = tid >> 3;
-    const int a_kc = tid & 7;
-    const uint32_t a_goff0 = (uint32_t)a_row0 * (uint32_t)KP + (uint32_t)a_kc * 16u;
-
-    v4f acc[MR][NR];
-#pragma unroll
-    for (int mi = 0; mi < MR; mi++)
-#pragma unroll
-        for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    v4i areg[A_LOADS];
-    v4i bq[2][NR][2];
-    int sav[2][MP], sbv[2][NP];
-
-    // Loads never sit under control flow: a K step past the end (prefetch of the last iteration) is
-    // redirected past the descriptor bounds, where the hardware returns zero without touching memory.
-    auto load_a = [&](int kt) {
-        const bool valid = kt < KT;
-#pragma unroll
-        for (int j = 0; j < A_LOADS; j++) {
-            const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)KP + (uint32_t)kt * TKB;
-            areg[j] = buf_load16(ra, valid ? off : 0xFFFFFFF0u, 0);
-        }
-    };
-    auto store_a = [&](int stage) {
-#pragma unroll
-        for (int j = 0; j < A_LOADS; j++)
-            *reinterpret_cast<v4i*>(&lds[stage][lds_off(a_row0 + 32 * j, a_kc)]) = areg[j];
-    };
-    auto load_b = [&](int kt, auto ST) {
-        constexpr int st = decltype(ST)::value;
-        const bool valid = kt < KT;
-        const uint32_t koff = valid ? (uint32_t)kt * 2048u : 0u;
-        const uint32_t soff = valid ? (uint32_t)kt * 256u : 0u;
-#pragma unroll
-        for (int ni = 0; ni < NR; ni++) {
-            const uint32_t voff = valid ? (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)KP : 0xFFFFFFF0u;
-            bq[st][ni][0] = buf_load16(rb, voff, koff);
-            bq[st][ni][1] = buf_load16(rb, voff, valid ? koff + 1024u : 0u);
-        }
-#pragma unroll
-        for (int mp = 0; mp < MP; mp++)
-            sav[st][mp] = buf_load4(rsa, valid ? (uint32_t)mp * (uint32_t)chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
-#pragma unroll
-        for (int np = 0; np < NP; np++)
-            sbv[st][np] = buf_load4(rsb, valid ? (uint32_t)np * (uint32_t)chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
-    };
-    // A fragments (m-block, 128-K half) are read one step ahead of the MFMAs that use them
-    auto compute = [&](auto ST) {
-        constexpr int st = decltype(ST)::value;
-        v4i af[2];
-        af[0] = *reinterpret_cast<const v4i*>(&lds[st][lds_off(li, lg)]);
-        static_for<MR * 2>([&](auto IDX) {
-            constexpr int idx = decltype(IDX)::value;
-            constexpr int mi = idx / 2, kh = idx % 2;
-            if constexpr (idx + 1 < MR * 2) {
-                constexpr int mi1 = (idx + 1) / 2, kh1 = (idx + 1) % 2;
-                af[(idx + 1) & 1] = *reinterpret_cast<const v4i*>(&lds[st][lds_off(mi1 * 16 + li, kh1 * 4 + lg)]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            static_for<NR>([&](auto NI) {
-                constexpr int ni = decltype(NI)::value;
-                acc[mi][ni] = mx_mfma<kh * 2 + (ni & 1), kh * 2 + (mi & 1)>(bq[st][ni][kh], af[idx & 1], acc[mi][ni],
-                                                                               sbv[st][ni / 2], sav[st][mi / 2]);
-            });
-            __builtin_amdgcn_sched_barrier(0);
-        });
-    };
-
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
-    load_a(0);
-    load_b(0, S0{});
-    store_a(0);
-    __syncthreads();
-
-    // two K steps per iteration (ping-pong); an odd step count ends with one step on zero operands
-    for (int kt = 0; kt < KT; kt += 2) {
-        load_a(kt + 1);
-        load_b(kt + 1, S1{});
-        compute(S0{});
-        store_a(1);
-        __syncthreads();
-
-        load_a(kt + 2);
-        load_b(kt + 2, S0{});
-        compute(S1{});
-        store_a(0);
-        __syncthreads();
-    }
-
-    static_for<MR>([&](auto MI) {
-        constexpr int mi = decltype(MI)::value;
-        const int m = m0 + mi * 16 + li;
-        if (m < p.M) {
-            static_for<NR>([&](auto NI) {
-                constexpr int ni = decltype(NI)::value;
-                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-                if (n < p.N) store_mx4(p, STORE, (size_t)m * (size_t)p.N + (size_t)n, acc[mi][ni]);
-            });
-        }
-    });
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -300,14 +137,6 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
     }
 }
 
-template <int MR, int NR, int STORE>
-hipError_t launch_tiled(const MxParams& p, hipStream_t stream) {
-    constexpr int TM = 16 * MR, TN = 64 * NR;
-    const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
-    hipLaunchKernelGGL((k_mxfp4_tiled<MR, NR, STORE>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, p);
-    return hipGetLastError();
-}
-
 template <int MB, int STORE>
 hipError_t launch_smallm(const MxParams& p, hipStream_t stream) {
     const int npw = NW / p.ksplit;
@@ -317,21 +146,6 @@ hipError_t launch_smallm(const MxParams& p, hipStream_t stream) {
 }
 
 }  // namespace
-
-// tile_m x tile_n in {256x256, 128x256, 64x256, 32x256, 64x128, 32x128}
-hipError_t psg_launch_mxfp4_tiled(const MxParams& p, int store, int tile_m, int tile_n, hipStream_t stream) {
-#define PSG_CASE(MR_, NR_)                                                                         \
-    if (tile_m == 16 * MR_ && tile_n == 64 * NR_)                                                  \
-        return store == STORE_ACC ? launch_tiled<MR_, NR_, STORE_ACC>(p, stream) : launch_tiled<MR_, NR_, STORE_C>(p, stream);
-    PSG_CASE(16, 4)
-    PSG_CASE(8, 4)
-    PSG_CASE(4, 4)
-    PSG_CASE(2, 4)
-    PSG_CASE(4, 2)
-    PSG_CASE(2, 2)
-#undef PSG_CASE
-    return hipErrorInvalidConfiguration;
-}
 
 // requires 1 <= M <= 32 and p.ksplit in {1,2,4,8}
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream) {

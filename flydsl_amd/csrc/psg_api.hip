@@ -10,7 +10,6 @@
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream);
-hipError_t psg_launch_mxfp4_tiled(const MxParams& p, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
 
 namespace {
@@ -56,7 +55,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     };
     static const Shape shapes8[] = {{128, 256, 2, 1.00}, {256, 256, 1, 0.95}, {64, 256, 2, 0.62}, {32, 256, 3, 0.36},
                                     {128, 128, 2, 0.70}, {64, 64, 5, 0.25}};
-    static const Shape shapesx[] = {{128, 256, 2, 1.00}, {256, 256, 1, 0.95}, {64, 256, 2, 0.62}, {32, 256, 3, 0.36},
+    static const Shape shapesx[] = {{256, 256, 1, 1.00}, {128, 256, 2, 0.86}, {64, 256, 2, 0.80}, {32, 256, 3, 0.40},
                                     {64, 128, 3, 0.40}, {32, 128, 4, 0.25}};
     const Shape* shapes = mx ? shapesx : shapes8;
     for (int i = 0; i < 6; i++)
@@ -116,7 +115,7 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
 }
 
 int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
-    A8W8Params p;
+    A8W8Params p{};
     p.c = out;
     p.a = static_cast<const uint8_t*>(a->a);
     p.b = static_cast<const uint8_t*>(a->b);
@@ -128,7 +127,9 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     p.K = a->K;
     p.epi = a->epilogue;
     p.out = a->out_dtype;
-    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 4;
+    // M-tiles per group of the XCD-aware tile order: 8 makes the set of tiles one XCD works on at a time roughly
+    // square in bytes (A rows vs W rows), which minimises what its L2 has to fetch
+    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;
     const int kind = a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : KIND_FP8;
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
@@ -195,7 +196,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     p.N = a->N;
     p.K = a->K;
     p.out = a->out_dtype;
-    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 4;
+    p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
     if (small) {
@@ -203,8 +204,20 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         e = psg_launch_mxfp4_smallm(p, store, static_cast<hipStream_t>(stream));
     } else {
         const Tile t = pick_tile(a->M, a->N, true, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
-        p.ksplit = 1;
-        e = psg_launch_mxfp4_tiled(p, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        A8W8Params q{};
+        q.c = p.c;
+        q.a = p.a;
+        q.b = p.b;
+        q.mx_sa = p.sa;
+        q.mx_sb = p.sb;
+        q.M = p.M;
+        q.N = p.N;
+        q.K = p.K;
+        q.group_m = p.group_m;
+        q.ksplit = 1;
+        q.epi = EPI_NONE;
+        q.out = p.out;
+        e = psg_launch_a8w8_tiled(q, KIND_MXFP4, store, t.m, t.n, static_cast<hipStream_t>(stream));
     }
     if (e != hipSuccess) return hip_fail(e, "psg_gemm_mxfp4 launch");
     g_err[0] = 0;

@@ -12,7 +12,7 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3 };
+enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3, KIND_MXFP4 = 4 };
 enum { OUT_BF16 = 0, OUT_FP16 = 1 };
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_RELU = 2, EPI_BIAS_SILU = 3, EPI_BIAS_GELU = 4 };
 // what a kernel writes: the scaled/activated C, or the raw accumulators
@@ -108,6 +108,8 @@ struct A8W8Params {
     int ksplit;   // K splits per n-block (small-M kernel)
     int epi;      // EPI_*
     int out;      // OUT_*
+    const uint8_t* mx_sa;  // MXFP4 only: shuffled e8m0 [ceil(M/32)*32, K/32]
+    const uint8_t* mx_sb;  // MXFP4 only: shuffled e8m0 [N, K/32]
 };
 
 struct MxParams {
