@@ -105,6 +105,9 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                 const uint32_t kbyte = kbase + (uint32_t)st_c * 16u;
                 tmp[ps] = buf_load16(ra, kbyte < slice_end ? (uint32_t)r * (uint32_t)K + kbyte : 0xFFFFFFF0u, 0);
             }
+            // (the fences keep the machine scheduler from sinking loads below their first use to save registers,
+            // which would serialise two memory latencies)
+            __builtin_amdgcn_sched_barrier(0);
             // 2. the W blocks of this chunk, all in flight at once
             v4i blo[NB][SPS], bhi[NB][SPS];
 #pragma unroll
@@ -119,6 +122,7 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                     blo[nb][u] = buf_load16_nt(rb, has_lo ? voff : 0xFFFFFFF0u, boff);
                     bhi[nb][u] = buf_load16_nt(rb, has_hi ? voff : 0xFFFFFFF0u, has_hi ? boff + 1024u : 0u);
                 }
+            __builtin_amdgcn_sched_barrier(0);
             // 3. A through the private LDS patch into fragment order while W is still on its way
 #pragma unroll
             for (int ps = 0; ps < 8; ps++) {

@@ -73,7 +73,7 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
 template <int KIND, int MR, int NR, int STORE>
-__global__ void __launch_bounds__(256, (MR <= 8 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
+__global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr int TM = 16 * MR;
     constexpr int TN = 64 * NR;
@@ -332,6 +332,7 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
 #define PSG_CASE(MR_, NR_) \
     if (tile_m == 16 * MR_ && tile_n == 64 * NR_) return launch_one<KIND, MR_, NR_, STORE>(p, stream);
     PSG_CASE(16, 4)
+    PSG_CASE(8, 8)
     PSG_CASE(8, 4)
     PSG_CASE(4, 4)
     PSG_CASE(2, 4)

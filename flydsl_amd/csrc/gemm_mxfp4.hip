@@ -100,6 +100,8 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
                     sbv[u] = buf_load4(rsb, (uint32_t)lane * 4u, (uint32_t)s * 256u);
                 }
             }
+            // keep every load of the chunk ahead of the first MFMA (the scheduler would otherwise sink some)
+            __builtin_amdgcn_sched_barrier(0);
             static_for<UNROLL>([&](auto U) {
                 constexpr int u = decltype(U)::value;
                 static_for<2>([&](auto KH) {

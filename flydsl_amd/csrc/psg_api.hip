@@ -58,8 +58,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     static const Shape shapesx[] = {{256, 256, 1, 1.00}, {128, 256, 2, 0.86}, {64, 256, 2, 0.80}, {32, 256, 3, 0.40},
                                     {64, 128, 3, 0.40}, {32, 128, 4, 0.25}};
     const Shape* shapes = mx ? shapesx : shapes8;
-    for (int i = 0; i < 6; i++)
-        if (shapes[i].m == hint_m && shapes[i].n == hint_n) return {hint_m, hint_n};
+    if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n};  // forced by the caller; the launcher rejects unknown shapes
     double best = -1.0;
     Tile t = {shapes[0].m, shapes[0].n};
     for (int i = 0; i < 6; i++) {
