@@ -65,23 +65,28 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) acc[nb][mb] = (acc_t){0, 0, 0, 0};
 
-    // The scales of the outputs this thread will finish are fetched now, so that their latency does not sit
-    // behind the reduction barrier at the very end of the kernel.  Finishing work item t = tid (+ NW*64):
-    // (n-block t/(MB*64) of the workgroup, m-block, lane).
+    // The scales of the outputs this thread will finish are fetched early (right behind the first chunk's loads),
+    // so that their latency does not sit behind the reduction barrier at the very end of the kernel.  Finishing
+    // work item t = tid (+ NW*64): (n-block t/(MB*64) of the workgroup, m-block, lane).
     constexpr int FIN = (NB * MB * NW * 64 + NW * 64 - 1) / (NW * 64);  // items per thread at ksplit 1
     float fin_sa[FIN];
     v4f fin_sb[FIN];
-    if constexpr (STORE != STORE_ACC) {
+    auto fetch_scales = [&]() {
+        if constexpr (STORE != STORE_ACC) {
 #pragma unroll
-        for (int f = 0; f < FIN; f++) {
-            const int t = tid + f * NW * 64;
-            const int nbq = (int)blockIdx.x * nbw * NB + t / (MB * 64);
-            const int m = ((t / 64) % MB) * 16 + li;
-            const bool live = t < nbw * NB * MB * 64 && nbq < n_blocks && m < p.M;
-            fin_sa[f] = live ? p.sa[m] : 0.f;
-            fin_sb[f] = live ? *reinterpret_cast<const v4f*>(p.sb + nbq * 16 + lg * 4) : (v4f){0.f, 0.f, 0.f, 0.f};
+            for (int f = 0; f < FIN; f++) {
+                const int t = tid + f * NW * 64;
+                const int nbq = (int)blockIdx.x * nbw * NB + t / (MB * 64);
+                const int m = ((t / 64) % MB) * 16 + li;
+                const bool live = t < nbw * NB * MB * 64 && nbq < n_blocks && m < p.M;
+                // clamp the ADDRESS for dead items instead of selecting the loaded value (a select would force
+                // a wait for these cold loads right here)
+                fin_sa[f] = p.sa[live ? m : 0];
+                fin_sb[f] = *reinterpret_cast<const v4f*>(p.sb + (live ? nbq * 16 + lg * 4 : 0));
+            }
         }
-    }
+    };
+    bool scales_fetched = false;
 
     if (my_nb < n_blocks) {
         // this wavefront's NB n-blocks; a block past N/16 (odd block count) reads as zero
@@ -122,6 +127,10 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                     blo[nb][u] = buf_load16_nt(rb, has_lo ? voff : 0xFFFFFFF0u, boff);
                     bhi[nb][u] = buf_load16_nt(rb, has_hi ? voff : 0xFFFFFFF0u, has_hi ? boff + 1024u : 0u);
                 }
+            if (!scales_fetched) {  // first chunk only (wave-uniform)
+                fetch_scales();
+                scales_fetched = true;
+            }
             __builtin_amdgcn_sched_barrier(0);
             // 3. A through the private LDS patch into fragment order while W is still on its way
 #pragma unroll
@@ -158,6 +167,8 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                     }
         }
     }
+
+    if (!scales_fetched) fetch_scales();  // wavefronts without an n-block still finish outputs
 
     // split-K reduction through LDS, fixed order
 #pragma unroll
