@@ -33,22 +33,25 @@ WORKLOADS = {
     "mxfp4_m32": ("mxfp4", "fp4", 32, 7168, 2048, "hbm"),
     "mxfp4_m4096": ("mxfp4", "fp4", 4096, 7168, 2048, "mfma"),
     "int8_plumbing_m128": ("a8w8", "int8", 128, 1024, 1024, "mfma"),
+    "bf16_m5120": ("a16w16", "bf16", 5120, 5120, 8320, "mfma"),
 }
 DEFAULT_WORKLOAD = "fp8_decode_m16"
-PEAK = {"hbm": 8000.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0}  # GB/s, TFLOP/s (dense, published)
+PEAK = {"hbm": 8000.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0, "bf16": 2500.0, "fp16": 2500.0}  # GB/s, TFLOP/s (dense, published)
 MALL_BYTES = 256 << 20
 
 
 def algorithmic_bytes(family, M, N, K):
     if family == "a8w8":
         return M * K + N * K + 2 * M * N + 4 * (M + N)
+    if family == "a16w16":
+        return 2 * M * K + 2 * N * K + 2 * M * N
     return M * K // 2 + N * K // 2 + 2 * M * N + (M + N) * (K // 32)
 
 
 def make_launcher(family, kind, M, N, K):
     import torch
 
-    if family == "a8w8":
+    if family in ("a8w8", "a16w16"):
         from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
         fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=64, in_dtype=kind)
@@ -77,12 +80,20 @@ def run_workload(name, steps, warmup, check=True):
     n_sets = max(2, min(32, math.ceil(2 * MALL_BYTES / nbytes)))
     if nbytes * n_sets > (8 << 30):
         n_sets = max(2, (8 << 30) // nbytes)
-    from flydsl_amd.synthetic import make_a8w8, make_mxfp4
+    from flydsl_amd.synthetic import make_a8w8, make_a16w16, make_mxfp4
 
-    host = make_a8w8(M, N, K, kind, seed=0) if family == "a8w8" else make_mxfp4(M, N, K, seed=0)
+    if family == "a8w8":
+        host = make_a8w8(M, N, K, kind, seed=0)
+    elif family == "a16w16":
+        host = make_a16w16(M, N, K, kind, seed=0, w_std=0.02)
+    else:
+        host = make_mxfp4(M, N, K, seed=0)
     sets = []
     for i in range(n_sets):
-        if family == "a8w8":
+        if family == "a16w16":
+            none = torch.empty(0, dtype=torch.float32, device=dev)
+            s = {"a": host["a_q"].to(dev), "b": host["b_shuf"].to(dev), "sa": none, "sb": none}
+        elif family == "a8w8":
             s = {"a": host["a_q"].to(dev), "b": host["b_shuf"].to(dev), "sa": host["sa"].to(dev), "sb": host["sb"].to(dev)}
         else:
             s = {"a": host["a_q"].to(dev), "b": host["b_shuf"].to(dev), "sa": host["sa_shuf"].to(dev), "sb": host["sb_shuf"].to(dev)}
@@ -140,7 +151,10 @@ def run_workload(name, steps, warmup, check=True):
 
         out = sets[(steps - 1) % n_sets]["c"].float().cpu().numpy()
         rows = np.arange(M) if M <= 256 else np.array(sorted({(i * 131 + 7) % M for i in range(64)}))
-        if family == "a8w8":
+        if family == "a16w16":
+            ref = O.run_torch(host["a_q"].view(torch.int16).numpy().view(np.uint16)[rows],
+                              host["b_q"].view(torch.int16).numpy().view(np.uint16), None, None, kind)
+        elif family == "a8w8":
             ref = O.run_torch(host["a_q"].view(torch.uint8).numpy()[rows], host["b_q"].view(torch.uint8).numpy(),
                               host["sa"].numpy()[rows], host["sb"].numpy(), kind)
         else:
@@ -261,7 +275,7 @@ def main():
     others = []
     if not args.no_others:
         for name in ("fp8_decode_m1", "fp8_decode_m16", "fp8_decode_m32", "fp8_prefill_m8192", "int8_ffn_m4096", "mxfp4_m32",
-                     "mxfp4_m4096"):
+                     "mxfp4_m4096", "bf16_m5120"):
             if name == args.workload:
                 continue
             b = WORKLOADS[name][5]
@@ -280,7 +294,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"fp8": "fp8_e4m3fn", "int8": "int8", "fp4": "mxfp4_e2m1"}[kind],
+        "dtype": {"fp8": "fp8_e4m3fn", "int8": "int8", "fp4": "mxfp4_e2m1", "bf16": "bf16", "fp16": "fp16"}[kind],
         "data": "synthetic (seed 0; A~N(0,1) per-token quantised, W~N(0,0.02) per-channel quantised and preshuffled; "
                 f"{main_res['operand_sets']} rotating operand sets)",
         "config": {"workload": f"{args.workload}: {kind} W8A8 preshuffle GEMM M={M} N={N} K={K}, bf16 out", "M": M, "N": N, "K": K,

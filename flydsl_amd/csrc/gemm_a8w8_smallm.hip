@@ -48,7 +48,8 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     const int lane = tid & 63;
     const int li = lane & 15;
     const int lg = lane >> 4;
-    const int K = p.K;
+    constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
+    const int K = IS16 ? (p.K << 1) : p.K;   // BYTES per operand row from here on
     const int ks = p.ksplit;           // 1, 2, 4 or 8
     const int nbw = NW / ks;           // wavefront groups (K-slice sets) per workgroup, NB n-blocks each
     const int my_ks = wave % ks;
@@ -72,7 +73,7 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     float fin_sa[FIN];
     v4f fin_sb[FIN];
     auto fetch_scales = [&]() {
-        if constexpr (STORE != STORE_ACC) {
+        if constexpr (STORE != STORE_ACC && !IS16) {
 #pragma unroll
             for (int f = 0; f < FIN; f++) {
                 const int t = tid + f * NW * 64;
@@ -157,6 +158,12 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                         if constexpr (KIND == KIND_INT8) {
                             acc[nb][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[nb][t], alo[t][mb], acc[nb][mb], 0, 0, 0);
                             acc[nb][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[nb][t], ahi[t][mb], acc[nb][mb], 0, 0, 0);
+                        } else if constexpr (KIND == KIND_BF16) {
+                            acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, blo[nb][t]), __builtin_bit_cast(v8bf, alo[t][mb]), acc[nb][mb], 0, 0, 0);
+                            acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bhi[nb][t]), __builtin_bit_cast(v8bf, ahi[t][mb]), acc[nb][mb], 0, 0, 0);
+                        } else if constexpr (KIND == KIND_FP16) {
+                            acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, blo[nb][t]), __builtin_bit_cast(v8h, alo[t][mb]), acc[nb][mb], 0, 0, 0);
+                            acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, bhi[nb][t]), __builtin_bit_cast(v8h, ahi[t][mb]), acc[nb][mb], 0, 0, 0);
                         } else {
                             const v8i bf = {blo[nb][t][0], blo[nb][t][1], blo[nb][t][2], blo[nb][t][3],
                                             bhi[nb][t][0], bhi[nb][t][1], bhi[nb][t][2], bhi[nb][t][3]};
@@ -194,10 +201,15 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
                 if constexpr (STORE == STORE_ACC) {
                     *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = sum;
                 } else {
-                    const float sa = fin_sa[f];
-                    const v4f sb = fin_sb[f];
-                    const v4f x = {((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
-                                   ((float)sum[3] * sa) * sb[3]};
+                    v4f x;
+                    if constexpr (IS16) {
+                        x = (v4f){(float)sum[0], (float)sum[1], (float)sum[2], (float)sum[3]};
+                    } else {
+                        const float sa = fin_sa[f];
+                        const v4f sb = fin_sb[f];
+                        x = (v4f){((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
+                                  ((float)sum[3] * sa) * sb[3]};
+                    }
                     store_c4(p, idx, n, x);
                 }
             }
@@ -229,5 +241,9 @@ hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int 
         return store == STORE_ACC ? launch_kind<KIND_INT8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_INT8, STORE_C>(p, nb, stream);
     if (kind == KIND_FP8)
         return store == STORE_ACC ? launch_kind<KIND_FP8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_FP8, STORE_C>(p, nb, stream);
+    if (kind == KIND_BF16)
+        return store == STORE_ACC ? launch_kind<KIND_BF16, STORE_ACC>(p, nb, stream) : launch_kind<KIND_BF16, STORE_C>(p, nb, stream);
+    if (kind == KIND_FP16)
+        return store == STORE_ACC ? launch_kind<KIND_FP16, STORE_ACC>(p, nb, stream) : launch_kind<KIND_FP16, STORE_C>(p, nb, stream);
     return hipErrorInvalidValue;
 }

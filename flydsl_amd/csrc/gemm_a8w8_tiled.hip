@@ -1,4 +1,4 @@
-// Compute-bound mainloop of the preshuffle GEMM for gfx950: int8, OCP fp8 and MXFP4 operands.
+// Compute-bound mainloop of the preshuffle GEMM for gfx950: int8, OCP fp8, MXFP4 and fp16/bf16 operands.
 //
 //   C[M,N] = A[M,K] * W[N,K]^T, W preshuffled into 1 KB fragment blocks [N/16][K/64][klane 4][nlane 16][16 B].
 //
@@ -13,6 +13,8 @@
 //             bytes [16g,16g+16) and [64+16g, 64+16g+16) of the 128-byte K step (g = lane/16) so that
 //             each half is exactly one preshuffled block; A uses the same K order.
 //       int8: two v_mfma_i32_16x16x64_i8 per K step (one per 64-byte half), int32 accumulate (exact).
+//       fp16/bf16: 2-byte elements are preshuffled as [N/16][K/32][4][16][8 elements], i.e. again 1 KB blocks of
+//             16 rows x 64 bytes; two v_mfma_f32_16x16x32_{f16,bf16} per 128-byte K step (64 elements), no scales.
 //       mxfp4: K is packed two elements per byte, so a 128-byte K step is 256 elements = one chunk of the
 //             shuffled e8m0 scale layout; two v_mfma_scale_f32_16x16x128_f8f6f4 per step (one per 64-byte
 //             half = one preshuffled block), each lane's 16 bytes are 32 consecutive K elements sharing one
@@ -44,6 +46,12 @@ __device__ __forceinline__ void mfma_f8(v4f& c, const v8i& a, const v8i& b) {
 }
 __device__ __forceinline__ void mfma_i8(v4i& c, const v4i& a, const v4i& b) {
     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_bf16(v4f& c, const v4i& a, const v4i& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_f16(v4f& c, const v4i& a, const v4i& b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 // fp4 x fp4 with per-lane e8m0 scales: scale byte of src0 = 2*HI + LO0 of dword s0, of src1 = 2*HI + LO1 of s1
 template <int HI, int LO0, int LO1>
@@ -94,7 +102,9 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     const int m0 = tm * TM;
     const int n0 = tn * TN;
     // K counts BYTES of one operand row from here on (two fp4 elements per byte)
-    const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : p.K;
+    constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
+    constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;  // per-token x per-channel fp32 scales in the epilogue
+    const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : (IS16 ? (p.K << 1) : p.K);
     const int KT = (K + TK - 1) / TK;
 
     // A: this tile's rows; rows >= M read as zero through the descriptor bound
@@ -215,6 +225,15 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
                 for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[S][ni], alo);
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[S][ni], ahi);
+            } else if constexpr (IS16) {
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], blo[S][ni], alo); else mfma_f16(acc[mi][ni], blo[S][ni], alo);
+                }
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], bhi[S][ni], ahi); else mfma_f16(acc[mi][ni], bhi[S][ni], ahi);
+                }
             } else if constexpr (KIND == KIND_MXFP4) {
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
@@ -269,7 +288,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     // epilogue operands, fetched in one batch (one memory latency for the whole tile, not one per fragment)
     float sa_v[MR];
     v4f sb_v[NR];
-    if constexpr (STORE != STORE_ACC && KIND != KIND_MXFP4) {
+    if constexpr (STORE != STORE_ACC && SCALED) {
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) {
             const int m = m0 + mi * 16 + li;
@@ -289,7 +308,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
         const int m = m0 + mi * 16 + li;
         if (m < p.M) {
             float sa = 0.f;
-            if constexpr (STORE != STORE_ACC && KIND != KIND_MXFP4) sa = sa_v[mi];
+            if constexpr (STORE != STORE_ACC && SCALED) sa = sa_v[mi];
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
                 const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
@@ -300,8 +319,8 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
                         *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = r;
                     } else {
                         v4f x;
-                        if constexpr (KIND == KIND_MXFP4) {
-                            x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};  // scales were applied by the MFMA
+                        if constexpr (!SCALED) {
+                            x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};  // no epilogue scales (MX: applied by the MFMA)
                         } else {
                             const v4f sb = sb_v[ni];
                             x = (v4f){((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2],
@@ -349,7 +368,7 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
 
 }  // namespace
 
-// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8 / KIND_MXFP4.  tile_m x tile_n must be one of the
+// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8 / KIND_FP16 / KIND_BF16 / KIND_MXFP4.  tile_m x tile_n must be one of the
 // instantiated shapes: 256x256, 128x256, 64x256, 32x256, then 128x128 and 64x64 (8-bit) or 64x128 and 32x128 (MXFP4).
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
     if (store == STORE_C && (p.epi != EPI_NONE || p.out != OUT_BF16)) store = STORE_C_GENERIC;
@@ -362,6 +381,16 @@ hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int t
         if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);
         if (store == STORE_C_GENERIC) return launch_shape<KIND_FP8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
         return launch_shape<KIND_FP8, STORE_C>(p, tile_m, tile_n, stream);
+    }
+    if (kind == KIND_BF16) {
+        if (store == STORE_ACC) return launch_shape<KIND_BF16, STORE_ACC>(p, tile_m, tile_n, stream);
+        if (store == STORE_C_GENERIC) return launch_shape<KIND_BF16, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
+        return launch_shape<KIND_BF16, STORE_C>(p, tile_m, tile_n, stream);
+    }
+    if (kind == KIND_FP16) {
+        if (store == STORE_ACC) return launch_shape<KIND_FP16, STORE_ACC>(p, tile_m, tile_n, stream);
+        if (store == STORE_C_GENERIC) return launch_shape<KIND_FP16, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
+        return launch_shape<KIND_FP16, STORE_C>(p, tile_m, tile_n, stream);
     }
     if (kind == KIND_MXFP4) {
         if (store == STORE_ACC) return launch_shape<KIND_MXFP4, STORE_ACC>(p, tile_m, tile_n, stream);

@@ -83,29 +83,29 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
 int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
     if (!a) return fail(PSG_E_NULL, "args is NULL");
     if (!a->a || !a->b) return fail(PSG_E_NULL, "a and b must be non-NULL");
+    const bool is16 = a->in_dtype == PSG_IN_FP16 || a->in_dtype == PSG_IN_BF16;
+    const int64_t eb = is16 ? 2 : 1;
     if (acc_only) {
         if (!acc) return fail(PSG_E_NULL, "acc must be non-NULL");
     } else {
         if (!a->c) return fail(PSG_E_NULL, "c must be non-NULL");
-        if (!a->scale_a || !a->scale_b) return fail(PSG_E_NULL, "scale_a and scale_b must be non-NULL for 8-bit inputs");
+        if (!is16 && (!a->scale_a || !a->scale_b)) return fail(PSG_E_NULL, "scale_a and scale_b must be non-NULL for 8-bit inputs");
         if (a->epilogue != PSG_EPI_NONE && !a->bias) return fail(PSG_E_NULL, "bias must be non-NULL when epilogue != none");
     }
-    if (a->in_dtype == PSG_IN_FP16 || a->in_dtype == PSG_IN_BF16)
-        return fail(PSG_E_UNSUPPORTED, "fp16/bf16 inputs are not built in this library yet");
-    if (a->in_dtype != PSG_IN_INT8 && a->in_dtype != PSG_IN_FP8_E4M3FN) return fail(PSG_E_DTYPE, "in_dtype %d unknown", a->in_dtype);
+    if (a->in_dtype < PSG_IN_INT8 || a->in_dtype > PSG_IN_BF16) return fail(PSG_E_DTYPE, "in_dtype %d unknown", a->in_dtype);
     if (a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
     if (a->epilogue < PSG_EPI_NONE || a->epilogue > PSG_EPI_BIAS_GELU) return fail(PSG_E_DTYPE, "epilogue %d unknown", a->epilogue);
     if (a->M < 1 || a->M > 65536) return fail(PSG_E_SHAPE, "M=%d outside [1, 65536]", a->M);
     if (a->N < 16 || a->N % 16) return fail(PSG_E_SHAPE, "N=%d must be a positive multiple of 16", a->N);
-    if (a->K < 64 || a->K % 64) return fail(PSG_E_SHAPE, "K=%d must be a positive multiple of 64", a->K);
-    if ((uint64_t)a->N * (uint64_t)a->K > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "N*K=%llu exceeds the 4 GiB descriptor range", (unsigned long long)a->N * a->K);
+    if (a->K < 64 / eb || (a->K * eb) % 64) return fail(PSG_E_SHAPE, "K=%d must be a positive multiple of %d", a->K, (int)(64 / eb));
+    if ((uint64_t)a->N * (uint64_t)a->K * (uint64_t)eb > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "N*K bytes exceed the 4 GiB descriptor range");
     if (!aligned(a->a, 16) || !aligned(a->b, 16)) return fail(PSG_E_ALIGN, "a and b must be 16-byte aligned");
     if (acc_only) {
         if (!aligned(acc, 16)) return fail(PSG_E_ALIGN, "acc must be 16-byte aligned");
     } else {
         if (!aligned(a->c, 8)) return fail(PSG_E_ALIGN, "c must be 8-byte aligned");
-        if (!aligned(a->scale_b, 16)) return fail(PSG_E_ALIGN, "scale_b must be 16-byte aligned");
-        if (!aligned(a->scale_a, 4)) return fail(PSG_E_ALIGN, "scale_a must be 4-byte aligned");
+        if (!is16 && !aligned(a->scale_b, 16)) return fail(PSG_E_ALIGN, "scale_b must be 16-byte aligned");
+        if (!is16 && !aligned(a->scale_a, 4)) return fail(PSG_E_ALIGN, "scale_a must be 4-byte aligned");
         if (a->epilogue != PSG_EPI_NONE && !aligned(a->bias, 8)) return fail(PSG_E_ALIGN, "bias must be 8-byte aligned");
     }
     if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
@@ -129,13 +129,15 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     // M-tiles per group of the XCD-aware tile order: 8 makes the set of tiles one XCD works on at a time roughly
     // square in bytes (A rows vs W rows), which minimises what its L2 has to fetch
     p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;
-    const int kind = a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : KIND_FP8;
+    const int kinds[4] = {KIND_INT8, KIND_FP8, KIND_FP16, KIND_BF16};
+    const int kind = kinds[a->in_dtype];
+    const int kbytes = (kind == KIND_FP16 || kind == KIND_BF16) ? a->K * 2 : a->K;
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
     if (small) {
         // two n-blocks per wavefront halve the A traffic per byte of W; keep one when that would leave too few
         // wavefronts to cover the memory latency
-        const int steps = (a->K + 127) / 128;
+        const int steps = (kbytes + 127) / 128;
         const int nb = (a->N / 16) >= 256 ? 2 : 1;
         p.ksplit = pick_ksplit((a->N / 16 + nb - 1) / nb, steps);
         e = psg_launch_a8w8_smallm(p, kind, store, nb, static_cast<hipStream_t>(stream));

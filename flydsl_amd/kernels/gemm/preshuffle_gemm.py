@@ -1,4 +1,4 @@
-"""Preshuffle GEMM entry point (int8 / OCP fp8 per-token x per-channel scaled, bf16/fp16 out).
+"""Preshuffle GEMM entry point (int8 / OCP fp8 per-token x per-channel scaled, or fp16 / bf16 unscaled; bf16/fp16 out).
 
 Drop-in for the reference's ``compile_preshuffle_gemm`` (kernels/gemm/preshuffle_gemm.py:108-128):
 same keyword-only signature and defaults, same ``ValueError`` conditions, and the returned callable
@@ -142,6 +142,4 @@ def compile_preshuffle_gemm(
     ``fn(C, A, B, scale_a, scale_b, bias, M, N, stream)``; ``bias`` is per-N in ``out_dtype`` and is
     only read when ``epilogue != "none"``."""
     _validate(N, K, tile_m, tile_n, tile_k, in_dtype, out_dtype, epilogue, use_async_copy, lds_stage, preload)
-    if in_dtype in ("fp16", "bf16"):
-        raise NotImplementedError(f"in_dtype={in_dtype!r}: 16-bit inputs are not built in this library yet")
     return PreshuffleGemm(N, K, in_dtype, out_dtype, epilogue, tile_m, tile_n, tile_k, xcd_swizzle)

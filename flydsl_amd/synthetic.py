@@ -64,3 +64,12 @@ def make_mxfp4(M, N, K, seed=0, w_std=0.02):
         "sa_shuf": layout.shuffle_scale_w4(sa, 1, False).contiguous(),
         "sb_shuf": layout.shuffle_scale_w4(sb, 1, False).contiguous(),
     }
+
+
+def make_a16w16(M, N, K, kind, seed=0, w_std=1.0):
+    """fp16 / bf16 operands (no quantisation, no scales), W preshuffled with the 2-byte layout."""
+    g = gen(seed)
+    dt = torch.float16 if kind == "fp16" else torch.bfloat16
+    a = torch.randn(M, K, generator=g, dtype=torch.float32).to(dt)
+    w = (torch.randn(N, K, generator=g, dtype=torch.float32) * w_std).to(dt)
+    return {"kind": kind, "a_q": a.contiguous(), "b_q": w.contiguous(), "b_shuf": layout.shuffle_weight(w.contiguous(), layout=(16, 16)).contiguous()}

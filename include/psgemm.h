@@ -60,12 +60,13 @@ enum psg_error {
 /*
  * Arguments of the 8-bit (and 16-bit) preshuffle GEMM.
  *   c        [M,N] row-major, out_dtype; rows >= M of the allocation are never written
- *   a        [M,K] row-major, 1 byte/element (int8 or e4m3fn); rows >= M are never read
+ *   a        [M,K] row-major, 1 byte/element (int8 or e4m3fn) or 2 bytes/element (fp16 / bf16); rows >= M are never read
  *   b        preshuffle of W[N,K]: byte of W[n,k] at
  *            (n/16)*16K + (k/64)*1024 + ((k%64)/16)*256 + (n%16)*16 + k%16      (tests/utils.py:76-96)
- *   scale_a  [M] fp32 per-token scales; scale_b [N] fp32 per-channel scales
+ *            (2-byte elements: element (n,k) at (n/16)*16K + (k/32)*512 + ((k%32)/8)*128 + (n%16)*8 + k%8, in elements)
+ *   scale_a  [M] fp32 per-token scales; scale_b [N] fp32 per-channel scales; ignored (may be NULL) for fp16 / bf16
  *   bias     [N] out_dtype, read only when epilogue != PSG_EPI_NONE
- *   N % 16 == 0, K % 64 == 0, 1 <= M <= 65536 (kernels/gemm/preshuffle_gemm.py:783-785)
+ *   N % 16 == 0, K*bytes_per_element % 64 == 0, 1 <= M <= 65536 (kernels/gemm/preshuffle_gemm.py:783-785)
  *   workspace / workspace_bytes: scratch for the small-M split-K path; may be NULL/0 when
  *            psg_workspace_bytes() returns 0 for the same (M,N,K,in_dtype).  Contents need no
  *            initialisation beyond being zero the first time the buffer is used; the kernels leave

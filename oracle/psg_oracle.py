@@ -298,7 +298,15 @@ def shuffle_scale_w4(scale: np.ndarray) -> np.ndarray:
 # ----------------------------------------------------------------------------------------------
 
 
+def f16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return np.asarray(b).view(np.float16).astype(np.float32)
+
+
 def _as_f32_operand(q: np.ndarray, kind: str) -> np.ndarray:
+    if kind == "bf16":
+        return bf16_bits_to_f32(np.asarray(q).view(np.uint16))
+    if kind == "fp16":
+        return f16_bits_to_f32(np.asarray(q).view(np.uint16))
     if kind == "int8":
         return np.asarray(q).view(np.int8).astype(np.float32)
     if kind == "fp8":
@@ -313,8 +321,11 @@ def run_torch(a_q, b_q, scale_a, scale_b, kind: str, bias=None) -> np.ndarray:
 
     Pinned by a float64 matmul of the same dequantised operands on small shapes.
     """
-    a32 = _as_f32_operand(a_q, kind) * np.asarray(scale_a, dtype=np.float32).reshape(-1, 1)
-    b32 = _as_f32_operand(b_q, kind) * np.asarray(scale_b, dtype=np.float32).reshape(-1, 1)
+    a32 = _as_f32_operand(a_q, kind)
+    b32 = _as_f32_operand(b_q, kind)
+    if scale_a is not None and scale_b is not None:  # fp16 / bf16 operands carry no scales (:108-109)
+        a32 = a32 * np.asarray(scale_a, dtype=np.float32).reshape(-1, 1)
+        b32 = b32 * np.asarray(scale_b, dtype=np.float32).reshape(-1, 1)
     c = a32 @ b32.T
     if bias is not None:
         c = c + np.asarray(bias, dtype=np.float32).reshape(1, -1)

@@ -77,14 +77,14 @@ def test_rejects_partial_a_tile(tile_m):
 
 @pytest.mark.parametrize("tile_m", [64, 96, 128, 160])
 def test_accepts_whole_a_tile(tile_m):
-    # the reference's case is bf16 with tile_k=64 (2 bytes/element); same byte count with 1-byte elements
+    compile_preshuffle_gemm(N=1024, K=2048, tile_m=tile_m, tile_n=256, tile_k=64, in_dtype="bf16", out_dtype="bf16")
     compile_preshuffle_gemm(N=1024, K=2048, tile_m=tile_m, tile_n=256, tile_k=128, in_dtype="int8", out_dtype="bf16")
 
 
 @pytest.mark.parametrize("bad", [(1,), (1, 2, 3), (-1, 0), (0, -1), 4])
 def test_preload_validation(bad):
     with pytest.raises((ValueError, TypeError)):
-        compile_preshuffle_gemm(N=1024, K=2048, tile_m=128, tile_n=256, tile_k=64, in_dtype="int8", out_dtype="bf16", preload=bad)
+        compile_preshuffle_gemm(N=1024, K=2048, tile_m=128, tile_n=256, tile_k=64, in_dtype="bf16", out_dtype="bf16", preload=bad)
 
 
 def test_other_validation_errors():
@@ -177,8 +177,8 @@ def test_validation_errors_come_back_as_codes_without_a_gpu():
     assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -3  # PSG_E_DTYPE
     args.in_dtype, args.a = 1, 0x1001
     assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -6  # PSG_E_ALIGN
-    args.a, args.in_dtype = 0x1000, 3
-    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -5  # PSG_E_UNSUPPORTED (bf16 inputs)
+    args.a, args.in_dtype, args.K = 0x1000, 3, 48
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -2  # bf16: K*2 must be a multiple of 64
     with pytest.raises(ValueError):
         _lib.check(-2, "x")
     with pytest.raises(RuntimeError):
