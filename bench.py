@@ -192,7 +192,10 @@ def cpu_baseline(name, host, budget_s=12.0):
     # bound the work: ~2*m*N*K flop at a conservative 50 GFLOP/s per 8 cores
     est = 2.0 * M * N * K / (6e9 * cores) + N * K / 2e8
     m_s = M if est <= budget_s else max(16, int(M * budget_s / est))
-    if family == "a8w8":
+    if family == "a16w16":
+        a, b = host["a_q"][:m_s], host["b_q"]
+        f = lambda: torch.mm(a.to(torch.float32), b.to(torch.float32).T)  # noqa: E731  (run_torch without scales)
+    elif family == "a8w8":
         a, b, sa, sb = host["a_q"][:m_s], host["b_q"], host["sa"][:m_s], host["sb"]
         f = lambda: O.run_torch_cpu(a, b, sa, sb)  # noqa: E731
     else:
