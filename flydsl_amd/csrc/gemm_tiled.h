@@ -21,6 +21,7 @@
 //             scale byte, selected from the lane's scale dword with op_sel (byte = 2*half + 16-row half).
 //   * Workgroup ids are remapped so that the ids the hardware deals to one XCD cover a compact
 //     group_m x tiles_n patch of tiles (A and B panels stay in that XCD's L2).
+#pragma once
 #include "psg_common.h"
 
 namespace {
@@ -367,35 +368,3 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
 }
 
 }  // namespace
-
-// Host entry used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8 / KIND_FP16 / KIND_BF16 / KIND_MXFP4.  tile_m x tile_n must be one of the
-// instantiated shapes: 256x256, 128x256, 64x256, 32x256, then 128x128 and 64x64 (8-bit) or 64x128 and 32x128 (MXFP4).
-hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
-    if (store == STORE_C && (p.epi != EPI_NONE || p.out != OUT_BF16)) store = STORE_C_GENERIC;
-    if (kind == KIND_INT8) {
-        if (store == STORE_ACC) return launch_shape<KIND_INT8, STORE_ACC>(p, tile_m, tile_n, stream);
-        if (store == STORE_C_GENERIC) return launch_shape<KIND_INT8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
-        return launch_shape<KIND_INT8, STORE_C>(p, tile_m, tile_n, stream);
-    }
-    if (kind == KIND_FP8) {
-        if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);
-        if (store == STORE_C_GENERIC) return launch_shape<KIND_FP8, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
-        return launch_shape<KIND_FP8, STORE_C>(p, tile_m, tile_n, stream);
-    }
-    if (kind == KIND_BF16) {
-        if (store == STORE_ACC) return launch_shape<KIND_BF16, STORE_ACC>(p, tile_m, tile_n, stream);
-        if (store == STORE_C_GENERIC) return launch_shape<KIND_BF16, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
-        return launch_shape<KIND_BF16, STORE_C>(p, tile_m, tile_n, stream);
-    }
-    if (kind == KIND_FP16) {
-        if (store == STORE_ACC) return launch_shape<KIND_FP16, STORE_ACC>(p, tile_m, tile_n, stream);
-        if (store == STORE_C_GENERIC) return launch_shape<KIND_FP16, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
-        return launch_shape<KIND_FP16, STORE_C>(p, tile_m, tile_n, stream);
-    }
-    if (kind == KIND_MXFP4) {
-        if (store == STORE_ACC) return launch_shape<KIND_MXFP4, STORE_ACC>(p, tile_m, tile_n, stream);
-        if (store == STORE_C_GENERIC) return launch_shape<KIND_MXFP4, STORE_C_GENERIC>(p, tile_m, tile_n, stream);
-        return launch_shape<KIND_MXFP4, STORE_C>(p, tile_m, tile_n, stream);
-    }
-    return hipErrorInvalidValue;
-}
