@@ -25,6 +25,8 @@ EXPORTS = (
     "psg_gemm_a8w8_acc",
     "psg_gemm_mxfp4",
     "psg_gemm_mxfp4_acc",
+    "psg_quant_pertoken",
+    "psg_quant_mxfp4",
 )
 
 
@@ -104,6 +106,12 @@ def lib() -> ctypes.CDLL:
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    handle.psg_quant_pertoken.restype = ctypes.c_int
+    handle.psg_quant_pertoken.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
+                                          ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+    handle.psg_quant_mxfp4.restype = ctypes.c_int
+    handle.psg_quant_mxfp4.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
+                                       ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
     got = handle.psg_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}")

@@ -11,6 +11,9 @@
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
+hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float* scale, int M, int K, int out_fp8, hipStream_t stream);
+hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
+                                  hipStream_t stream);
 
 namespace {
 
@@ -228,5 +231,30 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
 int psg_gemm_mxfp4(const psg_mxfp4_args* args, void* stream) { return mx_common(args, args ? args->c : nullptr, STORE_C, stream); }
 
 int psg_gemm_mxfp4_acc(const psg_mxfp4_args* args, void* acc, void* stream) { return mx_common(args, acc, STORE_ACC, stream); }
+
+int psg_quant_pertoken(const void* x, int32_t x_dtype, void* y, float* scale, int32_t M, int32_t K, int32_t out_dtype, void* stream) {
+    if (!x || !y || !scale) return fail(PSG_E_NULL, "x, y and scale must be non-NULL");
+    if (x_dtype < 0 || x_dtype > 2) return fail(PSG_E_DTYPE, "x_dtype %d unknown (0 fp32, 1 bf16, 2 fp16)", x_dtype);
+    if (out_dtype != PSG_IN_INT8 && out_dtype != PSG_IN_FP8_E4M3FN) return fail(PSG_E_DTYPE, "out_dtype must be int8 or fp8");
+    if (M < 1 || K < 8 || K % 8) return fail(PSG_E_SHAPE, "need M >= 1 and K a positive multiple of 8 (got M=%d K=%d)", M, K);
+    if (!aligned(x, 16) || !aligned(y, 8)) return fail(PSG_E_ALIGN, "x must be 16-byte and y 8-byte aligned");
+    const hipError_t e = psg_launch_quant_pertoken(x, x_dtype, y, scale, M, K, out_dtype == PSG_IN_FP8_E4M3FN, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_quant_pertoken launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+int psg_quant_mxfp4(const void* x, int32_t x_dtype, void* packed, void* scales, int32_t M, int32_t K, int32_t shuffled, void* stream) {
+    if (!x || !packed || !scales) return fail(PSG_E_NULL, "x, packed and scales must be non-NULL");
+    if (x_dtype < 0 || x_dtype > 2) return fail(PSG_E_DTYPE, "x_dtype %d unknown (0 fp32, 1 bf16, 2 fp16)", x_dtype);
+    if (M < 1 || K < 32 || K % 32) return fail(PSG_E_SHAPE, "need M >= 1 and K a positive multiple of 32 (got M=%d K=%d)", M, K);
+    if (shuffled && K % 256) return fail(PSG_E_SHAPE, "the shuffled scale layout needs K %% 256 == 0 (got K=%d)", K);
+    if (!aligned(x, 16) || !aligned(packed, 16)) return fail(PSG_E_ALIGN, "x and packed must be 16-byte aligned");
+    const int R = (M + 31) / 32 * 32;  // scales cover whole 32-row chunks; the padding rows get scale byte 0
+    const hipError_t e = psg_launch_quant_mxfp4(x, x_dtype, packed, scales, M, R, K, shuffled, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_quant_mxfp4 launch");
+    g_err[0] = 0;
+    return 0;
+}
 
 }  // extern "C"

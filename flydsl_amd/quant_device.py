@@ -1,0 +1,54 @@
+"""On-device activation quantisers (HIP kernels behind the C ABI): the same bytes as the host helpers in
+``flydsl_amd.quant`` (and therefore as the reference's ``pertoken_quant`` tests/utils.py:29-73 and
+``per_1x32_f4_quant`` + ``shuffle_scale_w4`` tests/kernels/utils/gemm_common_utils.py:675-704, 645-672), produced
+without leaving the GPU.  torch is used for the output allocations only."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .quant import fp4x2, fp8_e8m0
+
+_X_DTYPE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def _x_code(x):
+    if x.dtype not in _X_DTYPE:
+        raise TypeError(f"input dtype {x.dtype} is not supported (fp32 / bf16 / fp16)")
+    if not x.is_cuda or x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous 2-D device tensor")
+    return _X_DTYPE[x.dtype]
+
+
+def pertoken_quant(x: torch.Tensor, quant_dtype=torch.int8, stream=None):
+    """Per-row symmetric quantisation on the device.  Returns ``(y [M,K] quant_dtype, scale [M,1] fp32)``."""
+    code = _x_code(x)
+    if quant_dtype == torch.int8:
+        out = 0
+    elif quant_dtype == torch.float8_e4m3fn:
+        out = 1
+    else:
+        raise ValueError(f"quant_dtype must be torch.int8 or torch.float8_e4m3fn, got {quant_dtype}")
+    m, k = x.shape
+    y = torch.empty((m, k), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((m, 1), dtype=torch.float32, device=x.device)
+    rc = _lib.lib().psg_quant_pertoken(x.data_ptr(), code, y.data_ptr(), scale.data_ptr(), m, k, out, _lib.stream_handle(stream))
+    if rc:
+        _lib.check(rc, "psg_quant_pertoken")
+    return y.view(quant_dtype), scale
+
+
+def per_1x32_f4_quant(x: torch.Tensor, shuffle: bool = True, stream=None):
+    """OCP-MX fp4 quantisation on the device.  Returns ``(packed [M,K/2], scales)`` where ``scales`` are e8m0 bytes over
+    ``ceil(M/32)*32`` rows x ``K/32``: in the GEMM's shuffled layout when ``shuffle`` (default), row-major otherwise."""
+    code = _x_code(x)
+    m, k = x.shape
+    r = (m + 31) // 32 * 32
+    packed = torch.empty((m, k // 2), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((r, k // 32), dtype=torch.uint8, device=x.device)
+    rc = _lib.lib().psg_quant_mxfp4(x.data_ptr(), code, packed.data_ptr(), scales.data_ptr(), m, k, 1 if shuffle else 0,
+                                    _lib.stream_handle(stream))
+    if rc:
+        _lib.check(rc, "psg_quant_mxfp4")
+    return packed.view(fp4x2), scales.view(fp8_e8m0)

@@ -21,6 +21,8 @@
  *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm), fp4 x fp4, batch 1
  *   psg_gemm_mxfp4_acc  no counterpart: fp32 accumulators of the MXFP4 mainloop, for parity tests
  *   psg_workspace_bytes no counterpart (the reference has no split-K path)
+ *   psg_quant_pertoken  device version of the host quantiser tests/utils.py:29-73
+ *   psg_quant_mxfp4     device version of tests/kernels/utils/gemm_common_utils.py:675-704 (+ :645-672)
  */
 #ifndef PSGEMM_H
 #define PSGEMM_H
@@ -141,6 +143,22 @@ int psg_gemm_mxfp4(const psg_mxfp4_args *args, void *stream);
 /* Same mainloop, but writes the fp32 accumulators [M,N] to `acc` instead of C (no counterpart in the
  * reference; parity tests use it to look at the sum before the 16-bit rounding). */
 int psg_gemm_mxfp4_acc(const psg_mxfp4_args *args, void *acc, void *stream);
+
+/*
+ * On-device activation quantisers (the step before the GEMM).  The reference quantises on the host with
+ * tests/utils.py:29-73 (pertoken_quant) and tests/kernels/utils/gemm_common_utils.py:675-704 (per_1x32_f4_quant)
+ * followed by :645-672 (shuffle_scale_w4); these produce the same bytes on the device.
+ *   x_dtype: 0 fp32, 1 bf16, 2 fp16.  x is [M,K] row-major.
+ */
+
+/* y [M,K] int8 (out_dtype PSG_IN_INT8) or e4m3fn (PSG_IN_FP8_E4M3FN); scale [M] fp32 = max|row| / dtypeMax. K % 8 == 0. */
+int psg_quant_pertoken(const void *x, int32_t x_dtype, void *y, float *scale, int32_t M, int32_t K, int32_t out_dtype,
+                       void *stream);
+
+/* packed [M,K/2] e2m1 pairs; scales: e8m0 bytes over ceil(M/32)*32 rows x K/32, row-major (shuffled = 0) or in the
+ * shuffle_scale_w4 layout the GEMM reads (shuffled = 1, needs K % 256 == 0).  K % 32 == 0. */
+int psg_quant_mxfp4(const void *x, int32_t x_dtype, void *packed, void *scales, int32_t M, int32_t K, int32_t shuffled,
+                    void *stream);
 
 #ifdef __cplusplus
 }
