@@ -179,6 +179,51 @@ def run_workload(name, steps, warmup, check=True):
     return res, host
 
 
+def run_quant_workload(name, steps=50, warmup=5):
+    """The on-device quantisers that feed the GEMM: bf16 activations [M,K] -> fp8 + per-row scales, or -> MXFP4 + shuffled
+    e8m0 scales.  HBM-bound; algorithmic bytes = input + outputs, each touched once."""
+    import numpy as np
+    import torch
+
+    from flydsl_amd import quant_device
+    from oracle import psg_oracle as O
+
+    kind, M, K = {"quant_pertoken_fp8_m8192": ("fp8", 8192, 4096), "quant_mxfp4_m4096": ("fp4", 4096, 2048)}[name]
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    host = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    n_sets = max(2, min(32, math.ceil(2 * MALL_BYTES / (M * K * 2))))
+    xs = [host.to(dev) for _ in range(n_sets)]
+    if kind == "fp8":
+        f = lambda x: quant_device.pertoken_quant(x, quant_dtype=torch.float8_e4m3fn)  # noqa: E731
+        nbytes = M * K * 2 + M * K + M * 4
+    else:
+        f = lambda x: quant_device.per_1x32_f4_quant(x, shuffle=True)  # noqa: E731
+        nbytes = M * K * 2 + M * K // 2 + M * K // 32
+    for i in range(warmup):
+        out = f(xs[i % n_sets])
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for i in range(steps):
+        out = f(xs[i % n_sets])
+    ev1.record()
+    torch.cuda.synchronize()
+    sec = ev0.elapsed_time(ev1) * 1e-3 / steps
+    if kind == "fp8":
+        wy, ws = O.pertoken_quant(host.float().numpy(), "fp8")
+        ok = bool(np.array_equal(out[0].view(torch.uint8).cpu().numpy(), wy) and np.array_equal(out[1].cpu().numpy(), ws))
+    else:
+        wp, ws = O.per_1x32_f4_quant(host.float().numpy())
+        ok = bool(np.array_equal(out[0].view(torch.uint8).cpu().numpy(), wp) and
+                  np.array_equal(out[1].view(torch.uint8).cpu().numpy(), O.shuffle_scale_w4(ws)))
+    achieved = nbytes / sec / 1e9
+    return {"workload": name, "dtype": kind, "M": M, "K": K, "gb_per_s": achieved, "us_per_launch_events": sec * 1e6,
+            "operand_sets": n_sets, "parity_ok": ok, "timing": "eager launches incl. output allocation, HIP events",
+            "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK["hbm"], "unit": "GB/s", "frac": achieved / PEAK["hbm"],
+                         "traffic": None, "algorithmic_bytes": nbytes}}
+
+
 def cpu_baseline(name, host, budget_s=12.0):
     """The reference's torch CPU path (dequantise to fp32 + torch.mm) on the same seeded operands,
     timed on this box's host cores.  For workloads whose single pass exceeds the budget a row sample of
@@ -285,6 +330,8 @@ def main():
             r, _ = run_workload(name, 300 if b == "hbm" else (5 if name == "int8_ffn_m4096" else 20), 20 if b == "hbm" else 2)
             r["roofline"]["traffic"] = load_traffic(name)
             others.append(r)
+        for name in ("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"):
+            others.append(run_quant_workload(name))
 
     line = {
         "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",

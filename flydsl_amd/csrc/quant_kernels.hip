@@ -68,15 +68,27 @@ __device__ __forceinline__ float clean(float t, float dmax) {
 
 template <int OUT_FP8>
 __device__ __forceinline__ void quant_store8(const float* v, float s, uint8_t* dst) {
-    uint32_t b[8];
+    float q[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        const float q = v[e] / s;  // correctly rounded fp32 division
-        b[e] = OUT_FP8 ? f32_to_e4m3fn(q) : ((uint32_t)(int32_t)q & 0xFFu);  // float -> int truncates toward zero
-    }
+    for (int e = 0; e < 8; e++) q[e] = v[e] / s;  // correctly rounded fp32 division
     v2i o;
-    o[0] = (int)(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24));
-    o[1] = (int)(b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+    if constexpr (OUT_FP8) {
+        // v_cvt_pk_fp8_f32: two fp32 -> two OCP e4m3 bytes, round to nearest even (|q| <= 448 here, so its
+        // saturation never comes into play)
+        unsigned w0 = 0, w1 = 0;
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], w0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], w1, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
+        o[0] = (int)w0;
+        o[1] = (int)w1;
+    } else {
+        uint32_t b[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) b[e] = (uint32_t)(int32_t)q[e] & 0xFFu;  // float -> int truncates toward zero
+        o[0] = (int)(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24));
+        o[1] = (int)(b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+    }
     *reinterpret_cast<v2i*>(dst) = o;
 }
 
@@ -167,9 +179,12 @@ __global__ void __launch_bounds__(256) k_quant_mxfp4(const void* x, uint8_t* pac
         v4i o;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            uint32_t word = 0;
-#pragma unroll
-            for (int j = 0; j < 8; j++) word |= e2m1_code(v[w * 8 + j] / sf) << (4 * j);
+            // v_cvt_scalef32_pk_fp4_f32: (a, b) / scale -> two e2m1 codes (a in the low nibble) into one byte of the word
+            unsigned word = 0;
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 0], v[w * 8 + 1], sf, 0);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 2], v[w * 8 + 3], sf, 1);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 4], v[w * 8 + 5], sf, 2);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 6], v[w * 8 + 7], sf, 3);
             o[w] = (int)word;
         }
         *reinterpret_cast<v4i*>(packed + (size_t)r * (K >> 1) + (size_t)kb * 16) = o;
