@@ -2,7 +2,10 @@
 //
 //   C[M,N] = A[M,K] * W[N,K]^T, W preshuffled into 1 KB fragment blocks [N/16][K/64][klane 4][nlane 16][16 B].
 //
-// One workgroup = 4 wavefronts side by side along N; tile = (16*MR) x (64*NR) x 128 bytes of K.
+// One workgroup = 4 wavefronts arranged WM x WN (1x4: side by side along N, or 2x2); each wavefront owns MR x NR
+// MFMA blocks, so the tile is (16*MR*WM) x (16*NR*WN) x 128 bytes of K.  The 1x4 layout reads every W fragment
+// from memory once but makes every wavefront read the whole A tile from LDS; the 2x2 layout halves the LDS reads
+// and loads every W fragment twice (the second time from L1).
 //   * A tile: global -> VGPR -> LDS (XOR-swizzled 128-byte rows), double buffered, read back as
 //     MFMA fragments with ds_read_b128.
 //   * B fragments: each wave loads its own 1 KB blocks straight from global memory into the MFMA
@@ -81,17 +84,19 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
-template <int KIND, int MR, int NR, int STORE>
+template <int KIND, int MR, int NR, int WM, int STORE>
 __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
-    constexpr int TM = 16 * MR;
-    constexpr int TN = 64 * NR;
+    constexpr int WN = 4 / WM;
+    constexpr int TM = 16 * MR * WM;
+    constexpr int TN = 16 * NR * WN;
     constexpr int A_LOADS = TM / 32;  // 16-byte chunks of the A tile per thread
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * TK];
 
     const int tid = threadIdx.x;
     const int wave = wave_id();
+    const int wm = wave / WN, wn = wave % WN;  // this wavefront's place in the workgroup
     const int lane = tid & 63;
     const int li = lane & 15;
     const int lg = lane >> 4;
@@ -112,7 +117,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     const uint64_t a_rows = (uint64_t)(p.M - m0);
     __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a + (uint64_t)m0 * K, a_rows * (uint64_t)K);
     // B: this wave's NR n-blocks; blocks >= N/16 read as zero
-    const int nb0 = (n0 >> 4) + wave * NR;
+    const int nb0 = (n0 >> 4) + wn * NR;
     const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)K;
     const uint64_t b_total = (uint64_t)p.N * (uint64_t)K;
     __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
@@ -125,9 +130,10 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     if constexpr (KIND == KIND_MXFP4) {
         static_assert(KIND != KIND_MXFP4 || (MR % 2 == 0 && NR % 2 == 0), "scale chunks cover 32 rows");
         chunk_bytes = (uint32_t)KT * 256u;
-        const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5), sa_first = (uint64_t)(m0 >> 5);
-        rsa = make_rsrc(p.mx_sa + sa_first * chunk_bytes, (sa_chunks - sa_first) * chunk_bytes);
-        const uint64_t sb_chunks = (uint64_t)(p.N >> 5), sb_first = (uint64_t)((n0 >> 5) + wave * NP);
+        const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5), sa_first = (uint64_t)((m0 >> 5) + wm * MP);
+        rsa = make_rsrc(p.mx_sa + (sa_first < sa_chunks ? sa_first : sa_chunks) * chunk_bytes,
+                        sa_first < sa_chunks ? (sa_chunks - sa_first) * chunk_bytes : 0);
+        const uint64_t sb_chunks = (uint64_t)(p.N >> 5), sb_first = (uint64_t)((n0 >> 5) + wn * NP);
         rsb = make_rsrc(p.mx_sb + (sb_first < sb_chunks ? sb_first : sb_chunks) * chunk_bytes,
                         sb_first < sb_chunks ? (sb_chunks - sb_first) * chunk_bytes : 0);
     }
@@ -182,7 +188,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
         if (idx & 1) hi[ni] = v; else lo[ni] = v;
     };
     auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {
-        const int row = mi * 16 + li;
+        const int row = (wm * MR + mi) * 16 + li;
         flo = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
         fhi = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
     };
@@ -211,11 +217,14 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
                     else if constexpr (idx < N_LOADS) load_sc1(kt + 1, idx - 2 * NR, sav[S ^ 1], sbv[S ^ 1]);
                 });
             } else {
-                constexpr int j = mi - HALF;
-                if constexpr (j < A_LOADS) {
-                    store_a1(S ^ 1, j, areg[j]);
-                    load_a1(kt + 2, j, areg[j]);
-                }
+                constexpr int A_PER = (A_LOADS + (MR - HALF) - 1) / (MR - HALF);
+                static_for<A_PER>([&](auto Q) {
+                    constexpr int j = (mi - HALF) * A_PER + decltype(Q)::value;
+                    if constexpr (j < A_LOADS) {
+                        store_a1(S ^ 1, j, areg[j]);
+                        load_a1(kt + 2, j, areg[j]);
+                    }
+                });
             }
             // keep the memory instructions above ahead of this block's MFMAs (the machine scheduler would
             // otherwise cluster them at the top of the step)
@@ -292,12 +301,12 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     if constexpr (STORE != STORE_ACC && SCALED) {
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) {
-            const int m = m0 + mi * 16 + li;
+            const int m = m0 + (wm * MR + mi) * 16 + li;
             sa_v[mi] = p.sa[m < p.M ? m : p.M - 1];
         }
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
-            const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+            const int n = n0 + (wn * NR + ni) * 16 + lg * 4;
             sb_v[ni] = *reinterpret_cast<const v4f*>(p.sb + (n < p.N ? n : 0));
         }
     }
@@ -306,13 +315,13 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     // so the accumulators are never addressed dynamically.
     static_for<MR>([&](auto MI) {
         constexpr int mi = decltype(MI)::value;
-        const int m = m0 + mi * 16 + li;
+        const int m = m0 + (wm * MR + mi) * 16 + li;
         if (m < p.M) {
             float sa = 0.f;
             if constexpr (STORE != STORE_ACC && SCALED) sa = sa_v[mi];
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
-                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                const int n = n0 + (wn * NR + ni) * 16 + lg * 4;
                 if (n < p.N) {
                     const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
                     const acc_t r = acc[mi][ni];
@@ -339,29 +348,33 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     });
 }
 
-template <int KIND, int MR, int NR, int STORE>
+template <int KIND, int MR, int NR, int WM, int STORE>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
-    constexpr int TM = 16 * MR, TN = 64 * NR;
+    constexpr int TM = 16 * MR * WM, TN = 16 * NR * (4 / WM);
     const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
-    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, STORE>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 
+// p.ksplit selects the wavefront layout of the 256x256 tile: 2 = 2x2 wavefronts, anything else = 1x4
 template <int KIND, int STORE>
 hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t stream) {
-#define PSG_CASE(MR_, NR_) \
-    if (tile_m == 16 * MR_ && tile_n == 64 * NR_) return launch_one<KIND, MR_, NR_, STORE>(p, stream);
-    PSG_CASE(16, 4)
-    PSG_CASE(8, 8)
-    PSG_CASE(8, 4)
-    PSG_CASE(4, 4)
-    PSG_CASE(2, 4)
+#define PSG_CASE(MR_, NR_, WM_) \
+    if (tile_m == 16 * MR_ * WM_ && tile_n == 16 * NR_ * (4 / WM_)) return launch_one<KIND, MR_, NR_, WM_, STORE>(p, stream);
+    if (p.ksplit == 2) {
+        PSG_CASE(8, 8, 2)
+    }
+    PSG_CASE(16, 4, 1)
+    PSG_CASE(8, 8, 1)
+    PSG_CASE(8, 4, 1)
+    PSG_CASE(4, 4, 1)
+    PSG_CASE(2, 4, 1)
     if constexpr (KIND == KIND_MXFP4) {
-        PSG_CASE(4, 2)
-        PSG_CASE(2, 2)
+        PSG_CASE(4, 2, 1)
+        PSG_CASE(2, 2, 1)
     } else {
-        PSG_CASE(8, 2)
-        PSG_CASE(4, 1)
+        PSG_CASE(8, 2, 1)
+        PSG_CASE(4, 1, 1)
     }
 #undef PSG_CASE
     return hipErrorInvalidConfiguration;

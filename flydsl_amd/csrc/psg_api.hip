@@ -146,7 +146,7 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
         e = psg_launch_a8w8_smallm(p, kind, store, nb, static_cast<hipStream_t>(stream));
     } else {
         const Tile t = pick_tile(a->M, a->N, false, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
-        p.ksplit = 1;
+        p.ksplit = a->reserved == 2 ? 2 : 1;  // wavefront layout of the 256x256 tile (2 = 2x2), a test / tuning knob
         e = psg_launch_a8w8_tiled(p, kind, store, t.m, t.n, static_cast<hipStream_t>(stream));
     }
     if (e != hipSuccess) return hip_fail(e, "psg_gemm_a8w8 launch");
@@ -218,7 +218,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         q.N = p.N;
         q.K = p.K;
         q.group_m = p.group_m;
-        q.ksplit = 1;
+        q.ksplit = a->reserved == 2 ? 2 : 1;
         q.epi = EPI_NONE;
         q.out = p.out;
         e = psg_launch_a8w8_tiled(q, KIND_MXFP4, store, t.m, t.n, static_cast<hipStream_t>(stream));

@@ -55,6 +55,7 @@ def launch_gemm(
     _force_path=0,
     _tile=None,
     _acc=None,
+    _wave_layout=0,
 ):
     """Launch ``C[M,N] = A_mx[M,K] @ W_mx[N,K]^T`` on ``stream``.  The reference's constraints are kept:
     ``tile_k in {128, 256}``, ``tile_n % 128 == 0``, ``K % tile_k == 0`` (mxfp4_preshuffle.py:122,316)."""
@@ -87,6 +88,7 @@ def launch_gemm(
         args.tile_m, args.tile_n = int(_tile[0]), int(_tile[1])
     args.xcd_swizzle = int(xcd_swizzle)
     args.force_path = int(_force_path)
+    args.reserved = int(_wave_layout)
     lib = _lib.lib()
     if _acc is None:
         rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))

@@ -99,21 +99,23 @@ class PreshuffleGemm:
         if rc:
             _lib.check(rc, "psg_gemm_a8w8")
 
-    def accumulators(self, acc, A, B, M, N, stream=None, force_path=0, tile=None):
+    def accumulators(self, acc, A, B, M, N, stream=None, force_path=0, tile=None, wave_layout=0):
         """Write the raw accumulators ``[M, N]`` (int32 for int8, fp32 for fp8) into ``acc``."""
         args = self._fill(acc, A, B, None, None, None, M, N)
         args.force_path = int(force_path)
+        args.reserved = int(wave_layout)
         if tile is not None:
             args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
         rc = self._lib.psg_gemm_a8w8_acc(ctypes.byref(args), acc.data_ptr(), _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_gemm_a8w8_acc")
 
-    def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None):
+    def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None, wave_layout=0):
         """Like ``__call__`` but pins the regime (1 = MFMA mainloop, 2 = small-M) and optionally the
         native tile ``(tile_m, tile_n)``; for tests and benchmarks."""
         args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
         args.force_path = int(force_path)
+        args.reserved = int(wave_layout)
         if tile is not None:
             args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
         rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
