@@ -144,3 +144,23 @@ def stream_handle(stream) -> int:
     if h is None:
         raise TypeError(f"cannot use {type(stream).__name__} as a stream")
     return int(h)
+
+
+_workspaces = {}
+
+
+def workspace(device, nbytes: int):
+    """Per-device scratch for the split-K path (one torch allocation, grown on demand, zero-size means none).
+    Growing allocates, so the first call for a new largest problem must happen outside graph capture -- which the
+    reference's own protocol guarantees (``flyc.compile`` runs the launcher once before any capture).  Launches
+    that may overlap on one device (different streams) must not rely on this shared buffer."""
+    import torch
+
+    if nbytes <= 0:
+        return None
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    cur = _workspaces.get(key)
+    if cur is None or cur.numel() < nbytes:
+        cur = torch.empty(int(nbytes), dtype=torch.uint8, device=f"cuda:{key}")
+        _workspaces[key] = cur
+    return cur

@@ -43,8 +43,8 @@ struct Acc<KIND_INT8> {
 // MFMA through inline assembly with the accumulator constrained to the AGPR file ("+a").  With the builtin
 // the register allocator is free to place accumulators in either file; at 256 accumulator registers per lane
 // it then shuffles them between the files inside the main loop.  The accumulator of each call is both vDst
-// and SrcC (in-place accumulate); the compiler does not know these are MFMAs, so the kernel never reads an
-// accumulator with a non-MFMA instruction without a barrier and explicit wait states in between.
+// and SrcC (in-place accumulate); the compiler does not know these are MFMAs, so the kernel itself provides the
+// wait states between the last MFMA of a K step and anything else that may read an accumulator.
 __device__ __forceinline__ void mfma_f8(v4f& c, const v8i& a, const v8i& b) {
     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
@@ -112,6 +112,11 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;  // per-token x per-channel fp32 scales in the epilogue
     const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : (IS16 ? (p.K << 1) : p.K);
     const int KT = (K + TK - 1) / TK;
+    // split-K: workgroup blockIdx.y of p.splits covers K steps [kt_begin, kt_end) and (STORE_ACC only) writes its
+    // accumulators to slice blockIdx.y of the partials buffer
+    const int kt_per = (KT + p.splits - 1) / p.splits;
+    const int kt_begin = (int)blockIdx.y * kt_per;
+    const int kt_end = (kt_begin + kt_per) < KT ? (kt_begin + kt_per) : KT;
 
     // A: this tile's rows; rows >= M read as zero through the descriptor bound
     const uint64_t a_rows = (uint64_t)(p.M - m0);
@@ -161,7 +166,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     // until they are used, so no wait is forced early.
     auto load_a1 = [&](int kt, int j, v4i& dst) {
         const uint32_t k0 = (uint32_t)kt * TK;
-        const bool in_k = (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
+        const bool in_k = kt < kt_end && (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
         const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0;
         dst = buf_load16(ra, in_k ? off : 0xFFFFFFF0u, 0);
     };
@@ -172,7 +177,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     // the bounds-checked VGPR offset (blocks >= N/16 read as zero), the K position in the scalar offset.
     // MXFP4: load number 2*NR + q fetches scale dword q of the step (A-side chunks first, then W-side)
     auto load_sc1 = [&](int kt, int q, int* sa_dst, int* sb_dst) {
-        const bool has = kt < KT;
+        const bool has = kt < kt_end;
         const uint32_t soff = has ? (uint32_t)kt * 256u : 0u;
         if (q < MP) {
             sa_dst[q] = buf_load4(rsa, has ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
@@ -182,7 +187,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     };
     auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi) {
         const int ni = idx >> 1;
-        const bool has = (kt * TK + (idx & 1) * 64) < K;
+        const bool has = kt < kt_end && (kt * TK + (idx & 1) * 64) < K;
         const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
         const v4i v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, has ? (uint32_t)kt * 2048u + (uint32_t)(idx & 1) * 1024u : 0u);
         if (idx & 1) hi[ni] = v; else lo[ni] = v;
@@ -264,36 +269,39 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        // The compiler does not know that the asm statements above are MFMAs, so it inserts none of the wait
+        // states a non-MFMA read of an accumulator needs after the last MFMA that wrote it (11 for an 8-pass
+        // MFMA).  Nothing inside the loop reads accumulators, but the code after the loop does, and the compiler may
+        // place such a read (even a plain register copy) first thing after the loop.  Wait states directly behind
+        // the last MFMA of every step cover that: volatile asm statements keep their order, and code after the
+        // loop cannot move up across the barrier below.
+        asm volatile("s_nop 15" ::: "memory");
         __syncthreads();
     };
 
     // prologue: A(0) -> LDS stage 0, A(1) -> registers, W(0) -> set 0
 #pragma unroll
-    for (int j = 0; j < A_LOADS; j++) load_a1(0, j, areg[j]);
+    for (int j = 0; j < A_LOADS; j++) load_a1(kt_begin, j, areg[j]);
 #pragma unroll
-    for (int idx = 0; idx < 2 * NR; idx++) load_b1(0, idx, blo[0], bhi[0]);
+    for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin, idx, blo[0], bhi[0]);
     if constexpr (KIND == KIND_MXFP4) {
 #pragma unroll
-        for (int q = 0; q < MP + NP; q++) load_sc1(0, q, sav[0], sbv[0]);
+        for (int q = 0; q < MP + NP; q++) load_sc1(kt_begin, q, sav[0], sbv[0]);
     }
 #pragma unroll
     for (int j = 0; j < A_LOADS; j++) {
         store_a1(0, j, areg[j]);
-        load_a1(1, j, areg[j]);
+        load_a1(kt_begin + 1, j, areg[j]);
     }
     __syncthreads();
 
     // Two K steps per iteration (LDS / register ping-pong).  When the step count is odd the last "odd" step
     // multiplies zero operands (its loads were redirected past the bounds): harmless, and the loop body stays
     // free of control flow, which the software pipeline needs.
-    for (int kt = 0; kt < KT; kt += 2) {
+    for (int kt = kt_begin; kt < kt_end; kt += 2) {
         step(kt, std::integral_constant<int, 0>{});
         step(kt + 1, std::integral_constant<int, 1>{});
     }
-
-    // the last MFMAs (up to 8 passes of 4 cycles each) must have left the pipeline before anything else reads
-    // an accumulator: the loop's final barrier is followed by explicit wait states
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
     // epilogue operands, fetched in one batch (one memory latency for the whole tile, not one per fragment)
     float sa_v[MR];
@@ -326,7 +334,8 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
                     const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
                     const acc_t r = acc[mi][ni];
                     if constexpr (STORE == STORE_ACC) {
-                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + idx * 4) = r;
+                        const size_t slice = (size_t)blockIdx.y * (size_t)p.M * (size_t)p.N;
+                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + (slice + idx) * 4) = r;
                     } else {
                         v4f x;
                         if constexpr (!SCALED) {
@@ -352,16 +361,19 @@ template <int KIND, int MR, int NR, int WM, int STORE>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
     constexpr int TM = 16 * MR * WM, TN = 16 * NR * (4 / WM);
     const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
-    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, p);
+    const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
+    A8W8Params q = p;
+    q.splits = splits;
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, stream, q);
     return hipGetLastError();
 }
 
-// p.ksplit selects the wavefront layout of the 256x256 tile: 2 = 2x2 wavefronts, anything else = 1x4
+// p.wave_layout selects the wavefront layout of the 256x256 tile: 2 = 2x2 wavefronts, anything else = 1x4
 template <int KIND, int STORE>
 hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t stream) {
 #define PSG_CASE(MR_, NR_, WM_) \
     if (tile_m == 16 * MR_ * WM_ && tile_n == 16 * NR_ * (4 / WM_)) return launch_one<KIND, MR_, NR_, WM_, STORE>(p, stream);
-    if (p.ksplit == 2) {
+    if (p.wave_layout == 2) {
         PSG_CASE(8, 8, 2)
     }
     PSG_CASE(16, 4, 1)

@@ -11,6 +11,7 @@
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
+hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
 hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float* scale, int M, int K, int out_fp8, hipStream_t stream);
 hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
                                   hipStream_t stream);
@@ -83,6 +84,37 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     return t;
 }
 
+// Split-K for the regime between the streaming kernel (M <= 32) and problems with enough tiles to fill the GPU:
+// with few tiles every workgroup walks all of K behind a one-step prefetch and the launch is latency-bound.
+// Splitting K over `splits` workgroups per tile multiplies the loads in flight; the price is one fp32 slice of
+// [M,N] per split written and read back, so the split count is capped where that traffic reaches a quarter of W.
+// Returns 1 when splitting does not pay.  kbytes = bytes of one operand row.
+int pick_splits(int M, int N, int kbytes, Tile t) {
+    const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
+    const int steps = (kbytes + 127) / 128;
+    if (tiles >= 192 || steps < 32) return 1;
+    // measured optimum: about 16 K steps per workgroup, at most ~1024 workgroups, partial traffic bounded
+    int s = 1;
+    while (s < 8 && steps / (s * 2) >= 16 && tiles * (s * 2) <= 1024 && (long)(s * 2) * M * 16 <= kbytes) s *= 2;
+    return s;
+}
+
+// Tile + split plan of the tiled path.  With few tiles and a long K (the regime between the streaming kernel and
+// GPU-filling problems) small square-ish tiles with split-K measured best: 64x64 up to M=64, 128x128 above.
+struct Plan {
+    Tile t;
+    int splits;
+};
+Plan plan_tiled(int M, int N, int kbytes, bool mx) {
+    Tile t = pick_tile(M, N, mx, 0, 0);
+    const long tiles_big = (long)((M + 127) / 128) * (long)((N + 255) / 256);
+    const int steps = (kbytes + 127) / 128;
+    if (!mx && tiles_big < 192 && steps >= 48) t = M <= 64 ? Tile{64, 64} : Tile{128, 128};
+    return {t, pick_splits(M, N, kbytes, t)};
+}
+
+uint64_t splitk_bytes(int M, int N, int splits) { return splits > 1 ? (uint64_t)splits * M * N * 4ull : 0; }
+
 int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
     if (!a) return fail(PSG_E_NULL, "args is NULL");
     if (!a->a || !a->b) return fail(PSG_E_NULL, "a and b must be non-NULL");
@@ -145,9 +177,25 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
         p.ksplit = pick_ksplit((a->N / 16 + nb - 1) / nb, steps);
         e = psg_launch_a8w8_smallm(p, kind, store, nb, static_cast<hipStream_t>(stream));
     } else {
-        const Tile t = pick_tile(a->M, a->N, false, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
-        p.ksplit = a->reserved == 2 ? 2 : 1;  // wavefront layout of the 256x256 tile (2 = 2x2), a test / tuning knob
-        e = psg_launch_a8w8_tiled(p, kind, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
+        const Plan plan = plan_tiled(a->M, a->N, kbytes, false);
+        const Tile t = forced ? Tile{a->tile_m, a->tile_n} : plan.t;
+        p.ksplit = 1;
+        p.wave_layout = a->reserved == 2 ? 2 : 1;  // wavefront layout of the 256x256 tile (2 = 2x2), a test / tuning knob
+        // forced launches take the split count from tile_k (1..16); otherwise the planner decides
+        int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
+        if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
+        p.splits = splits;
+        if (splits > 1) {
+            A8W8Params part = p;
+            part.c = a->workspace;
+            e = psg_launch_a8w8_tiled(part, kind, STORE_ACC, t.m, t.n, static_cast<hipStream_t>(stream));
+            if (e == hipSuccess)
+                e = psg_launch_splitk_finalize(p, a->workspace, kind == KIND_INT8, kind == KIND_INT8 || kind == KIND_FP8,
+                                               static_cast<hipStream_t>(stream));
+        } else {
+            e = psg_launch_a8w8_tiled(p, kind, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        }
     }
     if (e != hipSuccess) return hip_fail(e, "psg_gemm_a8w8 launch");
     g_err[0] = 0;
@@ -162,9 +210,13 @@ int psg_abi_version(void) { return PSG_ABI_VERSION; }
 
 const char* psg_last_error(void) { return g_err; }
 
-uint64_t psg_workspace_bytes(int32_t, int32_t, int32_t, int32_t) {
-    // Both regimes reduce inside one workgroup (registers / LDS); no global scratch is needed.
-    return 0;
+uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) {
+    // Only the split-K variant of the tiled path (few tiles, long K) uses global scratch: one fp32 / int32 slice of
+    // [M,N] per split.  Without it (NULL or too small) the library runs the same problem unsplit.
+    if (M <= kSmallM || M < 1 || N < 16 || K < 64) return 0;
+    const bool mx = in_dtype == 4;  // MXFP4 (psg_gemm_mxfp4)
+    const int kbytes = mx ? K / 2 : ((in_dtype == PSG_IN_FP16 || in_dtype == PSG_IN_BF16) ? K * 2 : K);
+    return splitk_bytes(M, N, plan_tiled(M, N, kbytes, mx).splits);
 }
 
 int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
@@ -207,7 +259,11 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         p.ksplit = pick_ksplit(a->N / 32, a->K / 256);
         e = psg_launch_mxfp4_smallm(p, store, static_cast<hipStream_t>(stream));
     } else {
-        const Tile t = pick_tile(a->M, a->N, true, a->force_path == 1 ? a->tile_m : 0, a->force_path == 1 ? a->tile_n : 0);
+        const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
+        const Plan plan = plan_tiled(a->M, a->N, a->K / 2, true);
+        const Tile t = forced ? Tile{a->tile_m, a->tile_n} : plan.t;
+        int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
+        if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
         A8W8Params q{};
         q.c = p.c;
         q.a = p.a;
@@ -218,10 +274,19 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         q.N = p.N;
         q.K = p.K;
         q.group_m = p.group_m;
-        q.ksplit = a->reserved == 2 ? 2 : 1;
+        q.ksplit = 1;
+        q.wave_layout = a->reserved == 2 ? 2 : 1;
+        q.splits = splits;
         q.epi = EPI_NONE;
         q.out = p.out;
-        e = psg_launch_a8w8_tiled(q, KIND_MXFP4, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        if (splits > 1) {
+            A8W8Params part = q;
+            part.c = a->workspace;
+            e = psg_launch_a8w8_tiled(part, KIND_MXFP4, STORE_ACC, t.m, t.n, static_cast<hipStream_t>(stream));
+            if (e == hipSuccess) e = psg_launch_splitk_finalize(q, a->workspace, 0, 0, static_cast<hipStream_t>(stream));
+        } else {
+            e = psg_launch_a8w8_tiled(q, KIND_MXFP4, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        }
     }
     if (e != hipSuccess) return hip_fail(e, "psg_gemm_mxfp4 launch");
     g_err[0] = 0;

@@ -106,6 +106,8 @@ struct A8W8Params {
     int M, N, K;
     int group_m;  // M-tiles per group of the XCD-aware tile order (tiled kernel)
     int ksplit;   // K splits per n-block (small-M kernel)
+    int splits;   // tiled kernel: workgroups along K per tile (> 1 only with STORE_ACC into a partials buffer)
+    int wave_layout;  // tiled kernel: 2 = 2x2 wavefronts for the 256x256 tile, else 1x4
     int epi;      // EPI_*
     int out;      // OUT_*
     const uint8_t* mx_sa;  // MXFP4 only: shuffled e8m0 [ceil(M/32)*32, K/32]

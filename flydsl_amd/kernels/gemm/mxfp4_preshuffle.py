@@ -56,6 +56,7 @@ def launch_gemm(
     _tile=None,
     _acc=None,
     _wave_layout=0,
+    _splits=0,
 ):
     """Launch ``C[M,N] = A_mx[M,K] @ W_mx[N,K]^T`` on ``stream``.  The reference's constraints are kept:
     ``tile_k in {128, 256}``, ``tile_n % 128 == 0``, ``K % tile_k == 0`` (mxfp4_preshuffle.py:122,316)."""
@@ -90,6 +91,14 @@ def launch_gemm(
     args.force_path = int(_force_path)
     args.reserved = int(_wave_layout)
     lib = _lib.lib()
+    if _tile is not None:
+        args.tile_k = max(1, int(_splits))
+        need = args.tile_k * args.M * args.N * 4 if args.tile_k > 1 else 0
+    else:
+        need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
+    if need and _acc is None and hasattr(arg_c, "device"):
+        ws = _lib.workspace(arg_c.device, need)
+        args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
     if _acc is None:
         rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))
     else:

@@ -91,6 +91,10 @@ class PreshuffleGemm:
         args.scale_b = scale_b.data_ptr() if scale_b is not None and scale_b.numel() else None
         args.bias = bias.data_ptr() if bias is not None and bias.numel() else None
         args.M = int(M)
+        need = self._lib.psg_workspace_bytes(args.M, self.N, self.K, args.in_dtype)
+        if need:
+            ws = _lib.workspace(C.device, need)
+            args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         return args
 
     def __call__(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
@@ -105,19 +109,23 @@ class PreshuffleGemm:
         args.force_path = int(force_path)
         args.reserved = int(wave_layout)
         if tile is not None:
-            args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
+            args.tile_m, args.tile_n, args.tile_k = int(tile[0]), int(tile[1]), 1
         rc = self._lib.psg_gemm_a8w8_acc(ctypes.byref(args), acc.data_ptr(), _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_gemm_a8w8_acc")
 
-    def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None, wave_layout=0):
+    def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None, wave_layout=0, splits=1):
         """Like ``__call__`` but pins the regime (1 = MFMA mainloop, 2 = small-M) and optionally the
-        native tile ``(tile_m, tile_n)``; for tests and benchmarks."""
+        native tile ``(tile_m, tile_n)`` and the number of K splits; for tests and benchmarks."""
         args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
         args.force_path = int(force_path)
         args.reserved = int(wave_layout)
         if tile is not None:
             args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
+            args.tile_k = int(splits)
+            if splits > 1:
+                ws = _lib.workspace(C.device, int(splits) * int(M) * self.N * 4)
+                args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_gemm_a8w8")

@@ -216,3 +216,17 @@ def test_graph_capture_matches_eager():
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(c, eager)
+
+
+# ---- very short K (one or two mainloop steps): the accumulators are read right after the last MFMA ------------
+@pytest.mark.parametrize("K", [64, 128, 256])
+def test_short_k_every_tile(K):
+    M, N = 256, 512
+    d = make_a8w8(M, N, K, "int8", seed=K)
+    want = O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"]))
+    ref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")["c_bf16_bits"]
+    for tile in [(256, 256), (128, 512), (128, 256), (64, 256), (32, 256), (128, 128), (64, 64)]:
+        for _ in range(3):
+            c = _launch(d, M, N, K, force_path=1, tile=tile)
+            assert np.array_equal(bf16_bits(c[:M]), ref), f"tile {tile}"
+            assert np.array_equal(_acc(d, M, N, K, force_path=1, tile=tile), want), f"tile {tile}"

@@ -111,3 +111,15 @@ def test_mxfp4_rejects_unbuilt_variants():
         args[idx] = val
         with pytest.raises(NotImplementedError):
             launch_gemm(*args)
+
+
+@pytest.mark.parametrize("K", [256, 512])
+def test_mxfp4_short_k_every_tile(K):
+    # one or two mainloop steps: the accumulators are read right after the last MFMA
+    M, N = 256, 512
+    d = make_mxfp4(M, N, K, seed=K)
+    want = C.mxfp4(d["a_q"].numpy(), d["b_shuf"].numpy(), d["sa_shuf"].numpy(), d["sb_shuf"].numpy(), M, N, K)["out_f32"]
+    for tile in [(256, 256), (128, 256), (64, 256), (32, 256), (64, 128), (32, 128)]:
+        for _ in range(3):
+            acc = _run(d, M, N, K, force_path=1, tile=tile, acc=True)
+            assert np.allclose(acc, want, rtol=1e-5, atol=1e-5 * np.abs(want).max()), f"tile {tile}"
