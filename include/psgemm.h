@@ -20,7 +20,7 @@
  *                       (int32 for int8, fp32 for fp8) so parity tests can check them bit-exactly
  *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm), fp4 x fp4, batch 1
  *   psg_gemm_mxfp4_acc  no counterpart: fp32 accumulators of the MXFP4 mainloop, for parity tests
- *   psg_workspace_bytes no counterpart (the reference has no split-K path)
+ *   psg_workspace_bytes no counterpart (the reference's preshuffle GEMM has no split-K path)
  *   psg_quant_pertoken  device version of the host quantiser tests/utils.py:29-73
  *   psg_quant_mxfp4     device version of tests/kernels/utils/gemm_common_utils.py:675-704 (+ :645-672)
  */
@@ -69,10 +69,9 @@ enum psg_error {
  *   scale_a  [M] fp32 per-token scales; scale_b [N] fp32 per-channel scales; ignored (may be NULL) for fp16 / bf16
  *   bias     [N] out_dtype, read only when epilogue != PSG_EPI_NONE
  *   N % 16 == 0, K*bytes_per_element % 64 == 0, 1 <= M <= 65536 (kernels/gemm/preshuffle_gemm.py:783-785)
- *   workspace / workspace_bytes: scratch for the small-M split-K path; may be NULL/0 when
- *            psg_workspace_bytes() returns 0 for the same (M,N,K,in_dtype).  Contents need no
- *            initialisation beyond being zero the first time the buffer is used; the kernels leave
- *            it zeroed again.  Two launches that may overlap in time must not share one workspace.
+ *   workspace / workspace_bytes: scratch for the split-K plan of the tiled path (32 < M, few tiles, long K):
+ *            psg_workspace_bytes() bytes, no initialisation needed.  May always be NULL/0: the library then
+ *            runs the problem unsplit.  Two launches that may overlap in time must not share one workspace.
  *   tile_m/tile_n/tile_k, xcd_swizzle: the reference's tuning keywords; accepted as hints
  *            (0 = library's choice).  The library picks its own tiling per regime.
  */
@@ -127,7 +126,8 @@ int psg_abi_version(void);
 /* Thread-local text of the last error returned on this thread ("" if none). */
 const char *psg_last_error(void);
 
-/* Bytes of workspace psg_gemm_a8w8 needs for this problem (0 when the chosen path needs none). */
+/* Bytes of workspace the split-K plan would use for this problem (0 when the chosen plan needs none).
+ * in_dtype: enum psg_in_dtype, or 4 for psg_gemm_mxfp4. */
 uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype);
 
 /* C = epilogue((acc * scale_a[m]) * scale_b[n]) on `stream` (a hipStream_t passed as void*). */
