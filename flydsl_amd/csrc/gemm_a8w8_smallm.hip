@@ -3,7 +3,7 @@
 // The whole cost is streaming W once (N*K bytes), so the kernel is organised around the 1 KB preshuffled
 // blocks [N/16][K/64]: a wavefront owns one 16-column n-block and a contiguous slice of K, issues the block
 // loads of a chunk of K steps up front (one fully coalesced 1 KB load per block, 16 bytes per lane) and
-// feeds the registers straight into MFMA.  A workgroup is 8 wavefronts = (8/ksplit) n-blocks x ksplit
+// feeds the registers straight into MFMA.  A workgroup is NW (4 or 8) wavefronts = (NW/ksplit) n-blocks x ksplit
 // K-slices; the K-slices of one n-block always sit in one workgroup, so the split-K reduction happens in LDS
 // in a fixed order (deterministic, single launch, no workspace).
 //
@@ -21,7 +21,6 @@
 
 namespace {
 
-constexpr int NW = 8;       // wavefronts per workgroup
 constexpr int UNROLL = 4;   // 128-byte K steps per chunk when 16 rows of A are staged (2 when 32 rows are)
 
 template <int KIND>
@@ -34,7 +33,9 @@ struct Acc<KIND_INT8> {
 };
 
 // NB = n-blocks per wavefront: with two, the A slice a wavefront stages is shared by twice as much of W.
-template <int KIND, int MB, int NB, int STORE>
+// NW = wavefronts per workgroup (4 or 8): four with longer K slices leave fewer partial sums to reduce and smaller
+// workgroups to place; eight give more, shorter slices when K is short.
+template <int KIND, int MB, int NB, int NW, int STORE>
 __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr int ROWS = 16 * MB;          // A rows staged
@@ -217,33 +218,39 @@ __global__ void __launch_bounds__(NW * 64) k_a8w8_smallm(A8W8Params p) {
     }
 }
 
-template <int KIND, int MB, int NB, int STORE>
+template <int KIND, int MB, int NB, int NW, int STORE>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
     const int per_wg = (NW / p.ksplit) * NB;  // n-blocks per workgroup
     const int n_blocks = p.N / 16;
     const int grid = (n_blocks + per_wg - 1) / per_wg;
-    hipLaunchKernelGGL((k_a8w8_smallm<KIND, MB, NB, STORE>), dim3(grid), dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((k_a8w8_smallm<KIND, MB, NB, NW, STORE>), dim3(grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
 template <int KIND, int STORE>
-hipError_t launch_kind(const A8W8Params& p, int nb, hipStream_t stream) {
+hipError_t launch_kind(const A8W8Params& p, int nb, int nw, hipStream_t stream) {
     const int mb = p.M <= 16 ? 1 : 2;
-    if (mb == 1) return nb == 2 ? launch_one<KIND, 1, 2, STORE>(p, stream) : launch_one<KIND, 1, 1, STORE>(p, stream);
-    return nb == 2 ? launch_one<KIND, 2, 2, STORE>(p, stream) : launch_one<KIND, 2, 1, STORE>(p, stream);
+#define PSG_GO(MB_, NB_)                                                                                   \
+    return nw == 4 ? launch_one<KIND, MB_, NB_, 4, STORE>(p, stream) : launch_one<KIND, MB_, NB_, 8, STORE>(p, stream);
+    if (mb == 1) {
+        if (nb == 2) { PSG_GO(1, 2) } else { PSG_GO(1, 1) }
+    }
+    if (nb == 2) { PSG_GO(2, 2) } else { PSG_GO(2, 1) }
+#undef PSG_GO
 }
 
 }  // namespace
 
-// Host entry used by the C-ABI layer.  Requires 1 <= M <= 32, p.ksplit in {1,2,4,8}, nb (n-blocks per wavefront) in {1,2}.
-hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, hipStream_t stream) {
+// Host entry used by the C-ABI layer.  Requires 1 <= M <= 32, nw (wavefronts per workgroup) in {4,8}, p.ksplit a power of
+// two <= nw, nb (n-blocks per wavefront) in {1,2}.
+hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, int nw, hipStream_t stream) {
     if (kind == KIND_INT8)
-        return store == STORE_ACC ? launch_kind<KIND_INT8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_INT8, STORE_C>(p, nb, stream);
+        return store == STORE_ACC ? launch_kind<KIND_INT8, STORE_ACC>(p, nb, nw, stream) : launch_kind<KIND_INT8, STORE_C>(p, nb, nw, stream);
     if (kind == KIND_FP8)
-        return store == STORE_ACC ? launch_kind<KIND_FP8, STORE_ACC>(p, nb, stream) : launch_kind<KIND_FP8, STORE_C>(p, nb, stream);
+        return store == STORE_ACC ? launch_kind<KIND_FP8, STORE_ACC>(p, nb, nw, stream) : launch_kind<KIND_FP8, STORE_C>(p, nb, nw, stream);
     if (kind == KIND_BF16)
-        return store == STORE_ACC ? launch_kind<KIND_BF16, STORE_ACC>(p, nb, stream) : launch_kind<KIND_BF16, STORE_C>(p, nb, stream);
+        return store == STORE_ACC ? launch_kind<KIND_BF16, STORE_ACC>(p, nb, nw, stream) : launch_kind<KIND_BF16, STORE_C>(p, nb, nw, stream);
     if (kind == KIND_FP16)
-        return store == STORE_ACC ? launch_kind<KIND_FP16, STORE_ACC>(p, nb, stream) : launch_kind<KIND_FP16, STORE_C>(p, nb, stream);
+        return store == STORE_ACC ? launch_kind<KIND_FP16, STORE_ACC>(p, nb, nw, stream) : launch_kind<KIND_FP16, STORE_C>(p, nb, nw, stream);
     return hipErrorInvalidValue;
 }
