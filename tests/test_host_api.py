@@ -216,3 +216,28 @@ def test_product_code_does_not_touch_the_oracle():
                     if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "psg_oracle" in text:
                         bad.append(os.path.join(dirpath, f))
     assert not bad, bad
+
+
+def test_compat_aliases_install_and_do_not_shadow():
+    import flydsl_amd.compat as compat
+
+    added = compat.install()
+    try:
+        import flydsl.compiler as flyc
+        from tests.kernels.utils import gemm_common_utils
+        from tests.test_common import verify_output
+        from tests.utils import pertoken_quant, shuffle_weight
+
+        assert flyc.compile is __import__("flydsl_amd.compiler", fromlist=["compile"]).compile
+        assert pertoken_quant is quant.pertoken_quant and shuffle_weight is layout.shuffle_weight
+        assert gemm_common_utils.shuffle_scale_w4 is layout.shuffle_scale_w4
+        ref = torch.ones(10, 100)
+        out = ref.clone()
+        out[0, :40] += 1.0
+        assert verify_output(out, ref, atol=0.1, rtol=0.1)
+        out[0:2] += 1.0
+        assert not verify_output(out, ref, atol=0.1, rtol=0.1)
+        assert compat.install() == []  # second call adds nothing
+    finally:
+        for name in added:
+            sys.modules.pop(name, None)
