@@ -3,8 +3,9 @@
 Drop-in for the reference's ``launch_gemm`` (kernels/gemm/mxfp4_preshuffle.py:57-91): same positional
 signature.  Operands are raw device pointers (what ``flyc.from_c_void_p(fx.Uint8, t.data_ptr())``
 produces: an object with an integer ``value``, or a plain int, or a tensor).  Supported subset:
-``a_dtype == b_dtype == "fp4"``, ``batch == 1`` and all strides ``-1``; the rest raises
-``NotImplementedError``.
+``a_dtype == b_dtype == "fp4"`` and all strides ``-1`` (the contiguous ``[B, M, *]`` layout); ``batch > 1`` runs one
+launch per batch on the same stream with the reference's default batch strides (mxfp4_preshuffle.py:177-196).  The
+rest raises ``NotImplementedError``.
 """
 
 from __future__ import annotations
@@ -62,8 +63,8 @@ def launch_gemm(
     ``tile_k in {128, 256}``, ``tile_n % 128 == 0``, ``K % tile_k == 0`` (mxfp4_preshuffle.py:122,316)."""
     if a_dtype != "fp4" or b_dtype != "fp4":
         raise NotImplementedError(f"only fp4 x fp4 is built (got a_dtype={a_dtype!r}, b_dtype={b_dtype!r})")
-    if int(batch) != 1:
-        raise NotImplementedError("strided-batched launch (batch > 1) is not built")
+    if int(batch) < 1:
+        raise ValueError(f"batch must be >= 1, got {batch}")
     if any(int(s) >= 0 for s in (a_row_stride, a_batch_stride, sca_row_stride, sca_batch_stride, c_row_stride, c_batch_stride)):
         raise NotImplementedError("caller-controlled row/batch strides are not built; pass -1")
     if out_dtype not in _lib.OUT_DTYPE:
@@ -76,32 +77,39 @@ def launch_gemm(
         raise ValueError(f"K={K} must be a multiple of tile_k={tile_k}")
     if int(i32_n) != int(N):
         raise ValueError(f"runtime N={i32_n} differs from the compile-time N={N}")
-    args = _lib.MxArgs()
-    args.c = _addr(arg_c) if _acc is None else None
-    args.a = _addr(arg_a)
-    args.b = _addr(arg_b)
-    args.scale_a = _addr(arg_scale_a)
-    args.scale_b = _addr(arg_scale_b)
-    args.M, args.N, args.K = int(i32_m), int(N), int(K)
-    args.out_dtype = _lib.OUT_DTYPE[out_dtype]
-    args.tile_m, args.tile_n, args.tile_k = int(tile_m), int(tile_n), int(tile_k)
-    if _tile is not None:
-        args.tile_m, args.tile_n = int(_tile[0]), int(_tile[1])
-    args.xcd_swizzle = int(xcd_swizzle)
-    args.force_path = int(_force_path)
-    args.reserved = int(_wave_layout)
+    M, Nn, Kk = int(i32_m), int(N), int(K)
+    # default batch strides of the reference: A [B,M,K/2], W [B,N,K/2], scale_a over ceil(M/32) chunks, scale_b over N/32
+    # chunks of (K/256)*256 bytes each, C [B,M,N]
+    chunk = (Kk // 256) * 256
+    strides = (M * Nn * 2, M * (Kk // 2), Nn * (Kk // 2), ((M + 31) // 32) * chunk, (Nn // 32) * chunk)
+    base = (None if _acc is not None else _addr(arg_c), _addr(arg_a), _addr(arg_b), _addr(arg_scale_a), _addr(arg_scale_b))
     lib = _lib.lib()
-    if _tile is not None:
-        args.tile_k = max(1, int(_splits))
-        need = args.tile_k * args.M * args.N * 4 if args.tile_k > 1 else 0
-    else:
-        need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
-    if need and _acc is None and hasattr(arg_c, "device"):
-        ws = _lib.workspace(arg_c.device, need)
-        args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
-    if _acc is None:
-        rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))
-    else:
-        rc = lib.psg_gemm_mxfp4_acc(ctypes.byref(args), _addr(_acc), _lib.stream_handle(stream))
-    if rc:
-        _lib.check(rc, "psg_gemm_mxfp4")
+    for bz in range(int(batch)):
+        args = _lib.MxArgs()
+        args.c = None if base[0] is None else base[0] + bz * strides[0]
+        args.a = base[1] + bz * strides[1]
+        args.b = base[2] + bz * strides[2]
+        args.scale_a = base[3] + bz * strides[3]
+        args.scale_b = base[4] + bz * strides[4]
+        args.M, args.N, args.K = M, Nn, Kk
+        args.out_dtype = _lib.OUT_DTYPE[out_dtype]
+        args.tile_m, args.tile_n, args.tile_k = int(tile_m), int(tile_n), int(tile_k)
+        if _tile is not None:
+            args.tile_m, args.tile_n = int(_tile[0]), int(_tile[1])
+        args.xcd_swizzle = int(xcd_swizzle)
+        args.force_path = int(_force_path)
+        args.reserved = int(_wave_layout)
+        if _tile is not None:
+            args.tile_k = max(1, int(_splits))
+            need = args.tile_k * args.M * args.N * 4 if args.tile_k > 1 else 0
+        else:
+            need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
+        if need and _acc is None and hasattr(arg_c, "device"):
+            ws = _lib.workspace(arg_c.device, need)
+            args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+        if _acc is None:
+            rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))
+        else:
+            rc = lib.psg_gemm_mxfp4_acc(ctypes.byref(args), _addr(_acc) + bz * M * Nn * 4, _lib.stream_handle(stream))
+        if rc:
+            _lib.check(rc, "psg_gemm_mxfp4")

@@ -106,7 +106,7 @@ def test_mxfp4_rejects_unbuilt_variants():
     from kernels.gemm.mxfp4_preshuffle import launch_gemm
 
     base = [0, 0, 0, 0, 0, 32, 128, None, 128, 256, 32, 128, 256, "fp4", "bf16", "fp4", 1, -1, -1, -1, -1, -1, -1, 0]
-    for idx, val in ((13, "fp8"), (15, "fp8"), (16, 2), (17, 64)):
+    for idx, val in ((13, "fp8"), (15, "fp8"), (17, 64)):
         args = list(base)
         args[idx] = val
         with pytest.raises(NotImplementedError):
@@ -123,3 +123,20 @@ def test_mxfp4_short_k_every_tile(K):
         for _ in range(3):
             acc = _run(d, M, N, K, force_path=1, tile=tile, acc=True)
             assert np.allclose(acc, want, rtol=1e-5, atol=1e-5 * np.abs(want).max()), f"tile {tile}"
+
+
+def test_mxfp4_strided_batched_default_strides():
+    # batch > 1 with the reference's default strides: contiguous [B,M,*] operands, one result slab per batch
+    from kernels.gemm.mxfp4_preshuffle import launch_gemm
+
+    B, M, N, K = 3, 40, 256, 512
+    dev = torch.device("cuda")
+    ds = [make_mxfp4(M, N, K, seed=20 + b) for b in range(B)]
+    cat = lambda k: torch.cat([d[k].reshape(-1) for d in ds]).to(dev)
+    a, w, sa, sb = cat("a_q"), cat("b_shuf"), cat("sa_shuf"), cat("sb_shuf")
+    c = torch.zeros(B, M, N, dtype=torch.bfloat16, device=dev)
+    launch_gemm(c, a, w, sa, sb, M, N, torch.cuda.current_stream(), N, K, 64, 128, 256, "fp4", "bf16", "fp4", B, -1, -1, -1, -1, -1, -1, 0, 0)
+    torch.cuda.synchronize()
+    for b, d in enumerate(ds):
+        ref = O.run_torch_w4(d["a_q"].numpy(), d["b_q"].numpy(), d["sa"].numpy(), d["sb"].numpy())
+        _check(c[b].float().cpu().numpy(), ref)
