@@ -111,7 +111,8 @@ def test_other_validation_errors():
 
 def test_mxfp4_entry_rejects_what_is_not_built():
     base = [0, 0, 0, 0, 0, 32, 128, None, 128, 256, 32, 128, 256, "fp4", "bf16", "fp4", 1, -1, -1, -1, -1, -1, -1, 0]
-    for idx, val, exc in ((13, "fp8", NotImplementedError), (15, "fp8", NotImplementedError),                           (17, 64, NotImplementedError), (12, 64, ValueError), (11, 64, ValueError), (14, "fp32", ValueError),
+    for idx, val, exc in ((13, "fp8", NotImplementedError), (15, "fp8", NotImplementedError), (16, 0, ValueError),
+                          (17, 64, NotImplementedError), (12, 64, ValueError), (11, 64, ValueError), (14, "fp32", ValueError),
                           (6, 256, ValueError)):
         args = list(base)
         args[idx] = val
