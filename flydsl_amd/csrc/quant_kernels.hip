@@ -144,59 +144,57 @@ __global__ void __launch_bounds__(256) k_quant_pertoken(const void* x, uint8_t* 
     }
 }
 
-__device__ __forceinline__ uint32_t e2m1_code(float y) {
-    const float a = fabsf(y);
-    uint32_t c = (a > 0.25f) + (a >= 0.75f) + (a > 1.25f) + (a >= 1.75f) + (a > 2.5f) + (a >= 3.5f) + (a > 5.0f);
-    return c | ((__builtin_bit_cast(uint32_t, y) >> 28) & 8u);
-}
-
-// one thread per 32-element block; rows in [M, R) (padding up to a multiple of 32 rows) get zero codes / scale 0
+// Four consecutive lanes share one 32-element block (8 elements each, so a wavefront reads fully coalesced 16- or
+// 32-byte pieces); the block maximum is combined with two lane exchanges.  Rows in [M, R) (padding up to a multiple
+// of 32 rows) get scale byte 0 and no codes.
 template <int XT>
 __global__ void __launch_bounds__(256) k_quant_mxfp4(const void* x, uint8_t* packed, uint8_t* scales, int M, int R, int K,
                                                       int shuffled) {
     const int KB = K >> 5;
-    const size_t blk = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (blk >= (size_t)R * KB) return;
-    const int r = (int)(blk / KB), kb = (int)(blk % KB);
-    float v[32];
+    const size_t piece = (size_t)blockIdx.x * 256 + threadIdx.x;  // 8-element piece index over R x K
+    const size_t blk = piece >> 2;
+    const int sub = (int)(piece & 3);
+    const bool live = blk < (size_t)R * KB;
+    const int r = live ? (int)(blk / KB) : 0, kb = live ? (int)(blk % KB) : 0;
+    float v[8];
     float amax = 0.0f;
-    if (r < M) {
+    if (live && r < M) {
+        load8<XT>(x, (size_t)r * K + (size_t)kb * 32 + sub * 8, v);
 #pragma unroll
-        for (int j = 0; j < 4; j++) load8<XT>(x, (size_t)r * K + (size_t)kb * 32 + j * 8, v + j * 8);
-#pragma unroll
-        for (int e = 0; e < 32; e++) amax = fmaxf(amax, fabsf(v[e]));   // fmaxf drops NaN like torch.amax does not: inputs are finite
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
     } else {
 #pragma unroll
-        for (int e = 0; e < 32; e++) v[e] = 0.0f;
+        for (int e = 0; e < 8; e++) v[e] = 0.0f;
     }
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    if (!live) return;
     // scale byte: biased exponent of amax/4, +1 when bit 22 is set and (lower mantissa bits or a normal exponent)
     const uint32_t u = __builtin_bit_cast(uint32_t, amax / 4.0f);
     uint32_t e = (u >> 23) & 0xFFu;
     const bool up = (u & 0x400000u) && ((u & 0x3FFFFFu) || e > 0);
-    if (e == 0xFFu) e = 0xFFu; else if (up) e = (e + 1) & 0xFFu;
-    const float sf = e == 0 ? __builtin_bit_cast(float, 0x00400000u) : (e == 0xFF ? __builtin_bit_cast(float, 0x7F800001u) : __builtin_bit_cast(float, e << 23));
+    if (e != 0xFFu && up) e = (e + 1) & 0xFFu;
+    const float sf = e == 0 ? __builtin_bit_cast(float, 0x00400000u)
+                            : (e == 0xFF ? __builtin_bit_cast(float, 0x7F800001u) : __builtin_bit_cast(float, e << 23));
     if (r < M) {
-        v4i o;
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            // v_cvt_scalef32_pk_fp4_f32: (a, b) / scale -> two e2m1 codes (a in the low nibble) into one byte of the word
-            unsigned word = 0;
-            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 0], v[w * 8 + 1], sf, 0);
-            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 2], v[w * 8 + 3], sf, 1);
-            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 4], v[w * 8 + 5], sf, 2);
-            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[w * 8 + 6], v[w * 8 + 7], sf, 3);
-            o[w] = (int)word;
+        // v_cvt_scalef32_pk_fp4_f32: (a, b) / scale -> two e2m1 codes (a in the low nibble) into one byte of the word
+        unsigned word = 0;
+        word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[0], v[1], sf, 0);
+        word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[2], v[3], sf, 1);
+        word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[4], v[5], sf, 2);
+        word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, v[6], v[7], sf, 3);
+        *reinterpret_cast<unsigned*>(packed + (size_t)r * (K >> 1) + (size_t)kb * 16 + sub * 4) = word;
+    }
+    if (sub == 0) {
+        size_t off;
+        if (shuffled) {
+            off = (size_t)(r >> 5) * (32u * (size_t)KB) + (size_t)(kb >> 3) * 256 + (size_t)(kb & 3) * 64 + (size_t)(r & 15) * 4 +
+                  (size_t)((kb & 7) >> 2) * 2 + (size_t)((r & 31) >> 4);
+        } else {
+            off = (size_t)r * KB + kb;
         }
-        *reinterpret_cast<v4i*>(packed + (size_t)r * (K >> 1) + (size_t)kb * 16) = o;
+        scales[off] = (uint8_t)e;
     }
-    size_t off;
-    if (shuffled) {
-        off = (size_t)(r >> 5) * (32u * (size_t)KB) + (size_t)(kb >> 3) * 256 + (size_t)(kb & 3) * 64 + (size_t)(r & 15) * 4 +
-              (size_t)((kb & 7) >> 2) * 2 + (size_t)((r & 31) >> 4);
-    } else {
-        off = (size_t)r * KB + kb;
-    }
-    scales[off] = (uint8_t)e;
 }
 
 }  // namespace
@@ -213,7 +211,7 @@ hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float*
 
 hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
                                   hipStream_t stream) {
-    const size_t blocks = ((size_t)R * (K / 32) + 255) / 256;
+    const size_t blocks = ((size_t)R * (K / 32) * 4 + 255) / 256;  // four threads per 32-element block
     if (x_dtype == X_F32) hipLaunchKernelGGL((k_quant_mxfp4<X_F32>), dim3(blocks), dim3(256), 0, stream, x, (uint8_t*)packed, (uint8_t*)scales, M, R, K, shuffled);
     else if (x_dtype == X_BF16) hipLaunchKernelGGL((k_quant_mxfp4<X_BF16>), dim3(blocks), dim3(256), 0, stream, x, (uint8_t*)packed, (uint8_t*)scales, M, R, K, shuffled);
     else if (x_dtype == X_F16) hipLaunchKernelGGL((k_quant_mxfp4<X_F16>), dim3(blocks), dim3(256), 0, stream, x, (uint8_t*)packed, (uint8_t*)scales, M, R, K, shuffled);

@@ -137,3 +137,21 @@ def test_quantiser_argument_errors():
         quant_device.per_1x32_f4_quant(torch.zeros(4, 64, device="cuda"), shuffle=True)  # K % 256 for the shuffled layout
     with pytest.raises(TypeError):
         quant_device.pertoken_quant(torch.zeros(4, 64, device="cuda", dtype=torch.float64))
+
+
+def test_quantisers_with_caller_owned_outputs():
+    from flydsl_amd import quant_device
+
+    x = _x(64, 512, seed=9, spread=False).cuda()
+    y = torch.empty(64, 512, dtype=torch.uint8, device="cuda")
+    s = torch.empty(64, dtype=torch.float32, device="cuda")
+    y2, s2 = quant_device.pertoken_quant(x, quant_dtype=torch.float8_e4m3fn, out=(y, s))
+    ref_y, ref_s = quant_device.pertoken_quant(x, quant_dtype=torch.float8_e4m3fn)
+    assert y2.data_ptr() == y.data_ptr() and torch.equal(y2.view(torch.uint8), ref_y.view(torch.uint8)) and torch.equal(s.view(-1, 1), ref_s)
+    p = torch.empty(64, 256, dtype=torch.uint8, device="cuda")
+    sc = torch.empty(64, 16, dtype=torch.uint8, device="cuda")
+    quant_device.per_1x32_f4_quant(x, shuffle=False, out=(p, sc))
+    rp, rs = quant_device.per_1x32_f4_quant(x, shuffle=False)
+    assert torch.equal(p, rp.view(torch.uint8)) and torch.equal(sc, rs.view(torch.uint8))
+    with pytest.raises(ValueError):
+        quant_device.pertoken_quant(x, out=(y[:10], s))
