@@ -92,3 +92,9 @@ def test_example_shape_fp16():
     ref = _ref(d)
     c = _launch(d, M, N, K, out_dtype="fp16")
     _check(c[:M].float().cpu().numpy(), ref)
+
+
+def test_usage_example_runs_and_is_correct():
+    from flydsl_amd.examples import preshuffle_gemm_fp16
+
+    assert preshuffle_gemm_fp16.main(M=1024, N=2048, K=4096, iters=3)
