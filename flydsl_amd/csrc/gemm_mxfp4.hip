@@ -37,10 +37,10 @@ __device__ __forceinline__ void store_mx4(const P& p, int store, size_t idx, v4f
 // ------------------------------------------------------------------------------------------------
 // small-M kernel: M <= 32; wavefront = (n-pair of 32 columns, K slice of 256-K steps)
 // ------------------------------------------------------------------------------------------------
-constexpr int NW = 8;
 constexpr int UNROLL = 2;
 
-template <int MB, int STORE>
+// NW = wavefronts per workgroup (4 or 8), as in the 8-bit streaming kernel
+template <int MB, int NW, int STORE>
 __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
     __shared__ __attribute__((aligned(16))) v4f red[NW][MB * 2][64];
 
@@ -139,18 +139,22 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
     }
 }
 
-template <int MB, int STORE>
+template <int MB, int NW, int STORE>
 hipError_t launch_smallm(const MxParams& p, hipStream_t stream) {
     const int npw = NW / p.ksplit;
     const int n_pairs = p.N / 32;
-    hipLaunchKernelGGL((k_mxfp4_smallm<MB, STORE>), dim3((n_pairs + npw - 1) / npw), dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((k_mxfp4_smallm<MB, NW, STORE>), dim3((n_pairs + npw - 1) / npw), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// requires 1 <= M <= 32 and p.ksplit in {1,2,4,8}
-hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream) {
-    if (p.M <= 16) return store == STORE_ACC ? launch_smallm<1, STORE_ACC>(p, stream) : launch_smallm<1, STORE_C>(p, stream);
-    return store == STORE_ACC ? launch_smallm<2, STORE_ACC>(p, stream) : launch_smallm<2, STORE_C>(p, stream);
+// requires 1 <= M <= 32, nw (wavefronts per workgroup) in {4,8} and p.ksplit a power of two <= nw
+hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream) {
+#define PSG_GO(MB_)                                                                                             \
+    if (nw == 4) return store == STORE_ACC ? launch_smallm<MB_, 4, STORE_ACC>(p, stream) : launch_smallm<MB_, 4, STORE_C>(p, stream); \
+    return store == STORE_ACC ? launch_smallm<MB_, 8, STORE_ACC>(p, stream) : launch_smallm<MB_, 8, STORE_C>(p, stream);
+    if (p.M <= 16) { PSG_GO(1) }
+    PSG_GO(2)
+#undef PSG_GO
 }

@@ -10,7 +10,7 @@
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, int nw, hipStream_t stream);
-hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, hipStream_t stream);
+hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
 hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float* scale, int M, int K, int out_fp8, hipStream_t stream);
 hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
@@ -262,8 +262,13 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
     if (small) {
-        p.ksplit = pick_ksplit(a->N / 32, a->K / 256);
-        e = psg_launch_mxfp4_smallm(p, store, static_cast<hipStream_t>(stream));
+        // four wavefronts x four K slices per workgroup when every slice still holds two 256-K steps, else eight
+        const int kt = a->K / 256;
+        const int nw = kt >= 8 ? 4 : 8;
+        p.ksplit = pick_ksplit(a->N / 32, kt);
+        if (p.ksplit > nw) p.ksplit = nw;
+        if (nw == 4 && p.ksplit < 4) p.ksplit = 4;
+        e = psg_launch_mxfp4_smallm(p, store, nw, static_cast<hipStream_t>(stream));
     } else {
         const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
         const Plan plan = plan_tiled(a->M, a->N, a->K / 2, true);
