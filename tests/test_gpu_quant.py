@@ -155,3 +155,21 @@ def test_quantisers_with_caller_owned_outputs():
     assert torch.equal(p, rp.view(torch.uint8)) and torch.equal(sc, rs.view(torch.uint8))
     with pytest.raises(ValueError):
         quant_device.pertoken_quant(x, out=(y[:10], s))
+
+
+@pytest.mark.parametrize("qd,kind", [(torch.int8, "int8"), (torch.float8_e4m3fn, "fp8")])
+def test_pertoken_quant_division_is_exact_over_many_values(qd, kind):
+    # 33 M quotients with row scales from 2^-80 to 2^80 (both the fast per-row-reciprocal path and the plain
+    # division for extreme rows), compared byte for byte with the oracle's IEEE division
+    from flydsl_amd import quant_device
+
+    g = torch.Generator().manual_seed(77)
+    m, k = 4096, 8192
+    x = torch.randn(m, k, generator=g) * torch.pow(2.0, torch.linspace(-80, 80, m)).view(-1, 1)
+    x[:, 0] = x.abs().amax(dim=1)  # make sure the row maximum is hit exactly once more
+    y, s = quant_device.pertoken_quant(x.cuda(), quant_dtype=qd)
+    want_y, want_s = O.pertoken_quant(x.numpy(), kind)
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    got = y.view(torch.uint8).cpu().numpy()
+    bad = np.argwhere(got != want_y.view(np.uint8))
+    assert len(bad) == 0, (len(bad), bad[:5].tolist())
