@@ -210,11 +210,18 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
         constexpr int HALF = MR / 2;
         constexpr int N_LOADS = 2 * NR + (KIND == KIND_MXFP4 ? MP + NP : 0);  // W fragments (+ scale dwords)
         constexpr int B_PER = (N_LOADS + HALF - 1) / HALF;
-        v4i flo[2], fhi[2];
-        read_frag(S, 0, flo[0], fhi[0]);
+        // A fragments are read FRAG_AHEAD m-blocks ahead of the MFMAs that use them (register ring buffer)
+        constexpr int FRAG_AHEAD = MR >= 4 ? 2 : 1;
+        constexpr int FRAG_BUFS = FRAG_AHEAD + 1;
+        v4i flo[FRAG_BUFS], fhi[FRAG_BUFS];
+        static_for<FRAG_AHEAD>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if constexpr (i < MR) read_frag(S, i, flo[i % FRAG_BUFS], fhi[i % FRAG_BUFS]);
+        });
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
-            if constexpr (mi + 1 < MR) read_frag(S, mi + 1, flo[(mi + 1) & 1], fhi[(mi + 1) & 1]);
+            if constexpr (mi + FRAG_AHEAD < MR)
+                read_frag(S, mi + FRAG_AHEAD, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
             if constexpr (mi < HALF) {
                 static_for<B_PER>([&](auto Q) {
                     constexpr int idx = mi * B_PER + decltype(Q)::value;
@@ -234,7 +241,7 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
             // keep the memory instructions above ahead of this block's MFMAs (the machine scheduler would
             // otherwise cluster them at the top of the step)
             __builtin_amdgcn_sched_barrier(0);
-            const v4i alo = flo[mi & 1], ahi = fhi[mi & 1];
+            const v4i alo = flo[mi % FRAG_BUFS], ahi = fhi[mi % FRAG_BUFS];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[S][ni], alo);
