@@ -27,6 +27,8 @@ EXPORTS = (
     "psg_gemm_mxfp4_acc",
     "psg_quant_pertoken",
     "psg_quant_mxfp4",
+    "psg_tile_coords",
+    "psg_debug_tile_order",
 )
 
 
@@ -98,6 +100,10 @@ def lib() -> ctypes.CDLL:
     handle.psg_last_error.restype = ctypes.c_char_p
     handle.psg_workspace_bytes.restype = ctypes.c_uint64
     handle.psg_workspace_bytes.argtypes = [ctypes.c_int32] * 4
+    handle.psg_tile_coords.restype = None
+    handle.psg_tile_coords.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
+    handle.psg_debug_tile_order.restype = ctypes.c_int
+    handle.psg_debug_tile_order.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
     for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
@@ -146,21 +152,82 @@ def stream_handle(stream) -> int:
     return int(h)
 
 
-_workspaces = {}
+class WorkspacePool:
+    """Scratch buffers of the split-K plan, one per (device, stream).
+
+    Launches on one stream are ordered, so they may share a buffer; launches on different streams get different
+    buffers and cannot race.  A buffer that has been handed out is never released while the process lives: a
+    recorded HIP graph or a launch still in flight may hold its address, and the launches go through ctypes, which
+    the caching allocator knows nothing about.  When a larger problem arrives a new buffer is allocated and the old
+    one is parked.  Allocation is refused while the stream is being captured into a graph: run the launcher once
+    before the capture (the reference's ``flyc.compile`` protocol does) so that the buffer exists."""
+
+    def __init__(self, alloc=None, capturing=None):
+        import threading
+
+        self._lock = threading.Lock()
+        self._live = {}     # (device index, stream handle) -> current buffer
+        self._parked = []   # outgrown buffers, kept alive on purpose
+        self._alloc = alloc
+        self._capturing = capturing
+
+    def get(self, device_index: int, stream: int, nbytes: int):
+        if nbytes <= 0:
+            return None
+        key = (int(device_index), int(stream))
+        with self._lock:
+            cur = self._live.get(key)
+            if cur is not None and cur.numel() >= nbytes:
+                return cur
+            if (self._capturing or _torch_capturing)():
+                raise RuntimeError(
+                    f"the split-K plan needs {nbytes} bytes of workspace on stream {stream:#x} but none that large exists "
+                    "yet, and allocating during graph capture is not possible; call the launcher once (or "
+                    "flyc.compile) on this stream before capturing")
+            new = (self._alloc or _torch_alloc)(int(nbytes), key[0])
+            if cur is not None:
+                self._parked.append(cur)
+            self._live[key] = new
+            return new
 
 
-def workspace(device, nbytes: int):
-    """Per-device scratch for the split-K path (one torch allocation, grown on demand, zero-size means none).
-    Growing allocates, so the first call for a new largest problem must happen outside graph capture -- which the
-    reference's own protocol guarantees (``flyc.compile`` runs the launcher once before any capture).  Launches
-    that may overlap on one device (different streams) must not rely on this shared buffer."""
+def _torch_capturing() -> bool:
+    import torch
+
+    return bool(torch.cuda.is_current_stream_capturing())
+
+
+def _torch_alloc(nbytes: int, device_index: int):
+    import torch
+
+    return torch.empty(nbytes, dtype=torch.uint8, device=f"cuda:{device_index}")
+
+
+_pool = WorkspacePool()
+
+
+def workspace(device, nbytes: int, stream=0):
+    """Scratch for the split-K path on ``device`` for launches on ``stream`` (raw handle); ``None`` when ``nbytes`` is 0."""
     import torch
 
     if nbytes <= 0:
         return None
-    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
-    cur = _workspaces.get(key)
-    if cur is None or cur.numel() < nbytes:
-        cur = torch.empty(int(nbytes), dtype=torch.uint8, device=f"cuda:{key}")
-        _workspaces[key] = cur
-    return cur
+    d = torch.device(device)
+    index = d.index if d.index is not None else torch.cuda.current_device()
+    return _pool.get(index, int(stream), int(nbytes))
+
+
+def check_operand(name, t, *, min_elems, elem_sizes, device=None):
+    """Cheap host-side validation of a tensor operand before its raw address reaches a kernel: device tensor,
+    contiguous, expected element size, at least ``min_elems`` elements.  Returns the tensor's device."""
+    if not getattr(t, "is_cuda", False):
+        raise ValueError(f"{name} must be a device (cuda) tensor, got {getattr(t, 'device', type(t).__name__)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if t.element_size() not in elem_sizes:
+        raise ValueError(f"{name} has {t.element_size()}-byte elements ({t.dtype}); expected {' or '.join(map(str, elem_sizes))}")
+    if t.numel() < min_elems:
+        raise ValueError(f"{name} holds {t.numel()} elements, this call needs at least {min_elems}")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name} is on {t.device}, the output is on {device}")
+    return t.device

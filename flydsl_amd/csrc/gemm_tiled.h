@@ -26,6 +26,7 @@
 //     group_m x tiles_n patch of tiles (A and B panels stay in that XCD's L2).
 #pragma once
 #include "psg_common.h"
+#include "tile_order.h"
 
 namespace {
 
@@ -69,17 +70,7 @@ __device__ __forceinline__ void mfma_mx(v4f& c, const v4i& a, const v4i& b, int 
 __device__ __forceinline__ int lds_off(int row, int kc) { return row * TK + ((kc ^ ((row >> 1) & 7)) << 4); }
 
 __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
-    const int num = tiles_m * tiles_n;
-    const int q = num >> 3, r = num & 7;
-    const int xcd = id & 7, in_xcd = id >> 3;
-    const int wg = xcd * q + (xcd < r ? xcd : r) + in_xcd;
-    const int per_group = group_m * tiles_n;
-    const int g = wg / per_group;
-    const int first_m = g * group_m;
-    const int size_m = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-    const int in_g = wg - g * per_group;
-    tm = first_m + in_g % size_m;
-    tn = in_g / size_m;
+    psg_tile_order(id, tiles_m, tiles_n, group_m, &tm, &tn);
 }
 
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept

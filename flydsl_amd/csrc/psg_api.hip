@@ -7,11 +7,13 @@
 #include <cstring>
 
 #include "psg_common.h"
+#include "tile_order.h"
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, int nw, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
+hipError_t psg_launch_tile_order(int tiles_m, int tiles_n, int group_m, int32_t* out, hipStream_t stream);
 hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float* scale, int M, int K, int out_fp8, hipStream_t stream);
 hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
                                   hipStream_t stream);
@@ -19,6 +21,7 @@ hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void
 namespace {
 
 thread_local char g_err[512] = "";
+
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -143,6 +146,7 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
         if (!is16 && !aligned(a->scale_a, 4)) return fail(PSG_E_ALIGN, "scale_a must be 4-byte aligned");
         if (a->epilogue != PSG_EPI_NONE && !aligned(a->bias, 8)) return fail(PSG_E_ALIGN, "bias must be 8-byte aligned");
     }
+    if (a->workspace && !aligned(a->workspace, 16)) return fail(PSG_E_ALIGN, "workspace must be 16-byte aligned");
     if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
     if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
     return 0;
@@ -228,6 +232,23 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) 
 int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
     if (int rc = validate_a8w8(args, false, nullptr)) return rc;
     return run_a8w8(args, args->c, STORE_C, stream);
+}
+
+void psg_tile_coords(int32_t id, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t* tm, int32_t* tn) {
+    int a = 0, b = 0;
+    psg_tile_order(id, tiles_m, tiles_n, group_m, &a, &b);
+    *tm = a;
+    *tn = b;
+}
+
+int psg_debug_tile_order(int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t* out, void* stream) {
+    if (!out) return fail(PSG_E_NULL, "out must be non-NULL");
+    if (tiles_m < 1 || tiles_n < 1 || group_m < 1 || (int64_t)tiles_m * tiles_n > (1 << 24))
+        return fail(PSG_E_SHAPE, "need tiles_m, tiles_n, group_m >= 1 and at most 2^24 tiles");
+    const hipError_t e = psg_launch_tile_order(tiles_m, tiles_n, group_m, out, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_debug_tile_order launch");
+    g_err[0] = 0;
+    return 0;
 }
 
 int psg_gemm_a8w8_acc(const psg_a8w8_args* args, void* acc, void* stream) {

@@ -82,6 +82,17 @@ def launch_gemm(
     # chunks of (K/256)*256 bytes each, C [B,M,N]
     chunk = (Kk // 256) * 256
     strides = (M * Nn * 2, M * (Kk // 2), Nn * (Kk // 2), ((M + 31) // 32) * chunk, (Nn // 32) * chunk)
+    B = int(batch)
+    chunks_m = (M + 31) // 32
+    # operands given as tensors are checked on the host (raw addresses cannot be): device, contiguity, extent
+    for name, t, need in (("c", arg_c, B * M * Nn * 2), ("a", arg_a, B * M * (Kk // 2)), ("b", arg_b, B * Nn * (Kk // 2)),
+                          ("scale_a", arg_scale_a, B * chunks_m * chunk), ("scale_b", arg_scale_b, B * (Nn // 32) * chunk)):
+        if hasattr(t, "data_ptr") and hasattr(t, "is_cuda") and not (name == "c" and _acc is not None):
+            if not t.is_cuda or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous device tensor")
+            if t.numel() * t.element_size() < need:
+                raise ValueError(f"{name} holds {t.numel() * t.element_size()} bytes, this call needs at least {need}")
+    h = _lib.stream_handle(stream)
     base = (None if _acc is not None else _addr(arg_c), _addr(arg_a), _addr(arg_b), _addr(arg_scale_a), _addr(arg_scale_b))
     lib = _lib.lib()
     for bz in range(int(batch)):
@@ -105,11 +116,11 @@ def launch_gemm(
         else:
             need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
         if need and _acc is None and hasattr(arg_c, "device"):
-            ws = _lib.workspace(arg_c.device, need)
+            ws = _lib.workspace(arg_c.device, need, h)
             args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         if _acc is None:
-            rc = lib.psg_gemm_mxfp4(ctypes.byref(args), _lib.stream_handle(stream))
+            rc = lib.psg_gemm_mxfp4(ctypes.byref(args), h)
         else:
-            rc = lib.psg_gemm_mxfp4_acc(ctypes.byref(args), _addr(_acc) + bz * M * Nn * 4, _lib.stream_handle(stream))
+            rc = lib.psg_gemm_mxfp4_acc(ctypes.byref(args), _addr(_acc) + bz * M * Nn * 4, h)
         if rc:
             _lib.check(rc, "psg_gemm_mxfp4")

@@ -18,7 +18,7 @@ from typing import Optional
 
 from ... import _lib
 
-_A_COPY_GRANULARITY = 256 * 16  # threads x bytes per load of the reference's A-tile copy
+_A_COPY_GRANULARITY = 4096  # the reference's rule for tile_m * tile_k * elem_bytes (256 threads x 16 bytes)
 
 
 def _validate(N, K, tile_m, tile_n, tile_k, in_dtype, out_dtype, epilogue, use_async_copy, lds_stage, preload):
@@ -34,14 +34,15 @@ def _validate(N, K, tile_m, tile_n, tile_k, in_dtype, out_dtype, epilogue, use_a
     if out_dtype not in _lib.OUT_DTYPE:
         raise ValueError(f"out_dtype must be bf16/fp16, got {out_dtype!r}")
     elem_bytes = 1 if in_dtype in ("fp8", "int8") else 2
-    # :188-196 -- the reference's A-tile copy must divide evenly over 256 threads x 16 bytes
+    # :188-196 -- the reference refuses A tiles that its 256-thread x 16-byte copy cannot cover evenly.  The native
+    # kernels choose their own tiling, but a configuration the reference rejects is rejected here too, so that code
+    # written against either behaves the same.
     a_tile_bytes = tile_m * tile_k * elem_bytes
     if a_tile_bytes % _A_COPY_GRANULARITY != 0:
         raise ValueError(
-            f"tile_m * tile_k * elem_bytes must be a multiple of {_A_COPY_GRANULARITY} "
-            f"(total_threads * a_load_bytes); got tile_m={tile_m}, tile_k={tile_k}, "
-            f"elem_bytes={elem_bytes} -> {a_tile_bytes} bytes, leaving "
-            f"{a_tile_bytes % _A_COPY_GRANULARITY} bytes of the A tile unloaded"
+            f"tile_m * tile_k * elem_bytes must be a multiple of {_A_COPY_GRANULARITY} (the reference's A-tile rule, "
+            f"kept for compatibility; the tile keywords are hints here); got tile_m={tile_m}, tile_k={tile_k}, "
+            f"elem_bytes={elem_bytes} -> {a_tile_bytes} bytes"
         )
     # :200-203
     if preload is not None:
@@ -79,54 +80,81 @@ class PreshuffleGemm:
         args.xcd_swizzle = int(xcd_swizzle)
         self._proto = args
 
-    def _fill(self, C, A, B, scale_a, scale_b, bias, M, N):
+    def _prepare(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, out_elem=2, epilogue=True):
+        """Validate the operands on the host and fill the C struct.  The kernels address C, the scales and the bias
+        without bounds (only A and W go through bounded descriptors), so everything that could send a store or a load
+        outside an allocation is refused here, before any launch."""
         if int(N) != self.N:
             raise ValueError(f"N={N} differs from the N={self.N} this launcher was built for")
+        M = int(M)
+        if M < 1 or M > 65536:
+            raise ValueError(f"M={M} outside [1, 65536]")
+        eb = 1 if self.in_dtype in ("fp8", "int8") else 2
+        dev = _lib.check_operand("C", C, min_elems=M * self.N, elem_sizes=(out_elem,))
+        _lib.check_operand("A", A, min_elems=M * self.K, elem_sizes=(eb,), device=dev)
+        _lib.check_operand("B", B, min_elems=self.N * self.K, elem_sizes=(eb,), device=dev)
+        if B.numel() != self.N * self.K:
+            raise ValueError(f"B holds {B.numel()} elements, the preshuffled weight of this launcher has exactly {self.N * self.K}")
+        has_scales = eb == 1 and epilogue
+        if has_scales:
+            if scale_a is None or scale_b is None:
+                raise ValueError("scale_a and scale_b are required for 8-bit inputs")
+            _lib.check_operand("scale_a", scale_a, min_elems=M, elem_sizes=(4,), device=dev)
+            _lib.check_operand("scale_b", scale_b, min_elems=self.N, elem_sizes=(4,), device=dev)
+        has_bias = epilogue and self.epilogue != "none"
+        if has_bias:
+            if bias is None:
+                raise ValueError(f"epilogue={self.epilogue!r} needs a bias tensor")
+            _lib.check_operand("bias", bias, min_elems=self.N, elem_sizes=(2,), device=dev)
         args = _lib.A8W8Args()
         ctypes.memmove(ctypes.byref(args), ctypes.byref(self._proto), ctypes.sizeof(args))
         args.c = C.data_ptr()
         args.a = A.data_ptr()
         args.b = B.data_ptr()
-        args.scale_a = scale_a.data_ptr() if scale_a is not None and scale_a.numel() else None
-        args.scale_b = scale_b.data_ptr() if scale_b is not None and scale_b.numel() else None
-        args.bias = bias.data_ptr() if bias is not None and bias.numel() else None
-        args.M = int(M)
-        need = self._lib.psg_workspace_bytes(args.M, self.N, self.K, args.in_dtype)
+        args.scale_a = scale_a.data_ptr() if has_scales else None
+        args.scale_b = scale_b.data_ptr() if has_scales else None
+        args.bias = bias.data_ptr() if has_bias else None
+        args.M = M
+        h = _lib.stream_handle(stream)
+        need = self._lib.psg_workspace_bytes(args.M, self.N, self.K, args.in_dtype) if epilogue else 0
         if need:
-            ws = _lib.workspace(C.device, need)
+            ws = _lib.workspace(dev, need, h)
             args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
-        return args
+        return args, h
+
+    def _fill(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
+        return self._prepare(C, A, B, scale_a, scale_b, bias, M, N, stream)[0]
 
     def __call__(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
-        args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
-        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
+        args, h = self._prepare(C, A, B, scale_a, scale_b, bias, M, N, stream)
+        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), h)
         if rc:
             _lib.check(rc, "psg_gemm_a8w8")
 
     def accumulators(self, acc, A, B, M, N, stream=None, force_path=0, tile=None, wave_layout=0):
         """Write the raw accumulators ``[M, N]`` (int32 for int8, fp32 for fp8) into ``acc``."""
-        args = self._fill(acc, A, B, None, None, None, M, N)
+        args, h = self._prepare(acc, A, B, None, None, None, M, N, stream, out_elem=4, epilogue=False)
         args.force_path = int(force_path)
         args.reserved = int(wave_layout)
         if tile is not None:
             args.tile_m, args.tile_n, args.tile_k = int(tile[0]), int(tile[1]), 1
-        rc = self._lib.psg_gemm_a8w8_acc(ctypes.byref(args), acc.data_ptr(), _lib.stream_handle(stream))
+        rc = self._lib.psg_gemm_a8w8_acc(ctypes.byref(args), acc.data_ptr(), h)
         if rc:
             _lib.check(rc, "psg_gemm_a8w8_acc")
 
     def launch_forced(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None, force_path=0, tile=None, wave_layout=0, splits=1):
         """Like ``__call__`` but pins the regime (1 = MFMA mainloop, 2 = small-M) and optionally the
         native tile ``(tile_m, tile_n)`` and the number of K splits; for tests and benchmarks."""
-        args = self._fill(C, A, B, scale_a, scale_b, bias, M, N)
+        args, h = self._prepare(C, A, B, scale_a, scale_b, bias, M, N, stream)
         args.force_path = int(force_path)
         args.reserved = int(wave_layout)
         if tile is not None:
             args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
             args.tile_k = int(splits)
             if splits > 1:
-                ws = _lib.workspace(C.device, int(splits) * int(M) * self.N * 4)
+                ws = _lib.workspace(C.device, int(splits) * int(M) * self.N * 4, h)
                 args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
-        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), _lib.stream_handle(stream))
+        rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), h)
         if rc:
             _lib.check(rc, "psg_gemm_a8w8")
 

@@ -21,6 +21,12 @@ def _x_code(x):
     return _X_DTYPE[x.dtype]
 
 
+def _check_out(x, *outs):
+    for t in outs:
+        if not t.is_cuda or t.device != x.device or not t.is_contiguous():
+            raise ValueError("out tensors must be contiguous and on the same device as x")
+
+
 def pertoken_quant(x: torch.Tensor, quant_dtype=torch.int8, stream=None, out=None):
     """Per-row symmetric quantisation on the device.  Returns ``(y [M,K] quant_dtype, scale [M,1] fp32)``.
     ``out=(y, scale)`` reuses caller-owned outputs (1-byte ``[M,K]`` and fp32 ``[M]`` / ``[M,1]``): no allocation, so the
@@ -38,6 +44,7 @@ def pertoken_quant(x: torch.Tensor, quant_dtype=torch.int8, stream=None, out=Non
         scale = torch.empty((m, 1), dtype=torch.float32, device=x.device)
     else:
         y, scale = out
+        _check_out(x, y, scale)
         if y.numel() != m * k or y.element_size() != 1 or scale.numel() != m or scale.dtype != torch.float32:
             raise ValueError("out must be (1-byte [M,K], fp32 [M]) tensors")
         y = y.view(torch.uint8)
@@ -57,6 +64,7 @@ def per_1x32_f4_quant(x: torch.Tensor, shuffle: bool = True, stream=None, out=No
         packed = torch.empty((m, k // 2), dtype=torch.uint8, device=x.device)
         scales = torch.empty((r, k // 32), dtype=torch.uint8, device=x.device)
     else:  # caller-owned outputs: no allocation, graph-capturable
+        _check_out(x, *out)
         packed, scales = (t.view(torch.uint8) for t in out)
         if packed.numel() != m * (k // 2) or scales.numel() != r * (k // 32):
             raise ValueError("out must be (packed [M,K/2], scales [ceil(M/32)*32, K/32]) byte tensors")

@@ -21,6 +21,9 @@
  *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm), fp4 x fp4, batch 1
  *   psg_gemm_mxfp4_acc  no counterpart: fp32 accumulators of the MXFP4 mainloop, for parity tests
  *   psg_workspace_bytes no counterpart (the reference's preshuffle GEMM has no split-K path)
+ *   psg_tile_coords     the workgroup-id -> tile remap xcd_remap_bx_by
+ *                       kernels/common/mma/mfma_preshuffle_pipeline.py:685-729 (host evaluation of the function the
+ *                       tiled kernel uses); psg_debug_tile_order runs the same function on the device
  *   psg_quant_pertoken  device version of the host quantiser tests/utils.py:29-73
  *   psg_quant_mxfp4     device version of tests/kernels/utils/gemm_common_utils.py:675-704 (+ :645-672)
  */
@@ -73,7 +76,9 @@ enum psg_error {
  *            psg_workspace_bytes() bytes, no initialisation needed.  May always be NULL/0: the library then
  *            runs the problem unsplit.  Two launches that may overlap in time must not share one workspace.
  *   tile_m/tile_n/tile_k, xcd_swizzle: the reference's tuning keywords; accepted as hints
- *            (0 = library's choice).  The library picks its own tiling per regime.
+ *            (0 = library's choice).  The library picks its own tiling per regime.  xcd_swizzle > 0 is the number
+ *            of M-tiles per group of the tile order (psg_tile_coords); 0, which switches the remap off in the
+ *            reference, here means the library's default group of 8 (results do not depend on the tile order).
  */
 typedef struct psg_a8w8_args {
     void *c;
@@ -132,6 +137,14 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype);
 
 /* C = epilogue((acc * scale_a[m]) * scale_b[n]) on `stream` (a hipStream_t passed as void*). */
 int psg_gemm_a8w8(const psg_a8w8_args *args, void *stream);
+
+/* Tile (tm, tn) that workgroup `id` of a tiles_m x tiles_n launch of the tiled kernel works on, groups of `group_m`
+ * M-tiles; the reference's xcd_remap_bx_by with linear id = bx*gx + by, gx = tiles_n, gy = tiles_m,
+ * xcd_swizzle = group_m (kernels/common/mma/mfma_preshuffle_pipeline.py:685-729).  Host function, no GPU needed. */
+void psg_tile_coords(int32_t id, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t *tm, int32_t *tn);
+
+/* Evaluates the same function on the device for every id: out[2*id] = tm, out[2*id+1] = tn (int32 [tiles_m*tiles_n*2]). */
+int psg_debug_tile_order(int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t *out, void *stream);
 
 /* Same mainloop, but writes the raw accumulators [M,N] (int32 for int8, fp32 for fp8) to `acc`
  * instead of C.  c, scale_a, scale_b, bias are ignored. */

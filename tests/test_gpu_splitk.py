@@ -122,3 +122,46 @@ def test_mxfp4_splitk():
         torch.cuda.synchronize()
         ok, ratio = O.within_north_star_tolerance(c.float().cpu().numpy(), ref)
         assert ok, (splits, ratio)
+
+
+def test_two_streams_take_the_split_plan_without_sharing_a_workspace():
+    """Two launchers on two streams, both on the split-K plan, enqueued back to back so that they may overlap: each
+    stream has its own workspace, so both int8 results stay bit-exact."""
+    from flydsl_amd import _lib
+
+    M, N, K = 64, 2048, 8192
+    assert _lib.lib().psg_workspace_bytes(M, N, K, 0) > 0
+    dev = torch.device("cuda")
+    bias = torch.empty(0, dtype=torch.bfloat16, device=dev)
+    work = []
+    for seed in (11, 12):
+        d = make_a8w8(M, N, K, "int8", seed=seed)
+        t = {k: d[k].to(dev) for k in ("a_q", "b_shuf", "sa", "sb")}
+        ref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")["c_bf16_bits"]
+        work.append((t, ref, torch.zeros(M, N, dtype=torch.bfloat16, device=dev), torch.cuda.Stream(), _fn("int8", N, K)))
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for t, ref, c, s, fn in work:
+            fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s)
+    torch.cuda.synchronize()
+    h0, h1 = (_lib.stream_handle(w[3]) for w in work)
+    assert _lib._pool._live[(torch.cuda.current_device(), h0)] is not _lib._pool._live[(torch.cuda.current_device(), h1)]
+    for t, ref, c, s, fn in work:
+        assert np.array_equal(bf16_bits(c), ref)
+
+
+def test_workspace_growth_during_capture_is_refused():
+    M, N, K = 128, 1024, 8192
+    d = make_a8w8(M, N, K, "int8", seed=3)
+    dev = torch.device("cuda")
+    t = {k: d[k].to(dev) for k in ("a_q", "b_shuf", "sa", "sb")}
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    bias = torch.empty(0, dtype=torch.bfloat16, device=dev)
+    fn = _fn("int8", N, K)
+    s = torch.cuda.Stream()  # a stream that has no workspace yet
+    s.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="graph capture"):
+        with torch.cuda.graph(g, stream=s):
+            fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, torch.cuda.current_stream())
+    torch.cuda.synchronize()

@@ -123,7 +123,7 @@ def test_mxfp4_entry_rejects_what_is_not_built():
 # ---- the C ABI -------------------------------------------------------------------------------------
 def _declared_functions():
     text = open(HEADER).read()
-    return sorted(set(re.findall(r"^\s*(?:int|uint64_t|const char \*)\s*\**\s*(psg_\w+)\s*\(", text, flags=re.M)))
+    return sorted(set(re.findall(r"^\s*(?:int|void|uint64_t|const char \*)\s*\**\s*(psg_\w+)\s*\(", text, flags=re.M)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -134,6 +134,111 @@ def test_library_exports_every_declared_symbol():
         assert getattr(handle, n) is not None
     assert handle.psg_abi_version() == _lib.ABI_VERSION
     assert handle.psg_workspace_bytes(16, 6144, 4096, 1) == 0
+
+
+def test_tile_order_equals_the_oracle_remap_on_every_id():
+    """The function the tiled kernel uses to turn a workgroup id into a tile (evaluated on the host through the C ABI)
+    against the oracle's xcd_remap_bx_by, id by id, incl. ragged grids: tiles % 8 != 0, tiles_m % group_m != 0."""
+    from oracle import psg_oracle as O
+
+    handle = _lib.lib()
+    tm, tn = ctypes.c_int32(), ctypes.c_int32()
+    for tiles_m, tiles_n, group_m in [(32, 16, 8), (3, 4, 2), (7, 5, 3), (1, 13, 8), (13, 1, 4), (17, 9, 16), (64, 112, 8),
+                                      (5, 5, 1), (2, 3, 8), (9, 7, 4)]:
+        seen = set()
+        for bx in range(tiles_m):
+            for by in range(tiles_n):
+                lin = bx * tiles_n + by
+                handle.psg_tile_coords(lin, tiles_m, tiles_n, group_m, ctypes.byref(tm), ctypes.byref(tn))
+                want = O.xcd_remap_bx_by(bx, by, tiles_m * 16, tile_m=16, tile_n=64, n=tiles_n * 64, xcd_swizzle=group_m)
+                assert (tm.value, tn.value) == want, (tiles_m, tiles_n, group_m, bx, by)
+                seen.add(want)
+        assert len(seen) == tiles_m * tiles_n  # a bijection onto the tile grid
+
+
+def test_workspace_pool_never_releases_a_buffer_it_handed_out():
+    class Buf:
+        def __init__(self, n, dev):
+            self.n, self.dev = n, dev
+
+        def numel(self):
+            return self.n
+
+    made = []
+
+    def alloc(n, dev):
+        made.append(Buf(n, dev))
+        return made[-1]
+
+    capturing = [False]
+    pool = _lib.WorkspacePool(alloc=alloc, capturing=lambda: capturing[0])
+    a = pool.get(0, 0x10, 1000)
+    assert pool.get(0, 0x10, 500) is a and pool.get(0, 0x10, 1000) is a  # reuse while it is large enough
+    b = pool.get(0, 0x20, 1000)
+    assert b is not a  # another stream never shares
+    c = pool.get(1, 0x10, 1000)
+    assert c is not a and c.dev == 1  # nor another device
+    d = pool.get(0, 0x10, 4000)  # growth: a new buffer, the old one is parked, not dropped
+    assert d is not a and a in pool._parked and len(made) == 4
+    assert pool.get(0, 0x10, 0) is None
+    capturing[0] = True
+    assert pool.get(0, 0x10, 4000) is d  # an existing buffer may be used during capture
+    with pytest.raises(RuntimeError, match="graph capture"):
+        pool.get(0, 0x10, 8000)  # but growth during capture is refused
+    with pytest.raises(RuntimeError, match="graph capture"):
+        pool.get(0, 0x30, 10)
+    assert len(made) == 4
+
+
+def test_launchers_refuse_operands_that_would_send_a_kernel_out_of_bounds():
+    """Host-side checks before any launch (no GPU needed: every case fails on the first check it reaches)."""
+    fn = compile_preshuffle_gemm(N=64, K=128, tile_m=32, tile_n=64, tile_k=128, in_dtype="int8")
+    cpu = dict(c=torch.zeros(4, 64, dtype=torch.bfloat16), a=torch.zeros(4, 128, dtype=torch.int8),
+               b=torch.zeros(64, 128, dtype=torch.int8), sa=torch.zeros(4), sb=torch.zeros(64))
+    with pytest.raises(ValueError, match="device"):
+        fn(cpu["c"], cpu["a"], cpu["b"], cpu["sa"], cpu["sb"], None, 4, 64, 0)
+    with pytest.raises(ValueError, match="N=32 differs"):
+        fn(cpu["c"], cpu["a"], cpu["b"], cpu["sa"], cpu["sb"], None, 4, 32, 0)
+    with pytest.raises(ValueError, match="outside"):
+        fn(cpu["c"], cpu["a"], cpu["b"], cpu["sa"], cpu["sb"], None, 0, 64, 0)
+
+    class Fake:  # stands in for a device tensor
+        def __init__(self, numel, esize, contiguous=True, device="cuda:0"):
+            self._n, self._e, self._c, self.device, self.is_cuda, self.dtype = numel, esize, contiguous, device, True, "fake"
+
+        def numel(self):
+            return self._n
+
+        def element_size(self):
+            return self._e
+
+        def is_contiguous(self):
+            return self._c
+
+        def data_ptr(self):
+            raise AssertionError("the address must not be read before validation passed")
+
+    good = dict(C=Fake(4 * 64, 2), A=Fake(4 * 128, 1), B=Fake(64 * 128, 1), sa=Fake(4, 4), sb=Fake(64, 4))
+    for key, bad, msg in [("C", Fake(4 * 64 - 1, 2), "at least"), ("C", Fake(4 * 64, 4), "2"), ("A", Fake(3 * 128, 1), "at least"),
+                          ("A", Fake(4 * 128, 1, contiguous=False), "contiguous"), ("B", Fake(64 * 128 + 16, 1), "exactly"),
+                          ("sa", Fake(3, 4), "at least"), ("sb", Fake(64, 2), "4"), ("A", Fake(4 * 128, 1, device="cuda:1"), "is on")]:
+        ops = dict(good)
+        ops[key] = bad
+        with pytest.raises(ValueError, match=msg):
+            fn(ops["C"], ops["A"], ops["B"], ops["sa"], ops["sb"], None, 4, 64, 0)
+    fnb = compile_preshuffle_gemm(N=64, K=128, tile_m=32, tile_n=64, tile_k=128, in_dtype="int8", epilogue="bias")
+    with pytest.raises(ValueError, match="bias"):
+        fnb(good["C"], good["A"], good["B"], good["sa"], good["sb"], None, 4, 64, 0)
+    with pytest.raises(ValueError, match="at least"):
+        fnb(good["C"], good["A"], good["B"], good["sa"], good["sb"], Fake(63, 2), 4, 64, 0)
+    # the C ABI refuses a misaligned workspace
+    handle = _lib.lib()
+    args = _lib.A8W8Args()
+    args.a = args.b = args.c = args.scale_a = args.scale_b = 0x1000
+    args.M, args.N, args.K, args.in_dtype = 64, 64, 128, 0
+    args.workspace, args.workspace_bytes = 0x2004, 1 << 20
+    assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -6
+    assert b"workspace" in handle.psg_last_error()
 
 
 def test_struct_layouts_match_header():

@@ -106,3 +106,19 @@ def test_xcd_remap_is_a_bijection():
                 seen.add(nb)
         assert len(seen) == gx * gy
     assert O.xcd_remap_bx_by(3, 5, 100, tile_m=16, tile_n=64, n=1024, xcd_swizzle=0) == (3, 5)
+
+
+def test_xcd_remap_known_answers():
+    """Worked by hand from the reference's formula (kernels/common/mma/mfma_preshuffle_pipeline.py:685-729) for
+    M=768, N=1024, 256x256 tiles (gy=3 M-tiles, gx=4 N-tiles, 12 workgroups: q=1, r=4) and xcd_swizzle=2:
+      (bx,by) -> linear -> (xcd, in_xcd) -> wgid -> group / in_group -> (bx', by')
+      (0,0) -> 0  -> (0,0) -> 0        -> 0 / 0  -> (0,0)
+      (0,1) -> 1  -> (1,0) -> 1+1=2    -> 0 / 2  -> (0,1)
+      (1,1) -> 5  -> (5,0) -> 5+4=9    -> 1 / 1, last group holds 1 M-tile -> (2,1)
+      (2,1) -> 9  -> (1,1) -> 1+1+1=3  -> 0 / 3  -> (1,1)
+      (2,3) -> 11 -> (3,1) -> 3+3+1=7  -> 0 / 7  -> (1,3)
+      (1,3) -> 7  -> (7,0) -> 7+4=11   -> 1 / 3  -> (2,3)
+    A transposed (bx,by), a dropped remainder term or a row-major walk inside the group each break one of these."""
+    kw = dict(tile_m=256, tile_n=256, n=1024, xcd_swizzle=2)
+    for (bx, by), want in {(0, 0): (0, 0), (0, 1): (0, 1), (1, 1): (2, 1), (2, 1): (1, 1), (2, 3): (1, 3), (1, 3): (2, 3)}.items():
+        assert O.xcd_remap_bx_by(bx, by, 768, **kw) == want, (bx, by)
