@@ -153,38 +153,44 @@ def stream_handle(stream) -> int:
 
 
 class WorkspacePool:
-    """Scratch buffers of the split-K plan, one per (device, stream).
+    """Scratch buffers of the split-K plan, one per (owner, device, stream); an owner is one launcher object.
 
-    Launches on one stream are ordered, so they may share a buffer; launches on different streams get different
-    buffers and cannot race.  A buffer that has been handed out is never released while the process lives: a
-    recorded HIP graph or a launch still in flight may hold its address, and the launches go through ctypes, which
-    the caching allocator knows nothing about.  When a larger problem arrives a new buffer is allocated and the old
-    one is parked.  Allocation is refused while the stream is being captured into a graph: run the launcher once
-    before the capture (the reference's ``flyc.compile`` protocol does) so that the buffer exists."""
+    Launches on one stream are ordered, so they may share a buffer; launches on different streams, or through
+    different launchers, get different buffers and cannot race.  A buffer that has been handed out is never released
+    while the process lives: a recorded HIP graph or a launch still in flight may hold its address, and the launches
+    go through ctypes, which the caching allocator knows nothing about.  When a larger problem arrives a new buffer is
+    allocated and the old one is parked.  Nothing is allocated while the stream is being captured into a graph: a
+    capture on a stream that has no buffer yet borrows the buffer the same launcher got on another stream of that
+    device (the warm-up run the reference's ``flyc.compile`` protocol makes before any capture), so replays of that
+    graph must not overlap with launches of the same launcher on the warm-up stream; if there is none the call
+    raises."""
 
     def __init__(self, alloc=None, capturing=None):
         import threading
 
         self._lock = threading.Lock()
-        self._live = {}     # (device index, stream handle) -> current buffer
+        self._live = {}     # (owner, device index, stream handle) -> current buffer
         self._parked = []   # outgrown buffers, kept alive on purpose
         self._alloc = alloc
         self._capturing = capturing
 
-    def get(self, device_index: int, stream: int, nbytes: int):
+    def get(self, owner, device_index: int, stream: int, nbytes: int):
         if nbytes <= 0:
             return None
-        key = (int(device_index), int(stream))
+        key = (owner, int(device_index), int(stream))
         with self._lock:
             cur = self._live.get(key)
             if cur is not None and cur.numel() >= nbytes:
                 return cur
             if (self._capturing or _torch_capturing)():
+                for (o, d, _), buf in self._live.items():
+                    if o == owner and d == key[1] and buf.numel() >= nbytes:
+                        return buf
                 raise RuntimeError(
-                    f"the split-K plan needs {nbytes} bytes of workspace on stream {stream:#x} but none that large exists "
-                    "yet, and allocating during graph capture is not possible; call the launcher once (or "
-                    "flyc.compile) on this stream before capturing")
-            new = (self._alloc or _torch_alloc)(int(nbytes), key[0])
+                    f"the split-K plan needs {nbytes} bytes of workspace but this launcher has none that large on device "
+                    f"{key[1]} yet, and allocating during graph capture is not possible; call the launcher once (or "
+                    "flyc.compile) before capturing")
+            new = (self._alloc or _torch_alloc)(int(nbytes), key[1])
             if cur is not None:
                 self._parked.append(cur)
             self._live[key] = new
@@ -206,15 +212,16 @@ def _torch_alloc(nbytes: int, device_index: int):
 _pool = WorkspacePool()
 
 
-def workspace(device, nbytes: int, stream=0):
-    """Scratch for the split-K path on ``device`` for launches on ``stream`` (raw handle); ``None`` when ``nbytes`` is 0."""
+def workspace(device, nbytes: int, stream=0, owner="shared"):
+    """Scratch for the split-K path of launcher ``owner`` on ``device`` for launches on ``stream`` (raw handle);
+    ``None`` when ``nbytes`` is 0."""
     import torch
 
     if nbytes <= 0:
         return None
     d = torch.device(device)
     index = d.index if d.index is not None else torch.cuda.current_device()
-    return _pool.get(index, int(stream), int(nbytes))
+    return _pool.get(owner, index, int(stream), int(nbytes))
 
 
 def check_operand(name, t, *, min_elems, elem_sizes, device=None):

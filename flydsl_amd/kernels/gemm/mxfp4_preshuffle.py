@@ -116,7 +116,7 @@ def launch_gemm(
         else:
             need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
         if need and _acc is None and hasattr(arg_c, "device"):
-            ws = _lib.workspace(arg_c.device, need, h)
+            ws = _lib.workspace(arg_c.device, need, h, owner="mxfp4")
             args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         if _acc is None:
             rc = lib.psg_gemm_mxfp4(ctypes.byref(args), h)

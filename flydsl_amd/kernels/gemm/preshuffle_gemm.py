@@ -118,7 +118,7 @@ class PreshuffleGemm:
         h = _lib.stream_handle(stream)
         need = self._lib.psg_workspace_bytes(args.M, self.N, self.K, args.in_dtype) if epilogue else 0
         if need:
-            ws = _lib.workspace(dev, need, h)
+            ws = _lib.workspace(dev, need, h, owner=id(self))
             args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         return args, h
 
@@ -152,7 +152,7 @@ class PreshuffleGemm:
             args.tile_m, args.tile_n = int(tile[0]), int(tile[1])
             args.tile_k = int(splits)
             if splits > 1:
-                ws = _lib.workspace(C.device, int(splits) * int(M) * self.N * 4, h)
+                ws = _lib.workspace(C.device, int(splits) * int(M) * self.N * 4, h, owner=id(self))
                 args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
         rc = self._lib.psg_gemm_a8w8(ctypes.byref(args), h)
         if rc:

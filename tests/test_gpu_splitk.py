@@ -144,8 +144,17 @@ def test_two_streams_take_the_split_plan_without_sharing_a_workspace():
         for t, ref, c, s, fn in work:
             fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s)
     torch.cuda.synchronize()
-    h0, h1 = (_lib.stream_handle(w[3]) for w in work)
-    assert _lib._pool._live[(torch.cuda.current_device(), h0)] is not _lib._pool._live[(torch.cuda.current_device(), h1)]
+    bufs = [_lib._pool._live[(id(w[4]), torch.cuda.current_device(), _lib.stream_handle(w[3]))] for w in work]
+    assert bufs[0] is not bufs[1]
+    # one launcher on two streams: separate buffers as well
+    t, ref, c, s, fn = work[0]
+    c2 = torch.zeros_like(c)
+    s2 = torch.cuda.Stream()
+    fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s)
+    fn(c2, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s2)
+    torch.cuda.synchronize()
+    assert _lib._pool._live[(id(fn), torch.cuda.current_device(), _lib.stream_handle(s2))] is not bufs[0]
+    assert np.array_equal(bf16_bits(c2), ref)
     for t, ref, c, s, fn in work:
         assert np.array_equal(bf16_bits(c), ref)
 
@@ -157,8 +166,8 @@ def test_workspace_growth_during_capture_is_refused():
     t = {k: d[k].to(dev) for k in ("a_q", "b_shuf", "sa", "sb")}
     c = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
     bias = torch.empty(0, dtype=torch.bfloat16, device=dev)
-    fn = _fn("int8", N, K)
-    s = torch.cuda.Stream()  # a stream that has no workspace yet
+    fn = _fn("int8", N, K)  # a launcher that has no workspace yet
+    s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())
     g = torch.cuda.CUDAGraph()
     with pytest.raises(RuntimeError, match="graph capture"):

@@ -172,22 +172,27 @@ def test_workspace_pool_never_releases_a_buffer_it_handed_out():
 
     capturing = [False]
     pool = _lib.WorkspacePool(alloc=alloc, capturing=lambda: capturing[0])
-    a = pool.get(0, 0x10, 1000)
-    assert pool.get(0, 0x10, 500) is a and pool.get(0, 0x10, 1000) is a  # reuse while it is large enough
-    b = pool.get(0, 0x20, 1000)
+    a = pool.get("L1", 0, 0x10, 1000)
+    assert pool.get("L1", 0, 0x10, 500) is a and pool.get("L1", 0, 0x10, 1000) is a  # reuse while it is large enough
+    b = pool.get("L1", 0, 0x20, 1000)
     assert b is not a  # another stream never shares
-    c = pool.get(1, 0x10, 1000)
+    c = pool.get("L1", 1, 0x10, 1000)
     assert c is not a and c.dev == 1  # nor another device
-    d = pool.get(0, 0x10, 4000)  # growth: a new buffer, the old one is parked, not dropped
-    assert d is not a and a in pool._parked and len(made) == 4
-    assert pool.get(0, 0x10, 0) is None
+    e = pool.get("L2", 0, 0x10, 1000)
+    assert e is not a  # nor another launcher
+    d = pool.get("L1", 0, 0x10, 4000)  # growth: a new buffer, the old one is parked, not dropped
+    assert d is not a and a in pool._parked and len(made) == 5
+    assert pool.get("L1", 0, 0x10, 0) is None
     capturing[0] = True
-    assert pool.get(0, 0x10, 4000) is d  # an existing buffer may be used during capture
+    assert pool.get("L1", 0, 0x10, 4000) is d  # an existing buffer may be used during capture
+    assert pool.get("L1", 0, 0x30, 4000) is d  # a capture stream borrows the launcher's warm-up buffer on that device
     with pytest.raises(RuntimeError, match="graph capture"):
-        pool.get(0, 0x10, 8000)  # but growth during capture is refused
+        pool.get("L1", 0, 0x10, 8000)  # growth during capture is refused
     with pytest.raises(RuntimeError, match="graph capture"):
-        pool.get(0, 0x30, 10)
-    assert len(made) == 4
+        pool.get("L3", 0, 0x30, 10)  # and so is a first allocation
+    with pytest.raises(RuntimeError, match="graph capture"):
+        pool.get("L1", 1, 0x30, 2000)  # another device's buffer is never borrowed
+    assert len(made) == 5
 
 
 def test_launchers_refuse_operands_that_would_send_a_kernel_out_of_bounds():
