@@ -27,6 +27,9 @@ EXPORTS = (
     "psg_gemm_mxfp4_acc",
     "psg_quant_pertoken",
     "psg_quant_mxfp4",
+    "psg_init",
+    "psg_static_scratch_bytes",
+    "psg_gemm_a8w8_static",
     "psg_tile_coords",
     "psg_debug_tile_order",
 )
@@ -100,11 +103,15 @@ def lib() -> ctypes.CDLL:
     handle.psg_last_error.restype = ctypes.c_char_p
     handle.psg_workspace_bytes.restype = ctypes.c_uint64
     handle.psg_workspace_bytes.argtypes = [ctypes.c_int32] * 4
+    handle.psg_init.restype = ctypes.c_int
+    handle.psg_init.argtypes = []
+    handle.psg_static_scratch_bytes.restype = ctypes.c_uint64
+    handle.psg_static_scratch_bytes.argtypes = []
     handle.psg_tile_coords.restype = None
     handle.psg_tile_coords.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
     handle.psg_debug_tile_order.restype = ctypes.c_int
     handle.psg_debug_tile_order.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
-    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4"):
+    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]

@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "psg_common.h"
 #include "tile_order.h"
@@ -18,10 +19,20 @@ hipError_t psg_launch_quant_pertoken(const void* x, int x_dtype, void* y, float*
 hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void* scales, int M, int R, int K, int shuffled,
                                   hipStream_t stream);
 
+// Scratch of the entry point that allocates nothing (psg_gemm_a8w8_static): the split-K partial sums of the tiled
+// path live here instead of in a caller-supplied workspace.  Every GPU the library runs on holds its own copy of the
+// array at its own address until the process ends.  In host code the name below is only a stand-in for the symbol:
+// the device address is looked up once per device with hipGetSymbolAddress and that pointer is what kernels get.
+#define PSG_STATIC_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char scratch[PSG_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
 
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, filled on first use
+std::mutex g_scratch_mu;
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -152,6 +163,24 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
     return 0;
 }
 
+// Device address of `scratch` on the current device (looked up once per device, then cached).
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(PSG_E_UNSUPPORTED, "device index %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!ptr) return fail(PSG_E_WORKSPACE, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     A8W8Params p{};
     p.c = out;
@@ -232,6 +261,37 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) 
 int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
     if (int rc = validate_a8w8(args, false, nullptr)) return rc;
     return run_a8w8(args, args->c, STORE_C, stream);
+}
+
+int psg_init(void) {
+    void* ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    g_err[0] = 0;
+    return 0;
+}
+
+uint64_t psg_static_scratch_bytes(void) { return PSG_STATIC_SCRATCH_BYTES; }
+
+int psg_gemm_a8w8_static(const psg_a8w8_args* args, void* stream) {
+    if (int rc = validate_a8w8(args, false, nullptr)) return rc;
+    // what the same problem's plan would want as workspace; forced tiles take their split count from tile_k
+    uint64_t need = psg_workspace_bytes(args->M, args->N, args->K, args->in_dtype);
+    if (args->force_path == 1 && args->tile_m > 0 && args->tile_n > 0)
+        need = splitk_bytes(args->M, args->N, args->tile_k >= 1 && args->tile_k <= 16 ? args->tile_k : 1);
+    if (args->force_path == 2 || (args->force_path == 0 && args->M <= kSmallM)) need = 0;
+    if (need > PSG_STATIC_SCRATCH_BYTES)
+        return fail(PSG_E_WORKSPACE, "this problem's split-K plan needs %llu bytes of scratch, the static scratch holds %u; use "
+                    "psg_gemm_a8w8 with a caller workspace", (unsigned long long)need, PSG_STATIC_SCRATCH_BYTES);
+    psg_a8w8_args local = *args;
+    local.workspace = nullptr;
+    local.workspace_bytes = 0;
+    if (need) {
+        void* ptr = nullptr;
+        if (int rc = static_scratch(&ptr)) return rc;
+        local.workspace = ptr;  // the per-device address, never the symbol's host-side name
+        local.workspace_bytes = PSG_STATIC_SCRATCH_BYTES;
+    }
+    return run_a8w8(&local, local.c, STORE_C, stream);
 }
 
 void psg_tile_coords(int32_t id, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t* tm, int32_t* tn) {

@@ -131,6 +131,15 @@ class PreshuffleGemm:
         if rc:
             _lib.check(rc, "psg_gemm_a8w8")
 
+    def launch_static(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
+        """Same result through ``psg_gemm_a8w8_static``: the entry point that allocates nothing (its split-K partial
+        sums live in a scratch array inside the library's device image)."""
+        args, h = self._prepare(C, A, B, scale_a, scale_b, bias, M, N, stream)
+        args.workspace, args.workspace_bytes = None, 0
+        rc = self._lib.psg_gemm_a8w8_static(ctypes.byref(args), h)
+        if rc:
+            _lib.check(rc, "psg_gemm_a8w8_static")
+
     def accumulators(self, acc, A, B, M, N, stream=None, force_path=0, tile=None, wave_layout=0):
         """Write the raw accumulators ``[M, N]`` (int32 for int8, fp32 for fp8) into ``acc``."""
         args, h = self._prepare(acc, A, B, None, None, None, M, N, stream, out_elem=4, epilogue=False)

@@ -24,6 +24,8 @@
  *   psg_tile_coords     the workgroup-id -> tile remap xcd_remap_bx_by
  *                       kernels/common/mma/mfma_preshuffle_pipeline.py:685-729 (host evaluation of the function the
  *                       tiled kernel uses); psg_debug_tile_order runs the same function on the device
+ *   psg_gemm_a8w8_static, psg_init, psg_static_scratch_bytes
+ *                       no counterpart in the reference: for callers that cannot allocate (see below)
  *   psg_quant_pertoken  device version of the host quantiser tests/utils.py:29-73
  *   psg_quant_mxfp4     device version of tests/kernels/utils/gemm_common_utils.py:675-704 (+ :645-672)
  */
@@ -137,6 +139,23 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype);
 
 /* C = epilogue((acc * scale_a[m]) * scale_b[n]) on `stream` (a hipStream_t passed as void*). */
 int psg_gemm_a8w8(const psg_a8w8_args *args, void *stream);
+
+/*
+ * psg_gemm_a8w8 for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  It computes exactly what
+ * psg_gemm_a8w8 computes (same plan, same kernels, same bits) but ignores args->workspace: the split-K partial sums
+ * go to a scratch array that is part of the library's device image (psg_static_scratch_bytes() bytes, 32 MiB, one
+ * copy per GPU, held until the process ends).  The call allocates and frees nothing.  A problem whose split-K plan
+ * wants more than that is rejected with PSG_E_WORKSPACE (use psg_gemm_a8w8 with a caller workspace, or none).
+ * All calls on one GPU share that GPU's array: two calls that may overlap in time on one GPU (different streams)
+ * race; calls on one stream, or ordered by events, are safe.  Nothing needs clearing between calls: every partial
+ * that is read was written by the same call.
+ * psg_init() looks up the array's device address for the current device (otherwise done by the first call on that
+ * device); call it once per device before a graph capture that records psg_gemm_a8w8_static.
+ */
+int psg_init(void);
+uint64_t psg_static_scratch_bytes(void);
+int psg_gemm_a8w8_static(const psg_a8w8_args *args, void *stream);
 
 /* Tile (tm, tn) that workgroup `id` of a tiles_m x tiles_n launch of the tiled kernel works on, groups of `group_m`
  * M-tiles; the reference's xcd_remap_bx_by with linear id = bx*gx + by, gx = tiles_n, gy = tiles_m,

@@ -244,6 +244,7 @@ def test_launchers_refuse_operands_that_would_send_a_kernel_out_of_bounds():
     args.workspace, args.workspace_bytes = 0x2004, 1 << 20
     assert handle.psg_gemm_a8w8(ctypes.byref(args), None) == -6
     assert b"workspace" in handle.psg_last_error()
+    assert handle.psg_static_scratch_bytes() == 32 << 20
 
 
 def test_struct_layouts_match_header():
