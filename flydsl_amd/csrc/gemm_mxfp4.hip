@@ -131,8 +131,14 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
         const int f = (t / 64) % (MB * 2);
         const int mb = f >> 1, nb = f & 1;
         const int np = (int)blockIdx.x * npw + npi;
-        v4f sum = red[npi * ks][f][lane];
-        for (int j = 1; j < ks; j++) sum += red[npi * ks + j][f][lane];
+        // all partial sums are read in one batch (no wait between them), then added in slice order
+        v4f part[NW];
+#pragma unroll
+        for (int j = 0; j < NW; j++) part[j] = red[npi * ks + (j < ks ? j : 0)][f][lane];
+        v4f sum = part[0];
+#pragma unroll
+        for (int j = 1; j < NW; j++)
+            if (j < ks) sum += part[j];
         const int m = mb * 16 + li;
         const int n = np * 32 + nb * 16 + lg * 4;
         if (np < n_pairs && m < p.M) store_mx4(p, STORE, (size_t)m * (size_t)p.N + (size_t)n, sum);

@@ -11,7 +11,7 @@
 #include "tile_order.h"
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
-hipError_t psg_launch_a8w8_smallm(const A8W8Params& p, int kind, int store, int nb, int nw, hipStream_t stream);
+hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
 hipError_t psg_launch_tile_order(int tiles_m, int tiles_n, int group_m, int32_t* out, hipStream_t stream);
@@ -203,18 +203,7 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
     hipError_t e;
     if (small) {
-        // two n-blocks per wavefront halve the A traffic per byte of W; keep one when that would leave too few
-        // wavefronts to cover the memory latency
-        const int steps = (kbytes + 127) / 128;
-        const int nb = (a->N / 16) >= 256 ? 2 : 1;
-        const int groups = (a->N / 16 + nb - 1) / nb;
-        // four wavefronts per workgroup with four K slices when every slice still spans at least two chunks of
-        // four K steps and there are enough wavefronts to keep the memory system busy; eight otherwise
-        const int nw = (steps >= 32 && groups * 4 >= 512) ? 4 : 8;
-        p.ksplit = pick_ksplit(groups, steps);
-        if (p.ksplit > nw) p.ksplit = nw;
-        if (nw == 4 && p.ksplit < 4 && steps >= 4) p.ksplit = 4;
-        e = psg_launch_a8w8_smallm(p, kind, store, nb, nw, static_cast<hipStream_t>(stream));
+        e = psg_launch_a8w8_stream(p, kind, store, static_cast<hipStream_t>(stream));
     } else {
         const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
         const Plan plan = plan_tiled(a->M, a->N, kbytes, false);
