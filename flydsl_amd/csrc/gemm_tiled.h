@@ -75,13 +75,15 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
-template <int KIND, int MR, int NR, int WM, int STORE>
-__global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4>
+__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
-    constexpr int WN = 4 / WM;
+    constexpr int WN = WAVES / WM;
     constexpr int TM = 16 * MR * WM;
     constexpr int TN = 16 * NR * WN;
-    constexpr int A_LOADS = TM / 32;  // 16-byte chunks of the A tile per thread
+    constexpr int RPP = WAVES * 8;        // A rows one pass of the whole workgroup copies (8 threads x 16 bytes per row)
+    constexpr int A_LOADS = TM / RPP;     // 16-byte chunks of the A tile per thread
+    static_assert(TM % RPP == 0, "the A tile must be a whole number of copy passes");
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * TK];
 
@@ -158,11 +160,11 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     auto load_a1 = [&](int kt, int j, v4i& dst) {
         const uint32_t k0 = (uint32_t)kt * TK;
         const bool in_k = kt < kt_end && (k0 + (uint32_t)a_kc * 16u) < (uint32_t)K;
-        const uint32_t off = a_goff0 + (uint32_t)j * 32u * (uint32_t)K + k0;
+        const uint32_t off = a_goff0 + (uint32_t)j * (uint32_t)RPP * (uint32_t)K + k0;
         dst = buf_load16(ra, in_k ? off : 0xFFFFFFF0u, 0);
     };
     auto store_a1 = [&](int stage, int j, const v4i& src) {
-        *reinterpret_cast<v4i*>(&lds[stage][lds_off(a_row0 + 32 * j, a_kc)]) = src;
+        *reinterpret_cast<v4i*>(&lds[stage][lds_off(a_row0 + RPP * j, a_kc)]) = src;
     };
     // W fragment load number idx of a K step: n-block idx/2, 64-byte half idx%2.  The n-block select sits in
     // the bounds-checked VGPR offset (blocks >= N/16 read as zero), the K position in the scalar offset.
@@ -355,14 +357,14 @@ __global__ void __launch_bounds__(256, (MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W
     });
 }
 
-template <int KIND, int MR, int NR, int WM, int STORE>
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
-    constexpr int TM = 16 * MR * WM, TN = 16 * NR * (4 / WM);
+    constexpr int TM = 16 * MR * WM, TN = 16 * NR * (WAVES / WM);
     const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     A8W8Params q = p;
     q.splits = splits;
-    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE>), dim3(tiles_m * tiles_n, splits), dim3(256), 0, stream, q);
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE, WAVES>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
     return hipGetLastError();
 }
 
@@ -373,6 +375,9 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
     if (tile_m == 16 * MR_ * WM_ && tile_n == 16 * NR_ * (4 / WM_)) return launch_one<KIND, MR_, NR_, WM_, STORE>(p, stream);
     if (p.wave_layout == 2) {
         PSG_CASE(8, 8, 2)
+    }
+    if (p.wave_layout == 8) {  // eight wavefronts side by side along N: 256x256 tile, every W fragment loaded once
+        if (tile_m == 256 && tile_n == 256) return launch_one<KIND, 16, 2, 1, STORE, 8>(p, stream);
     }
     PSG_CASE(16, 4, 1)
     PSG_CASE(8, 8, 1)

@@ -60,25 +60,28 @@ int pick_ksplit(int units, int steps) {
 
 struct Tile {
     int m, n;
+    int waves;  // wavefronts per workgroup: 4 (side by side along N, or 2x2) or 8 (side by side along N)
 };
 
-// Tile choice for the MFMA mainloop.  Each shape has a measured relative efficiency at full occupancy (the
-// 128-row tiles run two workgroups per CU, so one workgroup's epilogue overlaps the other's mainloop; the 256-row
-// tile has the highest operand reuse but runs alone).  The score multiplies that by how evenly the tiles fill the
-// CUs' workgroup slots and by the fraction of each tile that is not padding.
+// Tile choice for the MFMA mainloop.  Each shape has a measured relative efficiency at full occupancy.  The 256x256
+// tile of eight wavefronts side by side along N loads every W fragment once per CU and moves the least data per flop:
+// on real data the chip is power-limited, so that is what decides (fp8 8192x4096x4096: 117 us against 134 us for
+// the 128x256 tile that runs two workgroups per CU; int8 4096x28672x8192: 775 against 940).  For MXFP4 the launch is
+// bound by the C stores and the 4- and 8-wavefront forms measure the same.  The score multiplies the efficiency by
+// how evenly the tiles fill the CUs' workgroup slots and by the fraction of each tile that is not padding.
 Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     struct Shape {
-        int m, n, per_cu;
+        int m, n, waves, per_cu;
         double eff;
     };
-    static const Shape shapes8[] = {{128, 256, 2, 1.00}, {256, 256, 1, 0.95}, {64, 256, 2, 0.62}, {32, 256, 3, 0.36},
-                                    {128, 128, 2, 0.70}, {64, 64, 5, 0.25}};
-    static const Shape shapesx[] = {{256, 256, 1, 1.00}, {128, 256, 2, 0.86}, {64, 256, 2, 0.80}, {32, 256, 3, 0.40},
-                                    {64, 128, 3, 0.40}, {32, 128, 4, 0.25}};
+    static const Shape shapes8[] = {{256, 256, 8, 1, 1.17}, {128, 256, 4, 2, 1.00}, {64, 256, 4, 2, 0.62}, {32, 256, 4, 3, 0.36},
+                                    {128, 128, 4, 2, 0.70}, {64, 64, 4, 5, 0.25}};
+    static const Shape shapesx[] = {{256, 256, 4, 1, 1.00}, {128, 256, 4, 2, 0.86}, {64, 256, 4, 2, 0.80}, {32, 256, 4, 3, 0.40},
+                                    {64, 128, 4, 3, 0.40}, {32, 128, 4, 4, 0.25}};
     const Shape* shapes = mx ? shapesx : shapes8;
-    if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n};  // forced by the caller; the launcher rejects unknown shapes
+    if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n, 4};  // forced by the caller; the launcher rejects unknown shapes
     double best = -1.0;
-    Tile t = {shapes[0].m, shapes[0].n};
+    Tile t = {shapes[0].m, shapes[0].n, shapes[0].waves};
     for (int i = 0; i < 6; i++) {
         const int tm = shapes[i].m, tn = shapes[i].n;
         const long tiles_m = (M + tm - 1) / tm, tiles_n = (N + tn - 1) / tn;
@@ -92,7 +95,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
         const double score = busy * pad * shapes[i].eff;
         if (score > best) {
             best = score;
-            t = {tm, tn};
+            t = {tm, tn, shapes[i].waves};
         }
     }
     return t;
@@ -123,7 +126,7 @@ Plan plan_tiled(int M, int N, int kbytes, bool mx) {
     Tile t = pick_tile(M, N, mx, 0, 0);
     const long tiles_big = (long)((M + 127) / 128) * (long)((N + 255) / 256);
     const int steps = (kbytes + 127) / 128;
-    if (!mx && tiles_big < 192 && steps >= 48) t = M <= 64 ? Tile{64, 64} : Tile{128, 128};
+    if (!mx && tiles_big < 192 && steps >= 48) t = M <= 64 ? Tile{64, 64, 4} : Tile{128, 128, 4};
     return {t, pick_splits(M, N, kbytes, t)};
 }
 
@@ -207,9 +210,10 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     } else {
         const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
         const Plan plan = plan_tiled(a->M, a->N, kbytes, false);
-        const Tile t = forced ? Tile{a->tile_m, a->tile_n} : plan.t;
+        const Tile t = forced ? Tile{a->tile_m, a->tile_n, 4} : plan.t;
         p.ksplit = 1;
-        p.wave_layout = a->reserved == 2 ? 2 : 1;  // wavefront layout of the 256x256 tile (2 = 2x2), a test / tuning knob
+        // wavefront layout of the 256x256 tile: the planner's choice, or forced (2 = 2x2, 8 = 1x8) by tests / tuning
+        p.wave_layout = a->reserved >= 2 ? a->reserved : (!forced && t.waves == 8 ? 8 : 1);
         // forced launches take the split count from tile_k (1..16); otherwise the planner decides
         int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
         if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
@@ -342,7 +346,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     } else {
         const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
         const Plan plan = plan_tiled(a->M, a->N, a->K / 2, true);
-        const Tile t = forced ? Tile{a->tile_m, a->tile_n} : plan.t;
+        const Tile t = forced ? Tile{a->tile_m, a->tile_n, 4} : plan.t;
         int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
         if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
         A8W8Params q{};
@@ -356,7 +360,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         q.K = p.K;
         q.group_m = p.group_m;
         q.ksplit = 1;
-        q.wave_layout = a->reserved == 2 ? 2 : 1;
+        q.wave_layout = a->reserved >= 2 ? a->reserved : 1;
         q.splits = splits;
         q.epi = EPI_NONE;
         q.out = p.out;

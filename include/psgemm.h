@@ -98,7 +98,7 @@ typedef struct psg_a8w8_args {
     int32_t tile_m, tile_n, tile_k;
     int32_t xcd_swizzle;
     int32_t force_path; /* 0 = auto, 1 = tiled MFMA mainloop, 2 = small-M split-K (tests/benchmarks) */
-    int32_t reserved;   /* 0; 2 = run a forced 256x256 tile with 2x2 wavefronts instead of 1x4 (tuning knob) */
+    int32_t reserved;   /* 0; tuning knob for a forced 256x256 tile: 2 = 2x2 wavefronts, 8 = eight wavefronts 1x8 (default 1x4) */
 } psg_a8w8_args;
 
 /*

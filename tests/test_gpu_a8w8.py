@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 SENTINEL = -8192.0
 
 
-def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, guard_rows=0, out_dtype="bf16"):
+def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, guard_rows=0, out_dtype="bf16", wave_layout=0):
     from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
     dev = torch.device("cuda")
@@ -35,12 +35,12 @@ def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, 
     sa, sb = d["sa"].to(dev), d["sb"].to(dev)
     bias_t = bias.to(dev) if bias is not None else torch.empty(0, dtype=tdt, device=dev)
     fn.launch_forced(c_alloc[:M].view(-1), a.view(-1), b.view(-1), sa, sb, bias_t, M, N, torch.cuda.current_stream(),
-                     force_path=force_path, tile=tile)
+                     force_path=force_path, tile=tile, wave_layout=wave_layout)
     torch.cuda.synchronize()
     return c_alloc
 
 
-def _acc(d, M, N, K, *, force_path=0, tile=None):
+def _acc(d, M, N, K, *, force_path=0, tile=None, wave_layout=0):
     from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
     dev = torch.device("cuda")
@@ -48,7 +48,7 @@ def _acc(d, M, N, K, *, force_path=0, tile=None):
     dt = torch.int32 if d["kind"] == "int8" else torch.float32
     acc = torch.full((M, N), -7, dtype=dt, device=dev)
     fn.accumulators(acc, d["a_q"].to(dev), d["b_shuf"].to(dev), M, N, torch.cuda.current_stream(), force_path=force_path,
-                    tile=tile)
+                    tile=tile, wave_layout=wave_layout)
     torch.cuda.synchronize()
     return acc.cpu().numpy()
 
@@ -230,3 +230,29 @@ def test_short_k_every_tile(K):
             c = _launch(d, M, N, K, force_path=1, tile=tile)
             assert np.array_equal(bf16_bits(c[:M]), ref), f"tile {tile}"
             assert np.array_equal(_acc(d, M, N, K, force_path=1, tile=tile), want), f"tile {tile}"
+
+
+# ---- the 256x256 tile of eight wavefronts (what the planner picks for problems that fill the GPU) and the 2x2 form ----
+@pytest.mark.parametrize("wave_layout", [8, 2])
+@pytest.mark.parametrize("M,N,K", [(128, 1024, 1024), (300, 272, 192), (257, 48, 64), (700, 528, 320), (600, 992, 4160)])
+def test_int8_wavefront_layouts_bit_exact(wave_layout, M, N, K):
+    d = make_a8w8(M, N, K, "int8", seed=M)
+    want = O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"]))
+    ref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")["c_bf16_bits"]
+    assert np.array_equal(_acc(d, M, N, K, force_path=1, tile=(256, 256), wave_layout=wave_layout), want)
+    c = _launch(d, M, N, K, force_path=1, tile=(256, 256), guard_rows=32, wave_layout=wave_layout)
+    assert np.array_equal(bf16_bits(c[:M]), ref)
+    assert (c[M:] == SENTINEL).all()
+
+
+@pytest.mark.parametrize("epilogue", ["none", "bias_silu"])
+def test_fp8_eight_wavefront_tile(epilogue):
+    M, N, K = 520, 784, 2112
+    d = make_a8w8(M, N, K, "fp8", seed=4, w_std=0.05)
+    g = torch.Generator().manual_seed(1)
+    bias = (torch.randn(N, generator=g) * 0.2).to(torch.bfloat16)
+    ref = O.run_torch(np_bytes(d["a_q"]), np_bytes(d["b_q"]), d["sa"].numpy(), d["sb"].numpy(), "fp8")
+    if epilogue != "none":
+        ref = O.apply_bias_act(ref, bias.float().numpy(), "silu")
+    c = _launch(d, M, N, K, force_path=1, tile=(256, 256), epilogue=epilogue, bias=bias, wave_layout=8)
+    _check_fp(c[:M].float().cpu().numpy(), ref)
