@@ -6,8 +6,9 @@
 A step is one GEMM launch on one set of synthetic operands (seed 0; activations N(0,1), weights
 N(0,0.02), quantised and preshuffled on the host, resident in HBM before the timed region).
 Steps rotate through enough independent operand sets that the weights cannot be served from the
-256 MB Infinity Cache.  The K timed steps are recorded once into a HIP graph and replayed, bracketed by
-``torch.cuda.synchronize()`` on both sides (wall clock -> ``value`` / ``ms_per_step``) and by HIP events
+256 MB Infinity Cache.  The K timed steps are recorded once into a HIP graph; the graph is replayed as often as
+it takes to time at least 50 ms of work (a K-step graph of a 7 us kernel is far too short to time once), bracketed
+by ``torch.cuda.synchronize()`` on both sides (wall clock -> ``value`` / ``ms_per_step``) and by HIP events
 on the launch stream (-> ``roofline.achieved``).  Prints ONE JSON line.
 """
 
@@ -38,6 +39,7 @@ WORKLOADS = {
 DEFAULT_WORKLOAD = "fp8_decode_m16"
 PEAK = {"hbm": 8000.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0, "bf16": 2500.0, "fp16": 2500.0}  # GB/s, TFLOP/s (dense, published)
 MALL_BYTES = 256 << 20
+MIN_TIMED_S = 0.05  # every timed region holds at least this much GPU work
 
 
 def algorithmic_bytes(family, M, N, K):
@@ -117,19 +119,27 @@ def run_workload(name, steps, warmup, check=True):
     torch.cuda.synchronize()
 
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # one timed probe replay sizes the number of replays so that every timed region holds at least MIN_TIMED_S of work
+    torch.cuda.synchronize()
+    ev0.record()
+    graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    replays = max(1, math.ceil(MIN_TIMED_S / max(ev0.elapsed_time(ev1) * 1e-3, 1e-7)))
     best_wall, best_ev = float("inf"), float("inf")
     for _ in range(3):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         ev0.record()
-        graph.replay()
+        for _r in range(replays):
+            graph.replay()
         ev1.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
         best_wall = min(best_wall, wall)
         best_ev = min(best_ev, ev0.elapsed_time(ev1) * 1e-3)
-    sec_per_step = best_wall / steps
-    kernel_s = best_ev / steps
+    sec_per_step = best_wall / (steps * replays)
+    kernel_s = best_ev / (steps * replays)
 
     # hot-cache figure (one operand set): informative only
     ghot = torch.cuda.CUDAGraph()
@@ -140,10 +150,11 @@ def run_workload(name, steps, warmup, check=True):
     ghot.replay()
     torch.cuda.synchronize()
     ev0.record()
-    ghot.replay()
+    for _r in range(replays):
+        ghot.replay()
     ev1.record()
     torch.cuda.synchronize()
-    hot_s = ev0.elapsed_time(ev1) * 1e-3 / steps
+    hot_s = ev0.elapsed_time(ev1) * 1e-3 / (steps * replays)
 
     ok = None
     if check:
@@ -170,7 +181,7 @@ def run_workload(name, steps, warmup, check=True):
         "workload": name, "dtype": kind, "M": M, "N": N, "K": K,
         "tflops": flops / sec_per_step / 1e12, "gb_per_s": nbytes / sec_per_step / 1e9,
         "us_per_step_wall": sec_per_step * 1e6, "us_per_launch_events": kernel_s * 1e6, "us_per_launch_hot_cache": hot_s * 1e6,
-        "operand_sets": n_sets, "parity_ok": ok,
+        "operand_sets": n_sets, "graph_replays_per_timing": replays, "parity_ok": ok,
         "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
                      "traffic": None, "algorithmic_bytes": nbytes, "flops": flops},
     }
@@ -229,12 +240,12 @@ def run_quant_workload(name, steps=50, warmup=5):
                   np.array_equal(out[1].view(torch.uint8).cpu().numpy(), O.shuffle_scale_w4(ws)))
     achieved = nbytes / sec / 1e9
     return {"workload": name, "dtype": kind, "M": M, "K": K, "gb_per_s": achieved, "us_per_launch_events": sec * 1e6,
-            "operand_sets": n_sets, "parity_ok": ok, "timing": "graph replay, caller-owned outputs, HIP events",
+            "operand_sets": n_sets, "graph_replays_per_timing": replays, "parity_ok": ok, "timing": "graph replay, caller-owned outputs, HIP events",
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK["hbm"], "unit": "GB/s", "frac": achieved / PEAK["hbm"],
                          "traffic": None, "algorithmic_bytes": nbytes}}
 
 
-def cpu_baseline(name, host, budget_s=12.0):
+def cpu_baseline(name, host, budget_s=12.0):  # budget_s bounds the CPU work of one workload
     """The reference's torch CPU path (dequantise to fp32 + torch.mm) on the same seeded operands,
     timed on this box's host cores.  For workloads whose single pass exceeds the budget a row sample of
     A is used (the weight side, which dominates the dequantisation cost, is always whole)."""
@@ -337,16 +348,22 @@ def main():
             if name == args.workload:
                 continue
             b = WORKLOADS[name][5]
-            r, _ = run_workload(name, 300 if b == "hbm" else (5 if name == "int8_ffn_m4096" else 20), 20 if b == "hbm" else 2)
+            r, h = run_workload(name, 300 if b == "hbm" else (5 if name == "int8_ffn_m4096" else 20), 20 if b == "hbm" else 2)
             r["roofline"]["traffic"] = load_traffic(name)
+            # the reference's CPU path beside every configuration (a bounded row sample, a few seconds each)
+            r["cpu_baseline"] = None if args.no_cpu else cpu_baseline(name, h, budget_s=3.0)
+            del h
             others.append(r)
         for name in ("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"):
             others.append(run_quant_workload(name))
 
     line = {
         "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",
-        "value": main_res["tflops"],
-        "unit": "TFLOP/s",
+        # whole-job throughput in the unit of the roofline that bounds the workload: bytes for the decode shapes
+        # (algorithmic bytes per launch / time per step), flops for the prefill shapes
+        "value": main_res["gb_per_s"] if bound == "hbm" else main_res["tflops"],
+        "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+        "tflops": main_res["tflops"],
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,
@@ -358,7 +375,8 @@ def main():
         "data": "synthetic (seed 0; A~N(0,1) per-token quantised, W~N(0,0.02) per-channel quantised and preshuffled; "
                 f"{main_res['operand_sets']} rotating operand sets)",
         "config": {"workload": f"{args.workload}: {kind} W8A8 preshuffle GEMM M={M} N={N} K={K}, bf16 out", "M": M, "N": N, "K": K,
-                   "timing": "K steps recorded into one HIP graph, replayed; wall clock between synchronizes"},
+                   "timing": f"K steps recorded into one HIP graph, replayed {main_res['graph_replays_per_timing']}x per timing "
+                             "(>= 50 ms of work); wall clock between synchronizes"},
         "gb_per_s": main_res["gb_per_s"],
         "parity_ok": main_res["parity_ok"],
         "us_per_launch_events": main_res["us_per_launch_events"],
@@ -370,7 +388,8 @@ def main():
     # the metric names two operating points; the second one (MFMA-bound prefill) is lifted out of the table for convenience
     for r in others:
         if r["workload"] == "fp8_prefill_m8192":
-            line["prefill_m8192"] = {"tflops": r["tflops"], "us_per_launch_events": r["us_per_launch_events"], "roofline": r["roofline"]}
+            line["prefill_m8192"] = {"tflops": r["tflops"], "us_per_launch_events": r["us_per_launch_events"], "roofline": r["roofline"],
+                                     "cpu_baseline": r.get("cpu_baseline")}
     print(json.dumps(line))
 
 
