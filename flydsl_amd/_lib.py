@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -57,6 +57,8 @@ class A8W8Args(ctypes.Structure):
         ("xcd_swizzle", ctypes.c_int32),
         ("force_path", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
+        ("b_layout", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
     ]
 
 

@@ -116,8 +116,12 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
 #pragma unroll
         for (int w = 0; w < NWIN; w++) {
             const int n = n_begin + w * 16 + li;
-            wvoff[w] = n < n_end ? (uint32_t)(n >> 4) * 16u * (uint32_t)K + (uint32_t)lg * 256u + (uint32_t)(n & 15) * 16u : OOB;
+            // preshuffled: 16-byte piece (K group lg, row n%16) of the 1 KB block; row-major [N,K]: row n, K offset 16*lg
+            const uint32_t off = p.b_rowmajor ? (uint32_t)n * (uint32_t)K + (uint32_t)lg * 16u
+                                              : (uint32_t)(n >> 4) * 16u * (uint32_t)K + (uint32_t)lg * 256u + (uint32_t)(n & 15) * 16u;
+            wvoff[w] = n < n_end ? off : OOB;
         }
+        const uint32_t w_step = p.b_rowmajor ? 128u : 2048u, w_half = p.b_rowmajor ? 64u : 1024u;
         const int st_c = lane % CPR;
         const int st_r0 = lane / CPR;
         const uint32_t slice_end = (uint32_t)(s_end * 128 < K ? s_end * 128 : K);
@@ -139,8 +143,8 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
                     const int s = s0 + u;
                     const bool has_lo = c < nchunks && s < s_end;      // wave-uniform
                     const bool has_hi = has_lo && (s * 128 + 64) < K;  // K % 128 == 64: the last step has no upper half
-                    wlo[w][u] = buf_load16_nt(rb, has_lo ? wvoff[w] : OOB, has_lo ? (uint32_t)s * 2048u : 0u);
-                    whi[w][u] = buf_load16_nt(rb, has_hi ? wvoff[w] : OOB, has_hi ? (uint32_t)s * 2048u + 1024u : 0u);
+                    wlo[w][u] = buf_load16_nt(rb, has_lo ? wvoff[w] : OOB, has_lo ? (uint32_t)s * w_step : 0u);
+                    whi[w][u] = buf_load16_nt(rb, has_hi ? wvoff[w] : OOB, has_hi ? (uint32_t)s * w_step + w_half : 0u);
                 }
             // keep the machine scheduler from sinking these loads below later code to save registers
             __builtin_amdgcn_sched_barrier(0);

@@ -178,11 +178,17 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
             sb_dst[q - MP] = buf_load4(rsb, has ? (uint32_t)(q - MP) * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
         }
     };
+    // W addressing.  Preshuffled: lane l reads bytes [16l, 16l+16) of the 1 KB block (n-block, 64-byte K block).
+    // Row-major [N,K] (the row-scale fp8 GEMM's plain-B call shape): the same fragment is 16 rows x 64 bytes, lane
+    // (row li, 16-byte K group lg) reads row li of the n-block at K offset 16*lg; 16 segments of 64 bytes per load
+    // instead of one contiguous KB.  Either way an n-block of 16 rows is 16*K bytes, so the descriptor is the same.
+    const uint32_t b_lane_off = p.b_rowmajor ? (uint32_t)li * (uint32_t)K + (uint32_t)lg * 16u : (uint32_t)lane * 16u;
+    const uint32_t b_step = p.b_rowmajor ? 128u : 2048u, b_half = p.b_rowmajor ? 64u : 1024u;
     auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi) {
         const int ni = idx >> 1;
         const bool has = kt < kt_end && (kt * TK + (idx & 1) * 64) < K;
-        const uint32_t voff = (uint32_t)lane * 16u + (uint32_t)ni * 16u * (uint32_t)K;
-        const v4i v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, has ? (uint32_t)kt * 2048u + (uint32_t)(idx & 1) * 1024u : 0u);
+        const uint32_t voff = b_lane_off + (uint32_t)ni * 16u * (uint32_t)K;
+        const v4i v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, has ? (uint32_t)kt * b_step + (uint32_t)(idx & 1) * b_half : 0u);
         if (idx & 1) hi[ni] = v; else lo[ni] = v;
     };
     auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {

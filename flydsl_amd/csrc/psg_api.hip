@@ -161,6 +161,7 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
         if (a->epilogue != PSG_EPI_NONE && !aligned(a->bias, 8)) return fail(PSG_E_ALIGN, "bias must be 8-byte aligned");
     }
     if (a->workspace && !aligned(a->workspace, 16)) return fail(PSG_E_ALIGN, "workspace must be 16-byte aligned");
+    if (a->b_layout != 0 && a->b_layout != 1) return fail(PSG_E_DTYPE, "b_layout=%d unknown (0 preshuffled, 1 row-major)", a->b_layout);
     if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
     if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
     return 0;
@@ -197,6 +198,7 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     p.K = a->K;
     p.epi = a->epilogue;
     p.out = a->out_dtype;
+    p.b_rowmajor = a->b_layout;
     // M-tiles per group of the XCD-aware tile order: 8 makes the set of tiles one XCD works on at a time roughly
     // square in bytes (A rows vs W rows), which minimises what its L2 has to fetch
     p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;

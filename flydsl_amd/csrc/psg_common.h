@@ -110,6 +110,7 @@ struct A8W8Params {
     int wave_layout;  // tiled kernel: 2 = 2x2 wavefronts for the 256x256 tile, else 1x4
     int epi;      // EPI_*
     int out;      // OUT_*
+    int b_rowmajor;  // 0: W preshuffled (1 KB fragment blocks); 1: W plain row-major [N,K] (8- and 16-bit kinds only)
     const uint8_t* mx_sa;  // MXFP4 only: shuffled e8m0 [ceil(M/32)*32, K/32]
     const uint8_t* mx_sb;  // MXFP4 only: shuffled e8m0 [N, K/32]
 };

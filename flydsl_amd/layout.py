@@ -72,3 +72,12 @@ def shuffle_scale_w4(src: torch.Tensor, experts_cnt: int = 1, gate_up: bool = Fa
     v = src.reshape(r // 32, 2, 16, kb // 8, 2, 4)
     #            r/32  kb/8  kb%4  r%16  kb half  r half
     return v.permute(0, 3, 5, 2, 4, 1).contiguous().reshape(r, kb)
+
+
+def preshuffle_b(b_t: torch.Tensor) -> torch.Tensor:
+    """Permute row-major 1-byte ``B_T [N, K]`` into the preshuffled fragment layout, as the reference's helper of the
+    row-scale fp8 GEMMs does (kernels/gemm/fp8_gemm_utils.py:24-28): blocks ``[N/16][K/64][4][16][16 B]``, i.e. the
+    byte map of ``shuffle_weight`` for 1-byte elements.  The result keeps that 5-D block shape."""
+    n, k = b_t.shape[-2:]
+    assert n % 16 == 0 and k % 64 == 0, f"need N%16==0 and K%64==0, got N={n} K={k}"
+    return b_t.reshape(n // 16, 16, k // 64, 4, 16).permute(0, 2, 3, 1, 4).contiguous()

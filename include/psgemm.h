@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 1
+#define PSG_ABI_VERSION 2
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
@@ -99,6 +99,9 @@ typedef struct psg_a8w8_args {
     int32_t xcd_swizzle;
     int32_t force_path; /* 0 = auto, 1 = tiled MFMA mainloop, 2 = small-M split-K (tests/benchmarks) */
     int32_t reserved;   /* 0; tuning knob for a forced 256x256 tile: 2 = 2x2 wavefronts, 8 = eight wavefronts 1x8 (default 1x4) */
+    int32_t b_layout;   /* 0 = b is preshuffled (above); 1 = b is plain row-major W[N,K], the b_preshuffled=False call
+                           shape of the reference's row-scale fp8 GEMMs (kernels/gemm/fp8_gemm_8wave.py:148) */
+    int32_t pad0;       /* 0 */
 } psg_a8w8_args;
 
 /*

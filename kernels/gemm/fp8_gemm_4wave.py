@@ -1,0 +1,2 @@
+"""Same import path as the reference's kernels/gemm/fp8_gemm_4wave.py."""
+from flydsl_amd.kernels.gemm.fp8_gemm_rowscale import compile_fp8_gemm_4w  # noqa: F401

@@ -247,15 +247,35 @@ def test_launchers_refuse_operands_that_would_send_a_kernel_out_of_bounds():
     assert handle.psg_static_scratch_bytes() == 32 << 20
 
 
+def test_rowscale_fp8_entry_points_keep_the_reference_assertions():
+    from kernels.gemm.fp8_gemm_4wave import compile_fp8_gemm_4w
+    from kernels.gemm.fp8_gemm_8wave import compile_fp8_gemm_8w
+    from kernels.gemm.fp8_gemm_utils import preshuffle_b
+
+    with pytest.raises(AssertionError):
+        compile_fp8_gemm_8w(K=4096, BLOCK_M=64, BLOCK_N=256)   # 8w needs BLOCK_M >= 128
+    with pytest.raises(AssertionError):
+        compile_fp8_gemm_8w(K=4096 + 64)                       # K % 128
+    with pytest.raises(AssertionError):
+        compile_fp8_gemm_4w(K=4096, BLOCK_M=96, BLOCK_N=64)    # BLOCK_M % 64
+    fn = compile_fp8_gemm_4w(K=256, BLOCK_M=64, BLOCK_N=64, use_xcd_remap=False, b_preshuffled=True)
+    with pytest.raises(ValueError, match="device"):
+        fn(torch.zeros(4, 256, dtype=torch.int8), torch.zeros(32, 256, dtype=torch.int8), torch.zeros(4, 32, dtype=torch.bfloat16),
+           torch.zeros(4), torch.zeros(32), 4, 32, 0)
+    # preshuffle_b is the byte map of shuffle_weight for 1-byte elements
+    w = torch.arange(64 * 256, dtype=torch.int32).remainder(251).to(torch.uint8).reshape(64, 256)
+    assert torch.equal(preshuffle_b(w).reshape(64, 256), layout.shuffle_weight(w).reshape(64, 256))
+
+
 def test_struct_layouts_match_header():
     src = r'''
     #include <stdio.h>
     #include <stddef.h>
     #include "psgemm.h"
     int main(void) {
-        printf("%zu %zu %zu %zu %zu %zu\n", sizeof(psg_a8w8_args), offsetof(psg_a8w8_args, workspace_bytes),
+        printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(psg_a8w8_args), offsetof(psg_a8w8_args, workspace_bytes),
                offsetof(psg_a8w8_args, M), offsetof(psg_a8w8_args, epilogue), offsetof(psg_a8w8_args, force_path),
-               offsetof(psg_a8w8_args, bias));
+               offsetof(psg_a8w8_args, bias), offsetof(psg_a8w8_args, b_layout));
         printf("%zu %zu %zu %zu\n", sizeof(psg_mxfp4_args), offsetof(psg_mxfp4_args, M), offsetof(psg_mxfp4_args, out_dtype),
                offsetof(psg_mxfp4_args, force_path));
         return 0;
@@ -268,7 +288,7 @@ def test_struct_layouts_match_header():
         out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
     a, m = _lib.A8W8Args, _lib.MxArgs
     want = [ctypes.sizeof(a), a.workspace_bytes.offset, a.M.offset, a.epilogue.offset, a.force_path.offset, a.bias.offset,
-            ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset]
+            a.b_layout.offset, ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset]
     assert [int(v) for v in out] == want
 
 
