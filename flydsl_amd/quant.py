@@ -98,7 +98,9 @@ def mxfp4_to_f32(x: torch.Tensor) -> torch.Tensor:
 def per_1x32_f4_quant(x, scale=None, quant_dtype=fp4x2, shuffle=False):
     """OCP-MX fp4 quantisation, one e8m0 scale per 32 consecutive elements of the last dim:
     scale byte = ``f32_to_e8m0(amax / 4)``, codes = e2m1(x / 2^(scale-127)).
-    Returns ``(packed [.., K/2], scale [R, K/32] as e8m0, scaled fp32 values)`` like the reference."""
+    Returns ``(packed [.., K/2], scale [R, K/32] as e8m0, scaled fp32 values)`` like the reference.  Byte-for-byte
+    equal to the reference's quantiser on finite inputs; NaN / Inf elements are not pinned (the threshold chain maps
+    NaN to code 0 and Inf to +-6)."""
     assert quant_dtype == fp4x2
     if shuffle:
         raise NotImplementedError("use shuffle_scale_w4 on the returned scales")

@@ -56,7 +56,9 @@ def pertoken_quant(x: torch.Tensor, quant_dtype=torch.int8, stream=None, out=Non
 
 def per_1x32_f4_quant(x: torch.Tensor, shuffle: bool = True, stream=None, out=None):
     """OCP-MX fp4 quantisation on the device.  Returns ``(packed [M,K/2], scales)`` where ``scales`` are e8m0 bytes over
-    ``ceil(M/32)*32`` rows x ``K/32``: in the GEMM's shuffled layout when ``shuffle`` (default), row-major otherwise."""
+    ``ceil(M/32)*32`` rows x ``K/32``: in the GEMM's shuffled layout when ``shuffle`` (default), row-major otherwise.
+    Finite inputs only: a NaN / Inf in a block does not give the reference's 0xFF scale byte (the block maximum drops
+    NaN)."""
     code = _x_code(x)
     m, k = x.shape
     r = (m + 31) // 32 * 32

@@ -184,6 +184,9 @@ int psg_gemm_mxfp4_acc(const psg_mxfp4_args *args, void *acc, void *stream);
  * tests/utils.py:29-73 (pertoken_quant) and tests/kernels/utils/gemm_common_utils.py:675-704 (per_1x32_f4_quant)
  * followed by :645-672 (shuffle_scale_w4); these produce the same bytes on the device.
  *   x_dtype: 0 fp32, 1 bf16, 2 fp16.  x is [M,K] row-major.
+ *   psg_quant_pertoken treats NaN / Inf like the reference (nan_to_num, then the row maximum).  psg_quant_mxfp4 is
+ *   defined for FINITE inputs only: a NaN or Inf inside a 32-element block does not produce the reference's 0xFF
+ *   scale byte (the block maximum is taken with fmaxf, which drops NaN).
  */
 
 /* y [M,K] int8 (out_dtype PSG_IN_INT8) or e4m3fn (PSG_IN_FP8_E4M3FN); scale [M] fp32 = max|row| / dtypeMax. K % 8 == 0. */
