@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -81,8 +81,20 @@ class MxArgs(ctypes.Structure):
         ("xcd_swizzle", ctypes.c_int32),
         ("force_path", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
+        ("a_dtype", ctypes.c_int32),
+        ("b_dtype", ctypes.c_int32),
+        ("batch", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
+        ("a_row_stride", ctypes.c_int64),
+        ("c_row_stride", ctypes.c_int64),
+        ("scale_a_chunk_stride", ctypes.c_int64),
+        ("a_batch_stride", ctypes.c_int64),
+        ("c_batch_stride", ctypes.c_int64),
+        ("scale_a_batch_stride", ctypes.c_int64),
     ]
 
+
+MX_DTYPE = {"fp4": 0, "fp6": 1, "fp8": 2}
 
 _lib = None
 

@@ -12,6 +12,7 @@
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
+hipError_t psg_launch_mx_generic(const MxGenParams& p, int af, int bf, int store, int batch, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
 hipError_t psg_launch_tile_order(int tiles_m, int tiles_n, int group_m, int32_t* out, hipStream_t stream);
@@ -315,15 +316,66 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     if (!a) return fail(PSG_E_NULL, "args is NULL");
     if (!out || !a->a || !a->b || !a->scale_a || !a->scale_b) return fail(PSG_E_NULL, "c, a, b, scale_a, scale_b must be non-NULL");
     if (a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
+    if (a->a_dtype < PSG_MX_FP4 || a->a_dtype > PSG_MX_FP8) return fail(PSG_E_DTYPE, "a_dtype %d unknown (0 fp4, 1 fp6, 2 fp8)", a->a_dtype);
+    if (a->b_dtype != PSG_MX_FP4 && a->b_dtype != PSG_MX_FP8) return fail(PSG_E_DTYPE, "b_dtype %d must be 0 (fp4) or 2 (fp8)", a->b_dtype);
     if (a->M < 1 || a->M > 65536) return fail(PSG_E_SHAPE, "M=%d outside [1, 65536]", a->M);
     if (a->N < 32 || a->N % 32) return fail(PSG_E_SHAPE, "N=%d must be a positive multiple of 32", a->N);
     if (a->K < 256 || a->K % 256) return fail(PSG_E_SHAPE, "K=%d must be a positive multiple of 256", a->K);
-    if ((uint64_t)a->N * (uint64_t)a->K / 2 > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "N*K/2 exceeds the 4 GiB descriptor range");
+    if (a->batch < 0 || a->batch > 65535) return fail(PSG_E_SHAPE, "batch=%d outside [0, 65535]", a->batch);
+    if (a->pad0 != 0) return fail(PSG_E_SHAPE, "pad0 must be 0");
+    const int batch = a->batch > 1 ? a->batch : 1;
+    const uint64_t a_row = a->a_dtype == PSG_MX_FP4 ? (uint64_t)a->K / 2 : (uint64_t)a->K;
+    const uint64_t b_row = a->b_dtype == PSG_MX_FP4 ? (uint64_t)a->K / 2 : (uint64_t)a->K;
+    const uint64_t chunk = (uint64_t)(a->K / 256) * 256;
+    if ((uint64_t)a->N * b_row > 0xFFFFFFFFull) return fail(PSG_E_SHAPE, "one batch of W exceeds the 4 GiB descriptor range");
+    if (a->a_row_stride < 0 || a->c_row_stride < 0 || a->scale_a_chunk_stride < 0 || a->a_batch_stride < 0 || a->c_batch_stride < 0 ||
+        a->scale_a_batch_stride < 0)
+        return fail(PSG_E_SHAPE, "strides must be >= 0 (0 = dense)");
+    const uint64_t a_rs = a->a_row_stride ? (uint64_t)a->a_row_stride : a_row;
+    const uint64_t c_rs = a->c_row_stride ? (uint64_t)a->c_row_stride : (uint64_t)a->N;
+    const uint64_t sa_cs = a->scale_a_chunk_stride ? (uint64_t)a->scale_a_chunk_stride : chunk;
+    if (a_rs < a_row || a_rs % 16) return fail(PSG_E_SHAPE, "a_row_stride=%lld must be a multiple of 16 and at least the %llu bytes of a row",
+                                               (long long)a_rs, (unsigned long long)a_row);
+    if (c_rs < (uint64_t)a->N || c_rs % 4) return fail(PSG_E_SHAPE, "c_row_stride=%lld must be a multiple of 4 elements and at least N", (long long)c_rs);
+    if (sa_cs < chunk || sa_cs % 4) return fail(PSG_E_SHAPE, "scale_a_chunk_stride=%lld must be a multiple of 4 and at least %llu", (long long)sa_cs,
+                                                (unsigned long long)chunk);
+    if ((uint64_t)a->M * a_rs > 0xFFFFFFFFull || (uint64_t)((a->M + 31) / 32) * sa_cs > 0xFFFFFFFFull)
+        return fail(PSG_E_SHAPE, "one batch of A or scale_a exceeds the 4 GiB descriptor range");
+    if (a->a_batch_stride % 16 || a->c_batch_stride % 8 || a->scale_a_batch_stride % 4)
+        return fail(PSG_E_ALIGN, "batch strides must keep a 16-byte, c 8-byte and scale_a 4-byte aligned");
     if (!aligned(a->a, 16) || !aligned(a->b, 16)) return fail(PSG_E_ALIGN, "a and b must be 16-byte aligned");
     if (!aligned(a->scale_a, 4) || !aligned(a->scale_b, 4)) return fail(PSG_E_ALIGN, "scales must be 4-byte aligned");
     if (!aligned(out, store == STORE_ACC ? 16 : 8)) return fail(PSG_E_ALIGN, "output must be %d-byte aligned", store == STORE_ACC ? 16 : 8);
-    if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
+    if (a->force_path < 0 || a->force_path > 3) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
+    const bool dense = a_rs == a_row && c_rs == (uint64_t)a->N && sa_cs == chunk;
+    const bool fp4_fast = a->a_dtype == PSG_MX_FP4 && a->b_dtype == PSG_MX_FP4 && batch == 1 && dense;
+    if ((a->force_path == 1 || a->force_path == 2) && !fp4_fast)
+        return fail(PSG_E_SHAPE, "force_path=%d is for dense, unbatched fp4 x fp4 only", a->force_path);
     if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    if (a->force_path == 3 || !fp4_fast) {
+        MxGenParams g;
+        g.c = out;
+        g.a = static_cast<const uint8_t*>(a->a);
+        g.b = static_cast<const uint8_t*>(a->b);
+        g.sa = static_cast<const uint8_t*>(a->scale_a);
+        g.sb = static_cast<const uint8_t*>(a->scale_b);
+        g.M = a->M;
+        g.N = a->N;
+        g.K = a->K;
+        g.out = a->out_dtype;
+        g.a_row_stride = (int64_t)a_rs;
+        g.c_row_stride = (int64_t)c_rs;
+        g.sa_chunk_stride = (int64_t)sa_cs;
+        g.a_batch = a->a_batch_stride ? a->a_batch_stride : (int64_t)((uint64_t)a->M * a_rs);
+        g.b_batch = (int64_t)((uint64_t)a->N * b_row);
+        g.c_batch = store == STORE_ACC ? (int64_t)a->M * a->N * 4 : (a->c_batch_stride ? a->c_batch_stride : (int64_t)((uint64_t)a->M * c_rs * 2));
+        g.sa_batch = a->scale_a_batch_stride ? a->scale_a_batch_stride : (int64_t)((uint64_t)((a->M + 31) / 32) * sa_cs);
+        g.sb_batch = (int64_t)((uint64_t)(a->N / 32) * chunk);
+        const hipError_t ge = psg_launch_mx_generic(g, a->a_dtype, a->b_dtype, store, batch, static_cast<hipStream_t>(stream));
+        if (ge != hipSuccess) return hip_fail(ge, "psg_gemm_mxfp4 launch");
+        g_err[0] = 0;
+        return 0;
+    }
     MxParams p;
     p.c = out;
     p.a = static_cast<const uint8_t*>(a->a);

@@ -127,6 +127,22 @@ struct MxParams {
     int out;  // OUT_*
 };
 
+// Arguments of the general MX kernel: any of fp4 / fp6 / fp8 A against fp4 / fp8 W, strided-batched.
+enum { MXF_FP4 = 0, MXF_FP6 = 1, MXF_FP8 = 2 };
+struct MxGenParams {
+    void* c;
+    const uint8_t* a;    // A rows: fp4 K/2 bytes; fp8 K bytes; fp6 K bytes (per 32 elements 24 packed bytes + 8 of padding)
+    const uint8_t* b;    // preshuffled W: K/2 bytes per row (fp4) or K (fp8)
+    const uint8_t* sa;   // shuffled e8m0, 32-row chunks of (K/256)*256 bytes
+    const uint8_t* sb;
+    int M, N, K;
+    int out;             // OUT_*
+    int64_t a_row_stride;      // bytes between rows of A
+    int64_t c_row_stride;      // ELEMENTS between rows of C
+    int64_t sa_chunk_stride;   // bytes between 32-row chunks of scale_a
+    int64_t a_batch, b_batch, c_batch, sa_batch, sb_batch;  // bytes between batches
+};
+
 // bias + activation + 16-bit conversion of four consecutive columns.  The variant is chosen at run time
 // (the epilogue is a vanishing part of any launch, so it is not worth a kernel instantiation per variant).
 template <int OUT, int EPI>

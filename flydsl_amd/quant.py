@@ -1,8 +1,10 @@
 """Host-side quantisers that feed the preshuffle GEMM (torch, any device).
 
 Same results as the reference's host utilities (``pertoken_quant`` tests/utils.py:29-73;
-``per_1x32_f4_quant`` and its codecs tests/kernels/utils/gemm_common_utils.py:14-71,142-275,675-704),
-written independently: the e2m1 rounding is a chain of threshold tests instead of fp32 bit tricks.
+``per_1x32_f4_quant`` and its codecs tests/kernels/utils/gemm_common_utils.py:14-71,142-275,675-704;
+``per_1x32_f6_quant`` / ``per_1x32_f8_quant`` / ``pack_fp6_e2m3`` / ``fp6_e2m3_to_f32`` :708-790),
+written independently: the e2m1 rounding is a chain of threshold tests and the e2m3 rounding a per-binade
+round-half-even instead of fp32 bit tricks.
 """
 
 from __future__ import annotations
@@ -112,3 +114,64 @@ def per_1x32_f4_quant(x, scale=None, quant_dtype=fp4x2, shuffle=False):
     packed = f32_to_mxfp4(y).view(torch.uint8).reshape(*shape[:-1], shape[-1] // 2).view(fp4x2)
     rows = x.reshape(-1, shape[-1]).shape[0]
     return packed, sc.view(torch.uint8).reshape(rows, -1).view(fp8_e8m0), y
+
+
+def f32_to_e2m3_codes(y: torch.Tensor) -> torch.Tensor:
+    """fp32 -> 6-bit e2m3 codes (uint8, one per element): nearest representable magnitude, ties to the even
+    mantissa, saturating at 7.5; sign in bit 5.  Magnitudes are spaced 1/8 below 2, 1/4 in [2, 4) and 1/2 above, and
+    the 5-bit magnitude code counts them in order, so each binade is one round-half-even."""
+    a = y.float().abs()
+    lo = torch.round(a * 8.0)
+    mid = 16.0 + torch.round((a - 2.0) * 4.0)
+    hi = 24.0 + torch.round((a - 4.0) * 2.0)
+    code = torch.where(a < 2.0, lo, torch.where(a < 4.0, mid, hi)).clamp(max=31.0).to(torch.uint8)
+    sign = (y.float().contiguous().view(torch.int32) < 0).to(torch.uint8) << 5
+    return code | sign
+
+
+def pack_fp6_e2m3(x_unpacked: torch.Tensor) -> torch.Tensor:
+    """uint8 codes (low 6 bits) ``[.., 4G]`` -> dense bytes ``[.., 3G]``; element j of each group of four sits at bits
+    [6j, 6j+6) of the group's 24 bits, least significant byte first."""
+    assert x_unpacked.dtype == torch.uint8 and x_unpacked.shape[-1] % 4 == 0
+    g = x_unpacked.reshape(*x_unpacked.shape[:-1], -1, 4).to(torch.int32) & 0x3F
+    word = g[..., 0] | (g[..., 1] << 6) | (g[..., 2] << 12) | (g[..., 3] << 18)
+    out = torch.stack([word & 0xFF, (word >> 8) & 0xFF, (word >> 16) & 0xFF], dim=-1).to(torch.uint8)
+    return out.reshape(*x_unpacked.shape[:-1], x_unpacked.shape[-1] // 4 * 3).contiguous()
+
+
+def fp6_e2m3_to_f32(x_unpacked: torch.Tensor) -> torch.Tensor:
+    """uint8 codes (low 6 bits: sign, 2 exponent bits with bias 1, 3 mantissa bits) -> fp32."""
+    c = (x_unpacked & 0x3F).to(torch.int32)
+    e, m = (c >> 3) & 3, (c & 7).float()
+    mag = torch.where(e == 0, m / 8.0, torch.ldexp(1.0 + m / 8.0, e - 1))
+    return torch.where((c & 0x20) != 0, -mag, mag)
+
+
+def per_1x32_f6_quant(x):
+    """OCP-MX fp6 (e2m3) quantisation of an A operand ``[M, K]``: scale byte = ``f32_to_e8m0(amax / 4)``, codes =
+    e2m3(x / 2^(scale-127)).  Returns ``(a_pad [M, K] uint8, scale [M, K/32] uint8, codes [M, K] uint8)`` like the
+    reference: ``a_pad`` holds per 32 elements the 24 packed bytes followed by 8 zero bytes, which is what the GEMM
+    reads.  Finite inputs only."""
+    shape = x.shape
+    blocks = x.reshape(-1, 32).float()
+    amax = blocks.abs().amax(dim=1)
+    sc = f32_to_e8m0(amax / 4.0)
+    y = blocks / e8m0_to_f32(sc).view(-1, 1)
+    codes = f32_to_e2m3_codes(y).reshape(shape).contiguous()
+    M, K = codes.shape[0], codes.shape[-1]
+    a_pad = torch.zeros(M, K // 32, 32, dtype=torch.uint8, device=x.device)
+    a_pad[:, :, :24] = pack_fp6_e2m3(codes).view(M, K // 32, 24)
+    return a_pad.view(M, K), sc.view(torch.uint8).reshape(M, -1), codes
+
+
+def per_1x32_f8_quant(x):
+    """OCP-MX fp8 (e4m3fn) quantisation: scale byte = ``f32_to_e8m0(max(amax, 1e-30) / 448)``, codes =
+    e4m3fn(clamp(x / 2^(scale-127), +-448)).  Returns ``(x_q [.., K] float8_e4m3fn, scale [.., K/32] uint8)``.
+    Finite inputs only."""
+    shape = x.shape
+    blocks = x.contiguous().reshape(-1, 32).float()
+    amax = blocks.abs().amax(dim=-1).clamp_min(1e-30)
+    sc = f32_to_e8m0(amax / 448.0)
+    sf = e8m0_to_f32(sc).clamp_min(1e-30)
+    x_q = (blocks / sf.view(-1, 1)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(shape).contiguous()
+    return x_q, sc.view(torch.uint8).reshape(*shape[:-1], shape[-1] // 32).contiguous()

@@ -66,6 +66,46 @@ def make_mxfp4(M, N, K, seed=0, w_std=0.02):
     }
 
 
+def make_mx(M, N, K, a_dtype="fp4", b_dtype="fp4", seed=0, w_std=0.02):
+    """MX operands in any supported format pair, built like the reference's harnesses
+    (tests/kernels/test_preshuffle_gemm.py:386-414 fp4, :507-527 fp6 x fp4, :630-647 fp8 x fp8): rows padded to 32
+    before quantisation, W and both scale arrays shuffled.  ``a_q`` / ``b_q`` are uint8 in the layout the GEMM reads
+    (fp4 packed nibbles, fp6 24+8-byte groups, fp8 bytes)."""
+    g = gen(seed)
+    x = torch.randn(M, K, generator=g, dtype=torch.float32)
+    w = torch.randn(N, K, generator=g, dtype=torch.float32) * w_std
+    xp = torch.zeros((M + 31) // 32 * 32, K)
+    xp[:M] = x
+    wp = torch.zeros((N + 31) // 32 * 32, K)
+    wp[:N] = w
+
+    def q(t, fmt):
+        if fmt == "fp4":
+            v, s, _ = quant.per_1x32_f4_quant(t)
+        elif fmt == "fp6":
+            v, s, _ = quant.per_1x32_f6_quant(t)
+        elif fmt == "fp8":
+            v, s = quant.per_1x32_f8_quant(t)
+        else:
+            raise ValueError(fmt)
+        return v.view(torch.uint8).contiguous(), s.view(torch.uint8).contiguous()
+
+    a_q, sa = q(xp, a_dtype)
+    b_q, sb = q(wp, b_dtype)
+    a_q, b_q = a_q[:M].contiguous(), b_q[:N].contiguous()
+    return {
+        "a_dtype": a_dtype,
+        "b_dtype": b_dtype,
+        "a_q": a_q,
+        "b_q": b_q,
+        "sa": sa,
+        "sb": sb,
+        "b_shuf": layout.shuffle_weight_w4(b_q, 16, False, False).contiguous(),
+        "sa_shuf": layout.shuffle_scale_w4(sa, 1, False).contiguous(),
+        "sb_shuf": layout.shuffle_scale_w4(sb, 1, False).contiguous(),
+    }
+
+
 def make_a16w16(M, N, K, kind, seed=0, w_std=1.0):
     """fp16 / bf16 operands (no quantisation, no scales), W preshuffled with the 2-byte layout."""
     g = gen(seed)

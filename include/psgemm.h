@@ -18,7 +18,8 @@
  *                       lib/Runtime/ROCm/FlyRocmRuntimeWrappers.cpp:58-64
  *   psg_gemm_a8w8_acc   no counterpart: the reference never exposes accumulators; this dumps them
  *                       (int32 for int8, fp32 for fp8) so parity tests can check them bit-exactly
- *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm), fp4 x fp4, batch 1
+ *   psg_gemm_mxfp4      kernels/gemm/mxfp4_preshuffle.py:57-488 (launch_gemm / kernel_gemm): fp4/fp6/fp8 A x fp4/fp8 W,
+ *                       caller strides, batch over grid.z
  *   psg_gemm_mxfp4_acc  no counterpart: fp32 accumulators of the MXFP4 mainloop, for parity tests
  *   psg_workspace_bytes no counterpart (the reference's preshuffle GEMM has no split-K path)
  *   psg_tile_coords     the workgroup-id -> tile remap xcd_remap_bx_by
@@ -39,7 +40,7 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 2
+#define PSG_ABI_VERSION 3
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
@@ -104,15 +105,34 @@ typedef struct psg_a8w8_args {
     int32_t pad0;       /* 0 */
 } psg_a8w8_args;
 
+/* Element formats of the MX GEMM's operands (kernels/gemm/mxfp4_preshuffle.py:70-72, a_dtype / b_dtype). */
+enum psg_mx_dtype { PSG_MX_FP4 = 0, PSG_MX_FP6 = 1, PSG_MX_FP8 = 2 };
+
 /*
- * Arguments of the MXFP4 preshuffle GEMM (fp4 e2m1 x fp4 e2m1, one e8m0 scale per 32 K elements).
- *   c        [M,N] row-major out_dtype
- *   a        [M,K/2] row-major packed e2m1, even k in the low nibble
- *   b        shuffle_weight_w4 of packed W[N,K/2] (same byte map as above with K/2 bytes per row)
- *   scale_a  shuffle_scale_w4 of e8m0 [ceil(M/32)*32, K/32]; scale_b the same over [N, K/32]
+ * Arguments of the MX preshuffle GEMM: A in fp4 (e2m1), fp6 (e2m3) or fp8 (e4m3fn), W in fp4 or fp8, one e8m0 scale
+ * per 32 K elements on both sides, optionally strided-batched (kernels/gemm/mxfp4_preshuffle.py:57-91).
+ *   c        [M,N] out_dtype, rows c_row_stride elements apart
+ *   a        rows a_row_stride bytes apart; a row is
+ *              fp4: K/2 bytes of packed e2m1, even k in the low nibble
+ *              fp8: K bytes of e4m3fn
+ *              fp6: K bytes: per 32 elements 24 bytes of packed e2m3 (element j at bits [6j, 6j+6) of the 192-bit
+ *                   little-endian group) followed by 8 bytes that are not read
+ *                   (tests/kernels/utils/gemm_common_utils.py pack_fp6_e2m3 + the fp8-sized padding of
+ *                   tests/kernels/test_preshuffle_gemm.py test_mfma_a6w4_preshuffle)
+ *   b        fp4: shuffle_weight_w4 of packed W[N,K/2]; fp8: shuffle_weight of W[N,K] (same 16x16-byte block map as
+ *            the 8-bit GEMM, K bytes per row)
+ *   scale_a  shuffle_scale_w4 of e8m0 [ceil(M/32)*32, K/32], 32-row chunks scale_a_chunk_stride bytes apart;
+ *            scale_b the same over [N, K/32], dense
  *            byte of S[r,kb] at (r/32)*32*(K/32) + (kb/8)*256 + (kb%4)*64 + (r%16)*4 + ((kb%8)/4)*2 + (r%32)/16
  *            (tests/kernels/utils/gemm_common_utils.py:645-672)
- *   N % 32 == 0, K % 256 == 0, 1 <= M <= 65536
+ *   N % 32 == 0, K % 256 == 0, 1 <= M <= 65536, 1 <= batch <= 65535 (0 is read as 1)
+ * Strides and batch: a stride of 0 means dense (a_row_stride = bytes of a row, c_row_stride = N,
+ * scale_a_chunk_stride = (K/256)*256, batch strides = the dense size of one batch: [B,M,*] for a / c,
+ * ceil(M/32) chunks for scale_a).  W and scale_b are always batch-dense (mxfp4_preshuffle.py:177-193).  Batch z reads
+ * a + z*a_batch_stride etc. (bytes) and all batches run in ONE launch (grid.z = batch).
+ * Which kernel runs: fp4 x fp4 with batch 1 and dense strides takes the tuned fp4 kernels (tiled mainloop, small-M
+ * split-K; workspace / tile_* / force_path 1, 2 apply to them only); everything else, or force_path 3, takes the
+ * general kernel, which ignores workspace and the tile arguments.
  */
 typedef struct psg_mxfp4_args {
     void *c;
@@ -126,8 +146,18 @@ typedef struct psg_mxfp4_args {
     int32_t out_dtype; /* enum psg_out_dtype */
     int32_t tile_m, tile_n, tile_k;
     int32_t xcd_swizzle;
-    int32_t force_path; /* 0 = auto, 1 = tiled, 2 = small-M */
+    int32_t force_path; /* 0 = auto, 1 = tiled (fp4 x fp4), 2 = small-M (fp4 x fp4), 3 = general kernel */
     int32_t reserved;
+    int32_t a_dtype;    /* enum psg_mx_dtype */
+    int32_t b_dtype;    /* PSG_MX_FP4 or PSG_MX_FP8 */
+    int32_t batch;      /* 0 or 1 = a single GEMM */
+    int32_t pad0;       /* 0 */
+    int64_t a_row_stride;         /* bytes; 0 = dense */
+    int64_t c_row_stride;         /* ELEMENTS; 0 = N */
+    int64_t scale_a_chunk_stride; /* bytes between 32-row chunks; 0 = dense */
+    int64_t a_batch_stride;       /* bytes; 0 = dense */
+    int64_t c_batch_stride;       /* bytes; 0 = dense */
+    int64_t scale_a_batch_stride; /* bytes; 0 = dense */
 } psg_mxfp4_args;
 
 /* ABI version of the loaded library (PSG_ABI_VERSION it was built with). */

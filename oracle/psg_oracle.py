@@ -120,22 +120,22 @@ def f32_to_e8m0(x: np.ndarray) -> np.ndarray:
     return exponent
 
 
-def f32_to_e2m1(x: np.ndarray) -> np.ndarray:
-    """fp32 -> 4-bit e2m1 code (one code per uint8), round-to-nearest-even, saturating to +-6.
+def f32_to_floatx(x: np.ndarray, ebits: int, mbits: int) -> np.ndarray:
+    """fp32 -> sign/ebits/mbits code in the low bits of a uint8, round-to-nearest-even, saturating to the largest
+    magnitude (no NaN / Inf codes).
 
-    Follows the bit-level algorithm of ``_f32_to_floatx_unpacked(x, 2, 1)``
-    (tests/kernels/utils/gemm_common_utils.py:162-275): saturate at >= 6, a denormal branch that
-    adds and subtracts a magic constant for |x| < 1, and a normal branch that re-biases the
-    exponent and adds a rounding bias with the tie bit.  Pinned against an independent
-    nearest-value search with ties-to-even on a dense sweep that contains every midpoint.
+    Follows the bit-level algorithm of ``_f32_to_floatx_unpacked``
+    (tests/kernels/utils/gemm_common_utils.py:162-275): saturate at >= max_normal, a denormal branch that adds and
+    subtracts a magic constant below min_normal, and a normal branch that re-biases the exponent and adds a rounding
+    bias with the tie bit.  Pinned for (2,1) and (2,3) against an independent nearest-value search with ties-to-even on
+    dense sweeps that contain every midpoint.
     """
     x = np.asarray(x, dtype=np.float32)
-    ebits, mbits = 2, 1
-    exp_bias = 1
-    max_int = 7
+    exp_bias = (1 << (ebits - 1)) - 1
+    max_int = (1 << (ebits + mbits)) - 1
     magic_adder = (1 << (23 - mbits - 1)) - 1
-    max_normal = 6.0
-    min_normal = 1.0
+    max_normal = 2.0 ** (((1 << ebits) - 1) - exp_bias) * (((1 << (mbits + 1)) - 1) / float(1 << mbits))
+    min_normal = 2.0 ** (1 - exp_bias)
     denorm_exp = (127 - exp_bias) + (23 - mbits) + 1
     denorm_mask_int = np.int32(denorm_exp << 23)
     denorm_mask_float = np.array(denorm_mask_int, dtype=np.int32).view(np.float32)
@@ -167,6 +167,51 @@ def f32_to_e2m1(x: np.ndarray) -> np.ndarray:
         np.uint8
     )
     return (out | sign_lp).astype(np.uint8)
+
+
+def f32_to_e2m1(x: np.ndarray) -> np.ndarray:
+    """fp32 -> 4-bit e2m1 code (one per uint8), RNE, saturating to +-6: ``_f32_to_floatx_unpacked(x, 2, 1)``."""
+    return f32_to_floatx(x, 2, 1)
+
+
+def f32_to_e2m3(x: np.ndarray) -> np.ndarray:
+    """fp32 -> 6-bit e2m3 code (one per uint8), RNE, saturating to +-7.5: ``_f32_to_floatx_unpacked(x, 2, 3)``
+    (tests/kernels/utils/gemm_common_utils.py:763)."""
+    return f32_to_floatx(x, 2, 3)
+
+
+def e2m3_to_f32(codes: np.ndarray) -> np.ndarray:
+    """6-bit e2m3 code (sign, 2 exponent bits with bias 1, 3 mantissa bits) -> fp32
+    (tests/kernels/utils/gemm_common_utils.py:727-741).  Pinned on all 64 codes against the format's definition
+    evaluated with ``ldexp`` and against the encoder's round trip."""
+    c = np.asarray(codes, dtype=np.uint8) & 0x3F
+    exp = ((c >> 3) & 0x3).astype(np.int32)
+    mant = (c & 0x7).astype(np.float32)
+    mag = np.where(exp == 0, mant / np.float32(8.0), np.ldexp(np.float32(1.0) + mant / np.float32(8.0), exp - 1))
+    return np.where((c & 0x20) != 0, -mag, mag).astype(np.float32)
+
+
+def pack_fp6(codes: np.ndarray) -> np.ndarray:
+    """Four 6-bit codes -> three bytes, little-endian bit order (element j of a group of four at bits [6j, 6j+6) of
+    the 24-bit group): ``pack_fp6_e2m3`` (tests/kernels/utils/gemm_common_utils.py:708-721).  Pinned against a
+    big-integer bit-string construction."""
+    c = np.asarray(codes, dtype=np.uint8)
+    assert c.shape[-1] % 4 == 0
+    g = (c.reshape(c.shape[:-1] + (-1, 4)).astype(np.uint32)) & 0x3F
+    word = g[..., 0] | (g[..., 1] << 6) | (g[..., 2] << 12) | (g[..., 3] << 18)
+    out = np.stack([word & 0xFF, (word >> 8) & 0xFF, (word >> 16) & 0xFF], axis=-1).astype(np.uint8)
+    return out.reshape(c.shape[:-1] + (c.shape[-1] // 4 * 3,))
+
+
+def unpack_fp6_padded(a_pad: np.ndarray) -> np.ndarray:
+    """Inverse of the A-operand layout of ``per_1x32_f6_quant``: ``[R, K]`` bytes (24 packed + 8 padding per 32
+    elements) -> ``[R, K]`` 6-bit codes.  Not in the reference; pinned as the inverse of ``pack_fp6``."""
+    p = np.asarray(a_pad, dtype=np.uint8)
+    r, k = p.shape
+    g = p.reshape(r, k // 32, 32)[:, :, :24].reshape(r, k // 32, 8, 3).astype(np.uint32)
+    word = g[..., 0] | (g[..., 1] << 8) | (g[..., 2] << 16)
+    codes = np.stack([(word >> (6 * j)) & 0x3F for j in range(4)], axis=-1)
+    return codes.reshape(r, k).astype(np.uint8)
 
 
 def pack_uint4(codes: np.ndarray) -> np.ndarray:
@@ -247,6 +292,49 @@ def per_1x32_f4_quant(x: np.ndarray):
     codes = f32_to_e2m1(y)
     packed = pack_uint4(codes.reshape(r, k))
     return packed, sc.reshape(r, k // 32)
+
+
+def per_1x32_f6_quant(x: np.ndarray):
+    """OCP-MX fp6 (e2m3) quantisation of an A operand (tests/kernels/utils/gemm_common_utils.py:744-770).
+
+    scale byte = ``f32_to_e8m0(amax / 4)`` (4 = 2^floor(log2 7.5)); codes = e2m3 RNE with saturation.  Returns
+    ``(a_pad [R, K] uint8, scale [R, K/32] uint8, codes [R, K] uint8)`` where ``a_pad`` holds per 32 elements the 24
+    packed bytes followed by 8 zero bytes (the layout the kernel reads).  Pinned through its parts plus composition
+    invariants (error at most half an e2m3 step at the chosen scale unless saturated; zero blocks -> scale 0, codes 0).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    r, k = x.shape
+    assert k % 32 == 0
+    blocks = x.reshape(-1, 32)
+    amax = np.abs(blocks).max(axis=1).astype(np.float32)
+    sc = f32_to_e8m0((amax / np.float32(4.0)).astype(np.float32))
+    sf = e8m0_to_f32(sc)
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = (blocks / sf[:, None]).astype(np.float32)
+    codes = f32_to_e2m3(y).reshape(r, k)
+    a_pad = np.zeros((r, k // 32, 32), dtype=np.uint8)
+    a_pad[:, :, :24] = pack_fp6(codes).reshape(r, k // 32, 24)
+    return a_pad.reshape(r, k), sc.reshape(r, k // 32), codes
+
+
+def per_1x32_f8_quant(x: np.ndarray):
+    """OCP-MX fp8 (e4m3fn) quantisation (tests/kernels/utils/gemm_common_utils.py:773-790).
+
+    ``amax`` clamped to >= 1e-30; scale byte = ``f32_to_e8m0(amax / 448)``; ``y = clamp(x / max(2^(s-127), 1e-30),
+    -448, 448)`` cast to e4m3fn (RNE).  Returns ``(codes [R, K] uint8, scale [R, K/32] uint8)``.  Pinned through its
+    parts plus composition invariants (block maximum decodes within one e4m3 step of itself; relative error of normal
+    values <= 2^-4).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    r, k = x.shape
+    assert k % 32 == 0
+    blocks = x.reshape(-1, 32)
+    amax = np.maximum(np.abs(blocks).max(axis=1).astype(np.float32), np.float32(1e-30))
+    sc = f32_to_e8m0((amax / np.float32(448.0)).astype(np.float32))
+    sf = np.maximum(e8m0_to_f32(sc), np.float32(1e-30))
+    with np.errstate(over="ignore", invalid="ignore"):
+        y = np.clip((blocks / sf[:, None]).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    return f32_to_e4m3fn(y).reshape(r, k), sc.reshape(r, k // 32)
 
 
 # ----------------------------------------------------------------------------------------------
@@ -358,6 +446,29 @@ def run_torch_w4(a_packed, b_packed, scale_a, scale_b) -> np.ndarray:
     UN-shuffled; scale arrays may have more rows than the operands (32-row padding)."""
     x = mxfp4_to_f32(a_packed)
     w = mxfp4_to_f32(b_packed)
+    xs = e8m0_to_f32(np.repeat(np.asarray(scale_a, dtype=np.uint8)[: x.shape[0]], 32, axis=1))
+    ws = e8m0_to_f32(np.repeat(np.asarray(scale_b, dtype=np.uint8)[: w.shape[0]], 32, axis=1))
+    return ((x * xs) @ (w * ws).T).astype(np.float32)
+
+
+def mx_operand_to_f32(q: np.ndarray, fmt: str) -> np.ndarray:
+    """Decode one MX operand to fp32 ``[R, K]``: ``fmt`` "fp4" (packed nibbles ``[R, K/2]``), "fp6" (the padded
+    ``[R, K]`` byte layout of ``per_1x32_f6_quant``) or "fp8" (e4m3fn bytes ``[R, K]``)."""
+    if fmt == "fp4":
+        return mxfp4_to_f32(q)
+    if fmt == "fp6":
+        return e2m3_to_f32(unpack_fp6_padded(q))
+    if fmt == "fp8":
+        return e4m3fn_to_f32(q)
+    raise ValueError(fmt)
+
+
+def run_torch_mx(a_q, b_q, scale_a, scale_b, a_fmt: str = "fp4", b_fmt: str = "fp4") -> np.ndarray:
+    """Parity oracle of the mixed-format MX GEMM: ``dequant(A) @ dequant(W)^T`` in fp32 with one e8m0 scale per 32 K
+    elements (tests/kernels/test_preshuffle_gemm.py:530-537 for fp6 x fp4, :650-653 for fp8 x fp8).  Operands and scales
+    are UN-shuffled; scale arrays may have more rows than the operands."""
+    x = mx_operand_to_f32(a_q, a_fmt)
+    w = mx_operand_to_f32(b_q, b_fmt)
     xs = e8m0_to_f32(np.repeat(np.asarray(scale_a, dtype=np.uint8)[: x.shape[0]], 32, axis=1))
     ws = e8m0_to_f32(np.repeat(np.asarray(scale_b, dtype=np.uint8)[: w.shape[0]], 32, axis=1))
     return ((x * xs) @ (w * ws).T).astype(np.float32)

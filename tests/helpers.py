@@ -5,7 +5,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from flydsl_amd.synthetic import make_a8w8, make_a16w16, make_mxfp4  # noqa: F401
+from flydsl_amd.synthetic import make_a8w8, make_a16w16, make_mx, make_mxfp4  # noqa: F401
 
 
 def np_bytes(t: torch.Tensor) -> np.ndarray:

@@ -109,15 +109,59 @@ def test_other_validation_errors():
     assert fn.N == 1024 and fn.K == 2048
 
 
-def test_mxfp4_entry_rejects_what_is_not_built():
+def test_mx_entry_validates_before_touching_the_gpu():
     base = [0, 0, 0, 0, 0, 32, 128, None, 128, 256, 32, 128, 256, "fp4", "bf16", "fp4", 1, -1, -1, -1, -1, -1, -1, 0]
-    for idx, val, exc in ((13, "fp8", NotImplementedError), (15, "fp8", NotImplementedError), (16, 0, ValueError),
-                          (17, 64, NotImplementedError), (12, 64, ValueError), (11, 64, ValueError), (14, "fp32", ValueError),
-                          (6, 256, ValueError)):
+    for idx, val in ((13, "fp5"), (15, "fp6"), (16, 0), (16, 70000), (12, 64), (11, 64), (14, "fp32"), (6, 256)):
         args = list(base)
         args[idx] = val
-        with pytest.raises(exc):
+        with pytest.raises(ValueError):
             launch_gemm(*args)
+
+
+def test_mx_c_abi_validation_codes():
+    handle = _lib.lib()
+    m = _lib.MxArgs()
+    m.c = m.a = m.b = m.scale_a = m.scale_b = 0x1000
+    m.M, m.N, m.K = 32, 128, 256
+    for field, val, code, word in (("a_dtype", 3, -3, b"a_dtype"), ("b_dtype", 1, -3, b"b_dtype"), ("batch", 70000, -2, b"batch"),
+                                   ("a_row_stride", 100, -2, b"a_row_stride"), ("a_row_stride", 120, -2, b"a_row_stride"),
+                                   ("c_row_stride", 64, -2, b"c_row_stride"), ("c_row_stride", 130, -2, b"c_row_stride"),
+                                   ("scale_a_chunk_stride", 128, -2, b"scale_a_chunk_stride"), ("a_batch_stride", 8, -6, b"batch strides"),
+                                   ("force_path", 4, -2, b"force_path"), ("pad0", 1, -2, b"pad0")):
+        old = getattr(m, field)
+        setattr(m, field, val)
+        assert handle.psg_gemm_mxfp4(ctypes.byref(m), None) == code, field
+        assert word in handle.psg_last_error(), (field, handle.psg_last_error())
+        setattr(m, field, old)
+    # the fp4-only paths refuse other formats, batches and strides
+    m.force_path, m.a_dtype = 1, 2
+    assert handle.psg_gemm_mxfp4(ctypes.byref(m), None) == -2 and b"fp4 x fp4" in handle.psg_last_error()
+    m.a_dtype, m.batch = 0, 2
+    assert handle.psg_gemm_mxfp4(ctypes.byref(m), None) == -2
+
+
+def test_mx_quantisers_match_the_oracle_byte_for_byte():
+    from flydsl_amd import quant
+    from oracle import psg_oracle as O
+
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((64, 256)) * rng.choice([1e-3, 1.0, 50.0], size=(64, 1))).astype(np.float32)
+    x[3, :32] = 0
+    a_pad, sc, codes = O.per_1x32_f6_quant(x)
+    tp, ts, tc = quant.per_1x32_f6_quant(torch.from_numpy(x))
+    assert np.array_equal(tp.numpy(), a_pad) and np.array_equal(ts.numpy(), sc) and np.array_equal(tc.numpy(), codes)
+    q, s8 = O.per_1x32_f8_quant(x)
+    tq, ts8 = quant.per_1x32_f8_quant(torch.from_numpy(x))
+    assert np.array_equal(tq.view(torch.uint8).numpy(), q) and np.array_equal(ts8.numpy(), s8)
+    # every midpoint between adjacent e2m3 magnitudes, and both neighbours of each
+    mags = O.e2m3_to_f32(np.arange(32, dtype=np.uint8))
+    mids = (mags[:-1] + mags[1:]) / 2
+    v = np.concatenate([mags, mids, np.nextafter(mids, np.float32(9)), np.nextafter(mids, np.float32(-9)), [7.75, 8.0, 1e3]]).astype(np.float32)
+    v = np.concatenate([v, -v])
+    assert np.array_equal(quant.f32_to_e2m3_codes(torch.from_numpy(v)).numpy(), O.f32_to_e2m3(v))
+    assert np.array_equal(quant.fp6_e2m3_to_f32(torch.arange(64, dtype=torch.uint8)).numpy(), O.e2m3_to_f32(np.arange(64, dtype=np.uint8)))
+    c = torch.from_numpy(rng.integers(0, 64, (4, 64), dtype=np.uint8))
+    assert np.array_equal(quant.pack_fp6_e2m3(c).numpy(), O.pack_fp6(c.numpy()))
 
 
 # ---- the C ABI -------------------------------------------------------------------------------------
@@ -276,8 +320,9 @@ def test_struct_layouts_match_header():
         printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(psg_a8w8_args), offsetof(psg_a8w8_args, workspace_bytes),
                offsetof(psg_a8w8_args, M), offsetof(psg_a8w8_args, epilogue), offsetof(psg_a8w8_args, force_path),
                offsetof(psg_a8w8_args, bias), offsetof(psg_a8w8_args, b_layout));
-        printf("%zu %zu %zu %zu\n", sizeof(psg_mxfp4_args), offsetof(psg_mxfp4_args, M), offsetof(psg_mxfp4_args, out_dtype),
-               offsetof(psg_mxfp4_args, force_path));
+        printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(psg_mxfp4_args), offsetof(psg_mxfp4_args, M), offsetof(psg_mxfp4_args, out_dtype),
+               offsetof(psg_mxfp4_args, force_path), offsetof(psg_mxfp4_args, a_dtype), offsetof(psg_mxfp4_args, batch),
+               offsetof(psg_mxfp4_args, a_row_stride), offsetof(psg_mxfp4_args, scale_a_batch_stride));
         return 0;
     }'''
     with tempfile.TemporaryDirectory() as d:
@@ -288,7 +333,8 @@ def test_struct_layouts_match_header():
         out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
     a, m = _lib.A8W8Args, _lib.MxArgs
     want = [ctypes.sizeof(a), a.workspace_bytes.offset, a.M.offset, a.epilogue.offset, a.force_path.offset, a.bias.offset,
-            a.b_layout.offset, ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset]
+            a.b_layout.offset, ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset,
+            m.a_dtype.offset, m.batch.offset, m.a_row_stride.offset, m.scale_a_batch_stride.offset]
     assert [int(v) for v in out] == want
 
 

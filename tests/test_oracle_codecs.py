@@ -106,3 +106,59 @@ def test_bf16_rounding_matches_library_cast():
     want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(O.f32_to_bf16_bits(x), want)
     assert np.array_equal(O.bf16_bits_to_f32(want), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+
+
+def _e2m3_magnitudes():
+    """The format's definition, stated with Fractions-free float64 arithmetic: exponent field 0 is subnormal (m/8),
+    otherwise 2^(e-1) * (1 + m/8)."""
+    return np.array([(m / 8.0) if e == 0 else (2.0 ** (e - 1)) * (1 + m / 8.0) for e in range(4) for m in range(8)])
+
+
+def test_e2m3_decode_all_codes():
+    mags = _e2m3_magnitudes()
+    assert mags[0] == 0 and mags[1] == 0.125 and mags[8] == 1.0 and mags[31] == 7.5 and (np.diff(mags) > 0).all()
+    want = np.concatenate([mags, -mags]).astype(np.float32)
+    got = O.e2m3_to_f32(np.arange(64, dtype=np.uint8))
+    assert np.array_equal(got, want) and np.signbit(got[32])
+    assert np.array_equal(O.e2m3_to_f32(np.arange(64, 256, dtype=np.uint8)), O.e2m3_to_f32(np.arange(64, 256, dtype=np.uint8) & 0x3F))
+
+
+def test_f32_to_e2m3_matches_bruteforce_nearest_even():
+    mags = _e2m3_magnitudes()
+    mids = ((mags[:-1] + mags[1:]) / 2).astype(np.float32)
+    near = np.concatenate([np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf))])
+    rng = np.random.default_rng(12)
+    x = np.concatenate([mags, mids, near, [7.5, 7.75, 8.0, 100.0, 1e-8, 0.0624, 0.0626], rng.uniform(0, 8, 6000)]).astype(np.float32)
+    x = np.concatenate([x, -x])
+    want = np.zeros(x.shape, dtype=np.uint8)
+    for i, v in enumerate(x.astype(np.float64)):
+        a = abs(v)
+        d = np.abs(mags - a)
+        best = np.flatnonzero(d == d.min())
+        code = best[0] if len(best) == 1 else [c for c in best if c % 2 == 0][0]  # tie -> even mantissa
+        if a >= 7.5:
+            code = 31
+        want[i] = code | (32 if np.signbit(np.float32(v)) else 0)
+    assert np.array_equal(O.f32_to_e2m3(x), want)
+    # the generic encoder with (2, 1) is the e2m1 encoder pinned above
+    assert np.array_equal(O.f32_to_floatx(x, 2, 1), O.f32_to_e2m1(x))
+
+
+def test_pack_fp6_against_bit_string():
+    rng = np.random.default_rng(13)
+    codes = rng.integers(0, 64, (3, 64), dtype=np.uint8)
+    packed = O.pack_fp6(codes)
+    assert packed.shape == (3, 48)
+    for r in range(3):
+        big = 0
+        for j, c in enumerate(codes[r].tolist()):
+            big |= c << (6 * j)  # element j at bits [6j, 6j+6) of one long little-endian integer
+        assert packed[r].tobytes() == big.to_bytes(48, "little")
+    # the spelled-out example of the reference's docstring: b0 = e1[1:0]<<6 | e0, b1 = e2[3:0]<<4 | e1>>2, b2 = e3<<2 | e2>>4
+    e = [0b101011, 0b110110, 0b011101, 0b100001]
+    assert O.pack_fp6(np.array([e], dtype=np.uint8)).tolist() == [[((e[1] & 3) << 6) | e[0], ((e[2] & 15) << 4) | (e[1] >> 2), (e[3] << 2) | (e[2] >> 4)]]
+    # padded layout round trip (24 packed + 8 padding bytes per 32 elements)
+    pad = np.zeros((3, 2, 32), dtype=np.uint8)
+    pad[:, :, :24] = packed.reshape(3, 2, 24)
+    pad[:, :, 24:] = 0xEE  # padding is never read
+    assert np.array_equal(O.unpack_fp6_padded(pad.reshape(3, 64)), codes)

@@ -125,6 +125,82 @@ def test_run_torch_w4_against_float64():
     assert np.allclose(O.run_torch_w4(ap, bp, sa, sb), want, rtol=1e-5, atol=1e-7)
 
 
+def test_per_1x32_f6_quant_invariants():
+    rng = np.random.default_rng(18)
+    x = (rng.standard_normal((8, 256)) * rng.choice([1e-4, 1.0, 50.0], (8, 1))).astype(np.float32)
+    x[2, 32:64] = 0.0
+    a_pad, sc, codes = O.per_1x32_f6_quant(x)
+    assert a_pad.shape == (8, 256) and sc.shape == (8, 8) and codes.shape == (8, 256)
+    assert not a_pad.reshape(8, 8, 32)[:, :, 24:].any()  # the 8 padding bytes are zero
+    assert np.array_equal(O.unpack_fp6_padded(a_pad), codes)
+    assert sc[2, 1] == 0 and not codes[2, 32:64].any()
+    scale = np.repeat(O.e8m0_to_f32(sc), 32, axis=1).astype(np.float64)
+    y = np.abs(x.astype(np.float64)) / scale
+    blk_max = np.abs(x).reshape(8, 8, 32).max(-1)
+    ratio = blk_max[sc > 0] / O.e8m0_to_f32(sc)[sc > 0]
+    assert (ratio > 2.0 * (1 - 1e-6)).all() and (ratio <= 6.0 * (1 + 1e-6)).all()  # same scale rule as fp4 (amax / 4)
+    deq = np.abs(O.e2m3_to_f32(codes).astype(np.float64))
+    half_step = np.where(y < 2, 0.0625, np.where(y < 4, 0.125, 0.25))
+    assert (np.abs(deq - y) <= half_step + 1e-9).all()  # never saturates: the block maximum is <= 6 < 7.5
+    assert (np.sign(O.e2m3_to_f32(codes)) * np.sign(x) >= 0).all()
+
+
+def test_per_1x32_f8_quant_invariants():
+    rng = np.random.default_rng(19)
+    x = (rng.standard_normal((8, 256)) * rng.choice([1e-4, 1.0, 50.0], (8, 1))).astype(np.float32)
+    x[2, 32:64] = 0.0
+    q, sc = O.per_1x32_f8_quant(x)
+    assert q.shape == (8, 256) and q.dtype == np.uint8 and sc.shape == (8, 8)
+    assert not (q[2, 32:64] & 0x7F).any()
+    # amax / 448 rounded to a power of two: the scaled block maximum lies in (448 * 2/3, 448 * 4/3]; what exceeds 448
+    # is clamped, so no code is NaN and every magnitude is at most 448
+    assert ((q & 0x7F) != 0x7F).all()
+    dec = O.e4m3fn_to_f32(q)
+    assert np.abs(dec).max() <= 448.0
+    sf = np.repeat(O.e8m0_to_f32(sc), 32, axis=1).astype(np.float64)
+    y = x.astype(np.float64) / sf
+    inside = (np.abs(y) <= 448) & (np.abs(y) >= 2.0**-6)
+    assert (np.abs(dec[inside] - y[inside]) <= np.abs(y[inside]) * 2.0**-4 + 1e-12).all()  # half an e4m3 step
+    clamped = np.abs(y) > 448
+    assert (np.abs(dec[clamped]) == 448).all()
+    # scale bytes by hand for two blocks: amax = 448 -> 2^0 (byte 127); amax = 3 -> 3/448 = 1.714 * 2^-8 -> rounds up to 2^-7
+    t = np.zeros((1, 64), dtype=np.float32)
+    t[0, 0], t[0, 32] = 448.0, 3.0
+    q2, s2 = O.per_1x32_f8_quant(t)
+    assert s2.tolist() == [[127, 120]] and q2[0, 0] == 0x7E and O.e4m3fn_to_f32(q2[:, 32])[0] == 384.0
+
+
+def test_run_torch_mx_against_float64():
+    rng = np.random.default_rng(20)
+    x = rng.standard_normal((5, 64)).astype(np.float32)
+    w = (rng.standard_normal((7, 64)) * 0.02).astype(np.float32)
+    a6, sa6, c6 = O.per_1x32_f6_quant(x)
+    a8, sa8 = O.per_1x32_f8_quant(x)
+    b4, sb4 = O.per_1x32_f4_quant(w)
+    b8, sb8 = O.per_1x32_f8_quant(w)
+    e2m3 = np.concatenate([[(m / 8.0) if e == 0 else (2.0 ** (e - 1)) * (1 + m / 8.0) for e in range(4) for m in range(8)]] * 2)
+    e2m3[32:] *= -1
+    e2m1 = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6])
+    e4m3 = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).double().numpy()
+
+    def val(q, s, fmt, i, t):
+        if fmt == "fp4":
+            v = e2m1[(q[i, t // 2] >> (4 * (t % 2))) & 15]
+        elif fmt == "fp6":  # bits [6j, 6j+6) of the 24-byte group
+            grp = int.from_bytes(q[i, 32 * (t // 32): 32 * (t // 32) + 24].tobytes(), "little")
+            v = e2m3[(grp >> (6 * (t % 32))) & 63]
+        else:
+            v = e4m3[q[i, t]]
+        return v * 2.0 ** (int(s[i, t // 32]) - 127)
+
+    for (aq, sa, af), (bq, sb, bf) in [((a6, sa6, "fp6"), (b4, sb4, "fp4")), ((a8, sa8, "fp8"), (b8, sb8, "fp8")),
+                                       ((a8, sa8, "fp8"), (b4, sb4, "fp4")), ((a6, sa6, "fp6"), (b8, sb8, "fp8"))]:
+        want = np.array([[sum(val(aq, sa, af, i, t) * val(bq, sb, bf, j, t) for t in range(64)) for j in range(7)] for i in range(5)])
+        assert np.allclose(O.run_torch_mx(aq, bq, sa, sb, af, bf), want, rtol=1e-5, atol=1e-7)
+    a4, sa4 = O.per_1x32_f4_quant(x)
+    assert np.array_equal(O.run_torch_mx(a4, b4, sa4, sb4), O.run_torch_w4(a4, b4, sa4, sb4))
+
+
 def test_activations_against_library():
     v = np.linspace(-12, 12, 4001).astype(np.float32).reshape(1, -1)
     t = torch.from_numpy(v)
