@@ -230,7 +230,14 @@ def run_quant_workload(name, steps=50, warmup=5):
     graph.replay()
     ev1.record()
     torch.cuda.synchronize()
-    sec = ev0.elapsed_time(ev1) * 1e-3 / steps
+    # one timed probe replay sizes the number of replays so that the timed region holds at least MIN_TIMED_S of work
+    replays = max(1, math.ceil(MIN_TIMED_S / max(ev0.elapsed_time(ev1) * 1e-3, 1e-7)))
+    ev0.record()
+    for _r in range(replays):
+        graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    sec = ev0.elapsed_time(ev1) * 1e-3 / (steps * replays)
     if kind == "fp8":
         wy, ws = O.pertoken_quant(host.float().numpy(), "fp8")
         ok = bool(np.array_equal(out[0].view(torch.uint8).cpu().numpy(), wy) and np.array_equal(out[1].cpu().numpy(), ws))

@@ -42,6 +42,11 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
     const int m0 = ((int)blockIdx.x / tiles_n) * TM, n0 = ((int)blockIdx.x % tiles_n) * TN;
     const uint64_t z = blockIdx.z;
     const int KT = p.K >> 7;                                   // 128-element steps (even: K % 256 == 0)
+    // split-K: workgroup blockIdx.y of p.splits covers the steps [kt_begin, kt_end), a whole number of 256-K scale chunks,
+    // and (STORE_ACC only) writes its accumulators to slice blockIdx.y of the partials buffer
+    const int kt_per = (((KT >> 1) + p.splits - 1) / p.splits) << 1;
+    const int kt_begin = (int)blockIdx.y * kt_per;
+    const int kt_end = (kt_begin + kt_per) < KT ? (kt_begin + kt_per) : KT;
     const uint32_t a_row_bytes = AF == MXF_FP4 ? (uint32_t)p.K >> 1 : (uint32_t)p.K;
     const uint32_t b_row_bytes = BF == MXF_FP4 ? (uint32_t)p.K >> 1 : (uint32_t)p.K;
     const uint32_t a_rs = (uint32_t)p.a_row_stride;
@@ -72,7 +77,7 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
             const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
-            const bool ok = row < TM && kt < KT;
+            const bool ok = row < TM && kt < kt_end;
             areg[j] = buf_load16(ra, ok ? (uint32_t)row * a_rs + (uint32_t)kc * 16u : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
         }
     };
@@ -88,7 +93,7 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
     auto load_b = [&](int kt, v8i* dst) {
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
-            const bool ok = kt < KT;
+            const bool ok = kt < kt_end;
             v8i v = {0, 0, 0, 0, 0, 0, 0, 0};
             if constexpr (BF == MXF_FP4) {
                 const v4i x = buf_load16(rb, ok ? (uint32_t)lane * 16u + (uint32_t)ni * 16u * b_row_bytes : 0xFFFFFFF0u, ok ? (uint32_t)kt * 1024u : 0u);
@@ -105,7 +110,7 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
     // scale dwords of a 256-K chunk kc: MR/2 on the A side, NR/2 on the W side
     int sav[2][MR / 2], sbv[2][NR / 2];
     auto load_sc = [&](int kc, int* sa_dst, int* sb_dst) {
-        const bool ok = kc < (KT >> 1);
+        const bool ok = kc < (kt_end >> 1);
 #pragma unroll
         for (int q = 0; q < MR / 2; q++) sa_dst[q] = buf_load4(rsa, ok ? (uint32_t)q * sa_cs + (uint32_t)lane * 4u : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u);
 #pragma unroll
@@ -154,17 +159,17 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
         __syncthreads();
     };
 
-    load_a(0);
-    load_b(0, bw[0]);
-    load_sc(0, sav[0], sbv[0]);
+    load_a(kt_begin);
+    load_b(kt_begin, bw[0]);
+    load_sc(kt_begin >> 1, sav[0], sbv[0]);
     store_a(0);
     __syncthreads();
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
-    for (int kt = 0; kt < KT; kt += 4) {  // two scale chunks per trip, so every register index is a constant
+    for (int kt = kt_begin; kt < kt_end; kt += 4) {  // two scale chunks per trip, so every register index is a constant
         step(kt, I0{}, I0{});
         step(kt + 1, I1{}, I0{});
-        if (kt + 2 < KT) {
+        if (kt + 2 < kt_end) {
             step(kt + 2, I0{}, I1{});
             step(kt + 3, I1{}, I1{});
         }
@@ -181,7 +186,8 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
             if (m < p.M && n < p.N) {
                 const v4f v = acc[mi][ni];
                 if constexpr (STORE == STORE_ACC) {
-                    *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cbase) + (size_t)m * (size_t)p.N + (size_t)n) = v;
+                    const size_t slice = (size_t)blockIdx.y * (size_t)p.M * (size_t)p.N;
+                    *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cbase) + slice + (size_t)m * (size_t)p.N + (size_t)n) = v;
                 } else {
                     const v2i r = p.out == OUT_BF16 ? pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]) : pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
                     *reinterpret_cast<v2i*>(reinterpret_cast<uint16_t*>(cbase) + (int64_t)m * c_rs + n) = r;
@@ -194,12 +200,13 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
 template <int AF, int BF, int STORE>
 hipError_t launch_fmt(const MxGenParams& p, int batch, hipStream_t stream) {
     // 64x128 tiles (32x128 when M <= 32)
+    const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     if (p.M <= 32) {
         const int tiles = ((p.M + 31) / 32) * ((p.N + 127) / 128);
-        hipLaunchKernelGGL((k_mx_generic<AF, BF, 2, 2, STORE>), dim3(tiles, 1, batch), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((k_mx_generic<AF, BF, 2, 2, STORE>), dim3(tiles, splits, batch), dim3(256), 0, stream, p);
     } else {
         const int tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
-        hipLaunchKernelGGL((k_mx_generic<AF, BF, 4, 2, STORE>), dim3(tiles, 1, batch), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((k_mx_generic<AF, BF, 4, 2, STORE>), dim3(tiles, splits, batch), dim3(256), 0, stream, p);
     }
     return hipGetLastError();
 }

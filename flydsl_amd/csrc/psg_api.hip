@@ -67,8 +67,9 @@ struct Tile {
 // Tile choice for the MFMA mainloop.  Each shape has a measured relative efficiency at full occupancy.  The 256x256
 // tile of eight wavefronts side by side along N loads every W fragment once per CU and moves the least data per flop:
 // on real data the chip is power-limited, so that is what decides (fp8 8192x4096x4096: 117 us against 134 us for
-// the 128x256 tile that runs two workgroups per CU; int8 4096x28672x8192: 775 against 940).  For MXFP4 the launch is
-// bound by the C stores and the 4- and 8-wavefront forms measure the same.  The score multiplies the efficiency by
+// the 128x256 tile that runs two workgroups per CU; int8 4096x28672x8192: 775 against 940).  MXFP4 4096x7168x2048:
+// 45 us with eight wavefronts against 52 with four, and 82 for the 128x256 tile, whose two workgroups per CU ask the
+// L2 for 47 bytes per clock at fp4 MFMA speed.  The score multiplies the efficiency by
 // how evenly the tiles fill the CUs' workgroup slots and by the fraction of each tile that is not padding.
 Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     struct Shape {
@@ -77,7 +78,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     };
     static const Shape shapes8[] = {{256, 256, 8, 1, 1.17}, {128, 256, 4, 2, 1.00}, {64, 256, 4, 2, 0.62}, {32, 256, 4, 3, 0.36},
                                     {128, 128, 4, 2, 0.70}, {64, 64, 4, 5, 0.25}};
-    static const Shape shapesx[] = {{256, 256, 4, 1, 1.00}, {128, 256, 4, 2, 0.86}, {64, 256, 4, 2, 0.80}, {32, 256, 4, 3, 0.40},
+    static const Shape shapesx[] = {{256, 256, 8, 1, 1.00}, {128, 256, 4, 2, 0.86}, {64, 256, 4, 2, 0.80}, {32, 256, 4, 3, 0.40},
                                     {64, 128, 4, 3, 0.40}, {32, 128, 4, 4, 0.25}};
     const Shape* shapes = mx ? shapesx : shapes8;
     if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n, 4};  // forced by the caller; the launcher rejects unknown shapes
@@ -114,6 +115,18 @@ int pick_splits(int M, int N, int kbytes, Tile t) {
     // measured optimum: about 16 K steps per workgroup, at most ~1024 workgroups, partial traffic bounded
     int s = 1;
     while (s < 8 && steps / (s * 2) >= 16 && tiles * (s * 2) <= 1024 && (long)(s * 2) * M * 16 <= kbytes) s *= 2;
+    return s;
+}
+
+// Split-K for the general MX kernel: its tiles are 64x128 (32x128 for M <= 32), so decode-like shapes launch few
+// workgroups; K is split until about two workgroups per CU exist, every split keeps at least eight 128-element steps
+// and the fp32 partials (written and read back once) stay below a quarter of the bytes of an fp4 W.
+int mx_general_splits(int M, int N, int K) {
+    const uint64_t w_bytes = (uint64_t)N * (uint64_t)K / 2;  // of fp4 W; fp8 W gets the same plan
+    const long tiles = (long)((M + (M <= 32 ? 31 : 63)) / (M <= 32 ? 32 : 64)) * (long)((N + 127) / 128);
+    const int steps = K / 128;
+    int s = 1;
+    while (s < 8 && tiles * (s * 2) <= 512 && steps / (s * 2) >= 8 && (uint64_t)(s * 2) * (uint64_t)M * (uint64_t)N * 8ull <= w_bytes / 4) s *= 2;
     return s;
 }
 
@@ -156,7 +169,7 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
     if (acc_only) {
         if (!aligned(acc, 16)) return fail(PSG_E_ALIGN, "acc must be 16-byte aligned");
     } else {
-        if (!aligned(a->c, 8)) return fail(PSG_E_ALIGN, "c must be 8-byte aligned");
+        if (!aligned(a->c, 16)) return fail(PSG_E_ALIGN, "c must be 16-byte aligned");
         if (!is16 && !aligned(a->scale_b, 16)) return fail(PSG_E_ALIGN, "scale_b must be 16-byte aligned");
         if (!is16 && !aligned(a->scale_a, 4)) return fail(PSG_E_ALIGN, "scale_a must be 4-byte aligned");
         if (a->epilogue != PSG_EPI_NONE && !aligned(a->bias, 8)) return fail(PSG_E_ALIGN, "bias must be 8-byte aligned");
@@ -248,6 +261,7 @@ const char* psg_last_error(void) { return g_err; }
 uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) {
     // Only the split-K variant of the tiled path (few tiles, long K) uses global scratch: one fp32 / int32 slice of
     // [M,N] per split.  Without it (NULL or too small) the library runs the same problem unsplit.
+    if (in_dtype == 5) return M >= 1 && N >= 32 && K >= 256 ? splitk_bytes(M, N, mx_general_splits(M, N, K)) : 0;  // general MX kernel
     if (M <= kSmallM || M < 1 || N < 16 || K < 64) return 0;
     const bool mx = in_dtype == 4;  // MXFP4 (psg_gemm_mxfp4)
     const int kbytes = mx ? K / 2 : ((in_dtype == PSG_IN_FP16 || in_dtype == PSG_IN_BF16) ? K * 2 : K);
@@ -345,7 +359,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         return fail(PSG_E_ALIGN, "batch strides must keep a 16-byte, c 8-byte and scale_a 4-byte aligned");
     if (!aligned(a->a, 16) || !aligned(a->b, 16)) return fail(PSG_E_ALIGN, "a and b must be 16-byte aligned");
     if (!aligned(a->scale_a, 4) || !aligned(a->scale_b, 4)) return fail(PSG_E_ALIGN, "scales must be 4-byte aligned");
-    if (!aligned(out, store == STORE_ACC ? 16 : 8)) return fail(PSG_E_ALIGN, "output must be %d-byte aligned", store == STORE_ACC ? 16 : 8);
+    if (!aligned(out, 16)) return fail(PSG_E_ALIGN, "output must be 16-byte aligned");
     if (a->force_path < 0 || a->force_path > 3) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
     const bool dense = a_rs == a_row && c_rs == (uint64_t)a->N && sa_cs == chunk;
     const bool fp4_fast = a->a_dtype == PSG_MX_FP4 && a->b_dtype == PSG_MX_FP4 && batch == 1 && dense;
@@ -363,6 +377,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         g.N = a->N;
         g.K = a->K;
         g.out = a->out_dtype;
+        g.splits = 1;
         g.a_row_stride = (int64_t)a_rs;
         g.c_row_stride = (int64_t)c_rs;
         g.sa_chunk_stride = (int64_t)sa_cs;
@@ -371,7 +386,25 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         g.c_batch = store == STORE_ACC ? (int64_t)a->M * a->N * 4 : (a->c_batch_stride ? a->c_batch_stride : (int64_t)((uint64_t)a->M * c_rs * 2));
         g.sa_batch = a->scale_a_batch_stride ? a->scale_a_batch_stride : (int64_t)((uint64_t)((a->M + 31) / 32) * sa_cs);
         g.sb_batch = (int64_t)((uint64_t)(a->N / 32) * chunk);
-        const hipError_t ge = psg_launch_mx_generic(g, a->a_dtype, a->b_dtype, store, batch, static_cast<hipStream_t>(stream));
+        hipError_t ge;
+        const int splits = batch == 1 && c_rs == (uint64_t)a->N && store == STORE_C ? mx_general_splits(a->M, a->N, a->K) : 1;
+        if (splits > 1 && a->workspace && aligned(a->workspace, 16) && a->workspace_bytes >= splitk_bytes(a->M, a->N, splits)) {
+            MxGenParams part = g;
+            part.c = a->workspace;
+            part.splits = splits;
+            ge = psg_launch_mx_generic(part, a->a_dtype, a->b_dtype, STORE_ACC, 1, static_cast<hipStream_t>(stream));
+            A8W8Params q{};
+            q.c = out;
+            q.M = a->M;
+            q.N = a->N;
+            q.K = a->K;
+            q.splits = splits;
+            q.epi = EPI_NONE;
+            q.out = a->out_dtype;
+            if (ge == hipSuccess) ge = psg_launch_splitk_finalize(q, a->workspace, 0, 0, static_cast<hipStream_t>(stream));
+        } else {
+            ge = psg_launch_mx_generic(g, a->a_dtype, a->b_dtype, store, batch, static_cast<hipStream_t>(stream));
+        }
         if (ge != hipSuccess) return hip_fail(ge, "psg_gemm_mxfp4 launch");
         g_err[0] = 0;
         return 0;
@@ -414,7 +447,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         q.K = p.K;
         q.group_m = p.group_m;
         q.ksplit = 1;
-        q.wave_layout = a->reserved >= 2 ? a->reserved : 1;
+        q.wave_layout = a->reserved >= 2 ? a->reserved : (!forced && t.waves == 8 ? 8 : 1);
         q.splits = splits;
         q.epi = EPI_NONE;
         q.out = p.out;

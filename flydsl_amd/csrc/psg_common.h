@@ -137,6 +137,7 @@ struct MxGenParams {
     const uint8_t* sb;
     int M, N, K;
     int out;             // OUT_*
+    int splits;          // workgroups along K per tile (> 1 only with STORE_ACC into a partials buffer, batch 1)
     int64_t a_row_stride;      // bytes between rows of A
     int64_t c_row_stride;      // ELEMENTS between rows of C
     int64_t sa_chunk_stride;   // bytes between 32-row chunks of scale_a

@@ -60,6 +60,7 @@ def launch_gemm(
     _acc=None,
     _wave_layout=0,
     _splits=0,
+    _no_split=False,
 ):
     """Launch ``C[b] = A_mx[b] @ W_mx[b]^T`` (``[M,K] x [N,K]``) for every batch ``b`` on ``stream``.  The reference's
     constraints are kept: ``tile_k in {128, 256}``, ``tile_n % 128 == 0``, ``K % tile_k == 0``
@@ -128,9 +129,13 @@ def launch_gemm(
             need = args.tile_k * args.M * args.N * 4 if args.tile_k > 1 else 0
         else:
             need = lib.psg_workspace_bytes(args.M, args.N, args.K, 4)
-        if need and _acc is None and hasattr(arg_c, "device"):
-            ws = _lib.workspace(arg_c.device, need, h, owner="mxfp4")
-            args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    elif B == 1 and c_rs == Nn and not _no_split:
+        need = lib.psg_workspace_bytes(args.M, args.N, args.K, 5)
+    else:
+        need = 0
+    if need and _acc is None and hasattr(arg_c, "device"):
+        ws = _lib.workspace(arg_c.device, need, h, owner="mxfp4")
+        args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
     if _acc is None:
         rc = lib.psg_gemm_mxfp4(ctypes.byref(args), h)
     else:

@@ -132,7 +132,8 @@ enum psg_mx_dtype { PSG_MX_FP4 = 0, PSG_MX_FP6 = 1, PSG_MX_FP8 = 2 };
  * a + z*a_batch_stride etc. (bytes) and all batches run in ONE launch (grid.z = batch).
  * Which kernel runs: fp4 x fp4 with batch 1 and dense strides takes the tuned fp4 kernels (tiled mainloop, small-M
  * split-K; workspace / tile_* / force_path 1, 2 apply to them only); everything else, or force_path 3, takes the
- * general kernel, which ignores workspace and the tile arguments.
+ * general kernel, which ignores the tile arguments and uses workspace (psg_workspace_bytes(M, N, K, 5) bytes) for
+ * split-K when batch is 1 and C is dense.
  */
 typedef struct psg_mxfp4_args {
     void *c;
@@ -167,7 +168,8 @@ int psg_abi_version(void);
 const char *psg_last_error(void);
 
 /* Bytes of workspace the split-K plan would use for this problem (0 when the chosen plan needs none).
- * in_dtype: enum psg_in_dtype, or 4 for psg_gemm_mxfp4. */
+ * in_dtype: enum psg_in_dtype, 4 for psg_gemm_mxfp4 on its fp4 x fp4 kernels, 5 for psg_gemm_mxfp4 on the general MX
+ * kernel (any other format pair, or force_path 3; batch 1 and dense C only, otherwise it runs unsplit). */
 uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype);
 
 /* C = epilogue((acc * scale_a[m]) * scale_b[n]) on `stream` (a hipStream_t passed as void*). */

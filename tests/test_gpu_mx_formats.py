@@ -115,6 +115,32 @@ def test_scale_extremes_select_the_right_scale_byte():
         assert np.allclose(acc, ref, rtol=1e-4, atol=_acc_atol(d, ref) * 0.1), (a_dtype, b_dtype)
 
 
+@pytest.mark.parametrize("a_dtype,b_dtype", [("fp8", "fp8"), ("fp6", "fp4")])
+def test_split_k_of_the_general_kernel(a_dtype, b_dtype):
+    # decode-like shape: few tiles, long K -> K is split over workgroups, partials reduced in a fixed order
+    from flydsl_amd import _lib
+    from kernels.gemm.mxfp4_preshuffle import launch_gemm
+
+    M, N, K = 32, 512, 8192
+    need = _lib.lib().psg_workspace_bytes(M, N, K, 5)
+    assert need == 4 * M * N * 4  # four splits
+    d = make_mx(M, N, K, a_dtype, b_dtype, seed=9, w_std=1.0)
+    ref = _ref(d)
+    dev = torch.device("cuda")
+    outs = []
+    for no_split in (False, True):
+        c = torch.full((M + 8, N), SENTINEL, dtype=torch.bfloat16, device=dev)
+        for _ in range(2):  # the second call reuses the parked workspace
+            launch_gemm(c, d["a_q"].to(dev), d["b_shuf"].to(dev), d["sa_shuf"].to(dev), d["sb_shuf"].to(dev), M, N, torch.cuda.current_stream(),
+                        N, K, 32, 128, 256, a_dtype, "bf16", b_dtype, 1, -1, -1, -1, -1, -1, -1, 0, 0, _no_split=no_split)
+        torch.cuda.synchronize()
+        _check(c[:M].float().cpu().numpy(), ref)
+        assert (c[M:] == SENTINEL).all()
+        outs.append(c[:M].float().cpu().numpy())
+    # split and unsplit sums differ only by fp32 summation order
+    assert np.abs(outs[0] - outs[1]).max() <= 2e-2 * np.abs(ref).max()
+
+
 def test_fp6_padding_bytes_are_not_read():
     M, N, K = 40, 128, 512
     d = make_mx(M, N, K, "fp6", "fp4", seed=6)
