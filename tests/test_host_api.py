@@ -164,6 +164,17 @@ def test_mx_quantisers_match_the_oracle_byte_for_byte():
     assert np.array_equal(quant.pack_fp6_e2m3(c).numpy(), O.pack_fp6(c.numpy()))
 
 
+def test_fp4_4wave_call_shape_keeps_the_reference_asserts():
+    from kernels.gemm.fp4_gemm_4wave import compile_fp4_gemm_4w
+
+    assert compile_fp4_gemm_4w(K=2048).K == 2048 and compile_fp4_gemm_4w(K=512, MN=(256, 256)).MN == (256, 256)
+    for bad in (300, 1280 + 256 * 0 + 128, 256 * 5, 256 * 7):  # not a multiple of 256; odd K-step counts
+        with pytest.raises(AssertionError):
+            compile_fp4_gemm_4w(K=bad)
+    with pytest.raises(TypeError):
+        compile_fp4_gemm_4w(2048)  # keyword-only like the reference
+
+
 # ---- the C ABI -------------------------------------------------------------------------------------
 def _declared_functions():
     text = open(HEADER).read()
