@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -32,6 +32,8 @@ EXPORTS = (
     "psg_gemm_a8w8_static",
     "psg_tile_coords",
     "psg_debug_tile_order",
+    "psg_moe_gemm",
+    "psg_moe_reduce",
 )
 
 
@@ -96,6 +98,34 @@ class MxArgs(ctypes.Structure):
 
 MX_DTYPE = {"fp4": 0, "fp6": 1, "fp8": 2}
 
+
+class MoeArgs(ctypes.Structure):
+    _fields_ = [
+        ("out", ctypes.c_void_p),
+        ("x", ctypes.c_void_p),
+        ("w", ctypes.c_void_p),
+        ("scale_x", ctypes.c_void_p),
+        ("scale_w", ctypes.c_void_p),
+        ("sorted_token_ids", ctypes.c_void_p),
+        ("sorted_expert_ids", ctypes.c_void_p),
+        ("sorted_weights", ctypes.c_void_p),
+        ("num_valid_ids", ctypes.c_void_p),
+        ("tokens", ctypes.c_int32),
+        ("topk", ctypes.c_int32),
+        ("experts", ctypes.c_int32),
+        ("model_dim", ctypes.c_int32),
+        ("inter_dim", ctypes.c_int32),
+        ("sorted_size", ctypes.c_int32),
+        ("blocks", ctypes.c_int32),
+        ("block_m", ctypes.c_int32),
+        ("in_dtype", ctypes.c_int32),
+        ("out_dtype", ctypes.c_int32),
+        ("stage", ctypes.c_int32),
+        ("doweight", ctypes.c_int32),
+        ("accumulate", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
+    ]
+
 _lib = None
 
 
@@ -125,7 +155,9 @@ def lib() -> ctypes.CDLL:
     handle.psg_tile_coords.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
     handle.psg_debug_tile_order.restype = ctypes.c_int
     handle.psg_debug_tile_order.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
-    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static"):
+    handle.psg_moe_reduce.restype = ctypes.c_int
+    handle.psg_moe_reduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int32] * 4 + [ctypes.c_void_p]
+    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]

@@ -1,0 +1,276 @@
+// MoE grouped GEMMs for gfx950 over expert-sorted token blocks, int8 or OCP fp8 operands with per-row fp32 scales.
+//
+// The sorted row list (one entry per routed (token, slot), padded per expert to whole blocks of BM rows) says which
+// row of x each tile row reads; one expert id per block says which slab of the preshuffled weights it multiplies.
+//   stage 1 (gate-up): y[t, slot, n] = silu(g) * u with g = x[t] . W1[e, n], u = x[t] . W1[e, inter + n]
+//   stage 2 (down):    y[n] = a2[t, slot] . W2[e, n] (* routing weight); added atomically into out[t] or written to
+//                      out[t*topk + slot]
+// Workgroup = four wavefronts side by side along N, tile BM x 64*NR, 128 bytes of K per step.  The A rows are
+// gathered (per-row offsets through a bounds-checked buffer descriptor: padding rows read zeros) into a two-stage
+// XOR-swizzled LDS tile; W fragments go straight from the expert's slab into MFMA operand registers (lane l reads
+// bytes [16l, 16l+16) of a 1 KB block, the same wire format as the plain GEMM).  Stage 1 keeps two accumulators per
+// fragment (gate and up) so silu(g)*u happens in registers.
+#include "psg_common.h"
+
+namespace {
+
+typedef __fp16 v2h __attribute__((ext_vector_type(2)));
+typedef __bf16 v2b __attribute__((ext_vector_type(2)));
+
+template <int KIND>
+struct MoeAcc {
+    using type = v4f;
+};
+template <>
+struct MoeAcc<KIND_INT8> {
+    using type = v4i;
+};
+
+__device__ __forceinline__ int moe_lds_off(int row, int kc) { return row * 128 + ((kc ^ ((row >> 1) & 7)) << 4); }
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+template <int KIND, int MR, int NR, int STAGE>
+__global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
+    using acc_t = typename MoeAcc<KIND>::type;
+    constexpr int BM = 16 * MR, TN = 64 * NR;
+    constexpr int NSET = STAGE == 1 ? 2 : 1;           // gate and up
+    constexpr int A_LOADS = (BM * 8 + 255) / 256;      // 16-byte chunks of the A tile per thread
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * 128];
+    __shared__ int ids[BM];
+
+    const int tid = threadIdx.x;
+    const int wave = wave_id();
+    const int lane = tid & 63, li = lane & 15, lg = lane >> 4;
+    const int blk = (int)blockIdx.y;
+    const int n0 = (int)blockIdx.x * TN;
+    if (blk * BM >= p.num_valid[0]) return;            // uniform: blocks past the sorted rows in use
+    const int e = p.expert_ids[blk];
+    if (e < 0 || e >= p.experts) return;               // uniform: a block without an expert
+
+    if (tid < BM) {
+        const int q = blk * BM + tid;
+        ids[tid] = q < p.sorted_size ? p.sorted_ids[q] : p.tokens;  // past the list = a padding row
+    }
+    __syncthreads();
+
+    // row of x (and of its scale) a tile row reads, or -1 for a padding row
+    auto x_row = [&](int r) {
+        const uint32_t sid = (uint32_t)ids[r];
+        const int t = (int)(sid & 0xFFFFFFu), s = (int)(sid >> 24);
+        if (t >= p.tokens || s >= p.topk) return -1;
+        return STAGE == 1 ? t : t * p.topk + s;
+    };
+
+    const int K = p.K, KT = K >> 7;
+    const int rows_x = STAGE == 1 ? p.tokens : p.tokens * p.topk;
+    const int rows_e = STAGE == 1 ? 2 * p.n_out : p.n_out;            // weight rows per expert
+    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.x, (uint64_t)rows_x * (uint64_t)K);
+    const uint8_t* w_e = p.w + (uint64_t)e * (uint64_t)rows_e * (uint64_t)K;
+    __amdgpu_buffer_rsrc_t rb = make_rsrc(w_e, (uint64_t)rows_e * (uint64_t)K);
+
+    uint32_t a_voff[A_LOADS];
+    int a_ldsoff[A_LOADS];
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) {
+        const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
+        const int xr = row < BM ? x_row(row) : -1;
+        a_voff[j] = xr >= 0 ? (uint32_t)xr * (uint32_t)K + (uint32_t)kc * 16u : 0xFFFFFFF0u;
+        a_ldsoff[j] = row < BM ? moe_lds_off(row, kc) : -1;
+    }
+    // n-blocks of this wavefront inside the expert's slab: set 0 = gate (or the only set), set 1 = up
+    uint32_t b_voff[NSET][NR];
+#pragma unroll
+    for (int s = 0; s < NSET; s++)
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) {
+            const int n = n0 + (wave * NR + ni) * 16;                 // first column of the block
+            const int nb = (n + s * p.n_out) >> 4;
+            b_voff[s][ni] = n < p.n_out ? (uint32_t)nb * 16u * (uint32_t)K + (uint32_t)lane * 16u : 0xFFFFFFF0u;
+        }
+
+    v4i areg[A_LOADS];
+    auto load_a = [&](int kt) {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++) {
+            const bool ok = kt < KT;
+            areg[j] = buf_load16(ra, ok ? a_voff[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 128u : 0u);
+        }
+    };
+    auto store_a = [&](int stage) {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++)
+            if (a_ldsoff[j] >= 0) *reinterpret_cast<v4i*>(&lds[stage][a_ldsoff[j]]) = areg[j];
+    };
+    v4i blo[2][NSET][NR], bhi[2][NSET][NR];
+    auto load_b = [&](int kt, int set) {
+#pragma unroll
+        for (int s = 0; s < NSET; s++)
+#pragma unroll
+            for (int ni = 0; ni < NR; ni++) {
+                const bool ok = kt < KT;
+                blo[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
+                bhi[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] + 1024u : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
+            }
+    };
+
+    acc_t acc[MR][NSET][NR];
+#pragma unroll
+    for (int mi = 0; mi < MR; mi++)
+#pragma unroll
+        for (int s = 0; s < NSET; s++)
+#pragma unroll
+            for (int ni = 0; ni < NR; ni++) acc[mi][s][ni] = (acc_t){0, 0, 0, 0};
+
+    auto step = [&](int kt, auto SP) __attribute__((always_inline)) {
+        constexpr int S = decltype(SP)::value;
+        load_a(kt + 1);
+        load_b(kt + 1, S ^ 1);
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            const int row = mi * 16 + li;
+            const v4i alo = *reinterpret_cast<const v4i*>(&lds[S][moe_lds_off(row, lg)]);
+            const v4i ahi = *reinterpret_cast<const v4i*>(&lds[S][moe_lds_off(row, 4 + lg)]);
+            static_for<NSET>([&](auto SI) {
+                constexpr int s = decltype(SI)::value;
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    if constexpr (KIND == KIND_INT8) {
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[S][s][ni], alo, acc[mi][s][ni], 0, 0, 0);
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[S][s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
+                    } else {
+                        const v8i w8 = __builtin_shufflevector(blo[S][s][ni], bhi[S][s][ni], 0, 1, 2, 3, 4, 5, 6, 7);
+                        const v8i a8 = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w8, a8, acc[mi][s][ni], 0, 0, 0, 0, 0, 0);
+                    }
+                });
+            });
+        });
+        store_a(S ^ 1);
+        __syncthreads();
+    };
+
+    load_a(0);
+    load_b(0, 0);
+    store_a(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; kt += 2) {
+        step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
+    }
+
+    // epilogue: lane owns rows mi*16 + li, columns n0 + (wave*NR + ni)*16 + lg*4 + 0..3
+    static_for<MR>([&](auto MI) {
+        constexpr int mi = decltype(MI)::value;
+        const int r = mi * 16 + li;
+        const int xr = x_row(r);
+        if (xr >= 0) {
+            const uint32_t sid = (uint32_t)ids[r];
+            const int t = (int)(sid & 0xFFFFFFu), slot = (int)(sid >> 24);
+            const float sx = p.sx[xr];
+            const float rw = p.doweight ? p.sorted_w[blk * BM + r] : 1.0f;
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                if (n < p.n_out) {
+                    v4f y;
+                    if constexpr (STAGE == 1) {
+                        const v4f swg = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + n);
+                        const v4f swu = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + p.n_out + n);
+                        const acc_t ag = acc[mi][0][ni], au = acc[mi][NSET - 1][ni];
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            const float g = ((float)ag[v] * sx) * swg[v], u = ((float)au[v] * sx) * swu[v];
+                            y[v] = silu(g) * u * rw;
+                        }
+                        const size_t idx = ((size_t)t * p.topk + slot) * (size_t)p.n_out + n;
+                        const v2i o = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(y[0], y[1], y[2], y[3]) : pack4_out16<OUT_FP16>(y[0], y[1], y[2], y[3]);
+                        *reinterpret_cast<v2i*>(static_cast<uint16_t*>(p.out) + idx) = o;
+                    } else {
+                        const v4f sw = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + n);
+                        const acc_t a = acc[mi][0][ni];
+#pragma unroll
+                        for (int v = 0; v < 4; v++) y[v] = (((float)a[v] * sx) * sw[v]) * rw;
+                        if (!p.accumulate) {
+                            const size_t idx = ((size_t)t * p.topk + slot) * (size_t)p.n_out + n;
+                            const v2i o = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(y[0], y[1], y[2], y[3]) : pack4_out16<OUT_FP16>(y[0], y[1], y[2], y[3]);
+                            *reinterpret_cast<v2i*>(static_cast<uint16_t*>(p.out) + idx) = o;
+                        } else {
+                            const size_t idx = (size_t)t * (size_t)p.n_out + n;
+                            if (p.out_dtype == OUT_F32) {
+                                float* o = static_cast<float*>(p.out) + idx;
+#pragma unroll
+                                for (int v = 0; v < 4; v++) unsafeAtomicAdd(o + v, y[v]);
+                            } else if (p.out_dtype == OUT_FP16) {
+                                auto* o = (__attribute__((address_space(1))) v2h*)(static_cast<uint16_t*>(p.out) + idx);
+                                __builtin_amdgcn_global_atomic_fadd_v2f16(o, (v2h){(__fp16)y[0], (__fp16)y[1]});
+                                __builtin_amdgcn_global_atomic_fadd_v2f16(o + 1, (v2h){(__fp16)y[2], (__fp16)y[3]});
+                            } else {
+                                auto* o = (__attribute__((address_space(1))) v2b*)(static_cast<uint16_t*>(p.out) + idx);
+                                __builtin_amdgcn_global_atomic_fadd_v2bf16(o, (v2b){(__bf16)y[0], (__bf16)y[1]});
+                                __builtin_amdgcn_global_atomic_fadd_v2bf16(o + 1, (v2b){(__bf16)y[2], (__bf16)y[3]});
+                            }
+                        }
+                    }
+                }
+            });
+        }
+    });
+}
+
+template <int KIND, int STAGE, int NR>
+hipError_t launch_nr(const MoeParams& p, int block_m, int blocks, hipStream_t stream) {
+    const dim3 grid((p.n_out + 64 * NR - 1) / (64 * NR), blocks, 1);
+#define PSG_MOE(MR_)                                                                                \
+    if (block_m == 16 * MR_) {                                                                      \
+        hipLaunchKernelGGL((k_moe_gemm<KIND, MR_, NR, STAGE>), grid, dim3(256), 0, stream, p);     \
+        return hipGetLastError();                                                                   \
+    }
+    PSG_MOE(1) PSG_MOE(2) PSG_MOE(4) PSG_MOE(8)
+#undef PSG_MOE
+    return hipErrorInvalidValue;
+}
+
+template <int KIND, int STAGE>
+hipError_t launch_kind(const MoeParams& p, int block_m, int blocks, hipStream_t stream) {
+    // 128 columns per workgroup when they divide the output and the block is small enough for the registers
+    if (p.n_out % 128 == 0 && block_m <= (STAGE == 1 ? 32 : 64)) return launch_nr<KIND, STAGE, 2>(p, block_m, blocks, stream);
+    return launch_nr<KIND, STAGE, 1>(p, block_m, blocks, stream);
+}
+
+}  // namespace
+
+// kind: KIND_INT8 / KIND_FP8; stage 1 or 2; block_m in {16, 32, 64, 128}; blocks = entries of expert_ids
+hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream) {
+    if (kind == KIND_INT8) return stage == 1 ? launch_kind<KIND_INT8, 1>(p, block_m, blocks, stream) : launch_kind<KIND_INT8, 2>(p, block_m, blocks, stream);
+    return stage == 1 ? launch_kind<KIND_FP8, 1>(p, block_m, blocks, stream) : launch_kind<KIND_FP8, 2>(p, block_m, blocks, stream);
+}
+
+// sum over the topk slots: y[t, :] = sum_s x[t, s, :] (16-bit in and out, fp32 sum in slot order)
+namespace {
+__global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t* y, int tokens, int topk, int dim, int out_dtype) {
+    const size_t q = (size_t)blockIdx.x * 256 + threadIdx.x;   // one thread per 4 columns
+    const size_t quads = (size_t)tokens * (size_t)(dim >> 2);
+    if (q >= quads) return;
+    const size_t t = q / (size_t)(dim >> 2), c = (q % (size_t)(dim >> 2)) << 2;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int k = 0; k < topk; k++) {
+        const v2i v = *reinterpret_cast<const v2i*>(x + (t * topk + k) * (size_t)dim + c);
+        const uint16_t h0 = (uint16_t)(v[0] & 0xFFFF), h1 = (uint16_t)((uint32_t)v[0] >> 16), h2 = (uint16_t)(v[1] & 0xFFFF), h3 = (uint16_t)((uint32_t)v[1] >> 16);
+        if (out_dtype == OUT_BF16) {
+            s0 += from_out16<OUT_BF16>(h0); s1 += from_out16<OUT_BF16>(h1); s2 += from_out16<OUT_BF16>(h2); s3 += from_out16<OUT_BF16>(h3);
+        } else {
+            s0 += from_out16<OUT_FP16>(h0); s1 += from_out16<OUT_FP16>(h1); s2 += from_out16<OUT_FP16>(h2); s3 += from_out16<OUT_FP16>(h3);
+        }
+    }
+    const v2i o = out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(s0, s1, s2, s3) : pack4_out16<OUT_FP16>(s0, s1, s2, s3);
+    *reinterpret_cast<v2i*>(y + t * (size_t)dim + c) = o;
+}
+}  // namespace
+
+hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, hipStream_t stream) {
+    const size_t quads = (size_t)tokens * (size_t)(dim >> 2);
+    hipLaunchKernelGGL(k_moe_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, static_cast<const uint16_t*>(x),
+                       static_cast<uint16_t*>(y), tokens, topk, dim, out_dtype);
+    return hipGetLastError();
+}

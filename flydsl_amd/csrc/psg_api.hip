@@ -12,6 +12,8 @@
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
+hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream);
+hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, hipStream_t stream);
 hipError_t psg_launch_mx_generic(const MxGenParams& p, int af, int bf, int store, int batch, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
@@ -468,6 +470,68 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
 int psg_gemm_mxfp4(const psg_mxfp4_args* args, void* stream) { return mx_common(args, args ? args->c : nullptr, STORE_C, stream); }
 
 int psg_gemm_mxfp4_acc(const psg_mxfp4_args* args, void* acc, void* stream) { return mx_common(args, acc, STORE_ACC, stream); }
+
+int psg_moe_gemm(const psg_moe_args* a, void* stream) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!a->out || !a->x || !a->w || !a->scale_x || !a->scale_w || !a->sorted_token_ids || !a->sorted_expert_ids || !a->num_valid_ids)
+        return fail(PSG_E_NULL, "out, x, w, scale_x, scale_w, sorted_token_ids, sorted_expert_ids, num_valid_ids must be non-NULL");
+    if (a->doweight && !a->sorted_weights) return fail(PSG_E_NULL, "sorted_weights must be non-NULL when doweight is set");
+    if (a->stage != 1 && a->stage != 2) return fail(PSG_E_SHAPE, "stage=%d must be 1 or 2", a->stage);
+    if (a->in_dtype != PSG_IN_INT8 && a->in_dtype != PSG_IN_FP8_E4M3FN) return fail(PSG_E_DTYPE, "in_dtype %d must be int8 or fp8", a->in_dtype);
+    if (a->out_dtype < PSG_OUT_BF16 || a->out_dtype > PSG_OUT_F32) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
+    if (a->out_dtype == PSG_OUT_F32 && !(a->stage == 2 && a->accumulate))
+        return fail(PSG_E_DTYPE, "fp32 output exists only for stage 2 with accumulate (kernels/moe/moe_gemm_2stage/gemm2.py:629)");
+    if (a->pad0 != 0) return fail(PSG_E_SHAPE, "pad0 must be 0");
+    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
+    if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
+    if (a->experts < 1) return fail(PSG_E_SHAPE, "experts=%d must be positive", a->experts);
+    if (a->block_m != 16 && a->block_m != 32 && a->block_m != 64 && a->block_m != 128) return fail(PSG_E_SHAPE, "block_m=%d must be 16, 32, 64 or 128", a->block_m);
+    if (a->blocks < 1 || a->blocks > 65535) return fail(PSG_E_SHAPE, "blocks=%d outside [1, 65535]", a->blocks);
+    if (a->sorted_size < 1) return fail(PSG_E_SHAPE, "sorted_size=%d must be positive", a->sorted_size);
+    const int K = a->stage == 1 ? a->model_dim : a->inter_dim, n_out = a->stage == 1 ? a->inter_dim : a->model_dim;
+    if (K < 128 || K % 128) return fail(PSG_E_SHAPE, "K=%d of stage %d must be a positive multiple of 128", K, a->stage);
+    if (n_out < 16 || n_out % 16) return fail(PSG_E_SHAPE, "output width %d of stage %d must be a positive multiple of 16", n_out, a->stage);
+    const uint64_t rows_x = a->stage == 1 ? (uint64_t)a->tokens : (uint64_t)a->tokens * (uint64_t)a->topk;
+    const uint64_t rows_e = a->stage == 1 ? 2ull * (uint64_t)n_out : (uint64_t)n_out;
+    if (rows_x * (uint64_t)K > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "x exceeds the 4 GiB descriptor range");
+    if (rows_e * (uint64_t)K > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "one expert's weights exceed the 4 GiB descriptor range");
+    if (!aligned(a->x, 16) || !aligned(a->w, 16) || !aligned(a->scale_w, 16) || !aligned(a->out, 16))
+        return fail(PSG_E_ALIGN, "x, w, scale_w and out must be 16-byte aligned");
+    MoeParams p;
+    p.out = a->out;
+    p.x = static_cast<const uint8_t*>(a->x);
+    p.w = static_cast<const uint8_t*>(a->w);
+    p.sx = a->scale_x;
+    p.sw = a->scale_w;
+    p.sorted_ids = a->sorted_token_ids;
+    p.expert_ids = a->sorted_expert_ids;
+    p.sorted_w = a->sorted_weights;
+    p.num_valid = a->num_valid_ids;
+    p.tokens = a->tokens;
+    p.topk = a->topk;
+    p.experts = a->experts;
+    p.n_out = n_out;
+    p.K = K;
+    p.sorted_size = a->sorted_size;
+    p.out_dtype = a->out_dtype;
+    p.doweight = a->doweight ? 1 : 0;
+    p.accumulate = a->stage == 2 && a->accumulate ? 1 : 0;
+    const hipError_t e = psg_launch_moe_gemm(p, a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : KIND_FP8, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_gemm launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+int psg_moe_reduce(const void* x, void* y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void* stream) {
+    if (!x || !y) return fail(PSG_E_NULL, "x and y must be non-NULL");
+    if (dtype != PSG_OUT_BF16 && dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "dtype %d must be bf16 or fp16", dtype);
+    if (tokens < 1 || topk < 1 || model_dim < 4 || model_dim % 4) return fail(PSG_E_SHAPE, "need tokens, topk >= 1 and model_dim a positive multiple of 4");
+    if (!aligned(x, 8) || !aligned(y, 8)) return fail(PSG_E_ALIGN, "x and y must be 8-byte aligned");
+    const hipError_t e = psg_launch_moe_reduce(x, y, tokens, topk, model_dim, dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_reduce launch");
+    g_err[0] = 0;
+    return 0;
+}
 
 int psg_quant_pertoken(const void* x, int32_t x_dtype, void* y, float* scale, int32_t M, int32_t K, int32_t out_dtype, void* stream) {
     if (!x || !y || !scale) return fail(PSG_E_NULL, "x, y and scale must be non-NULL");

@@ -144,6 +144,27 @@ struct MxGenParams {
     int64_t a_batch, b_batch, c_batch, sa_batch, sb_batch;  // bytes between batches
 };
 
+// Arguments of the MoE grouped GEMMs (gate-up stage and down stage) over sorted token blocks.
+constexpr int OUT_F32 = 2;
+struct MoeParams {
+    void* out;
+    const uint8_t* x;           // stage 1: [tokens, K]; stage 2: [tokens*topk, K]
+    const uint8_t* w;           // preshuffled [experts * rows_per_expert, K] (rows_per_expert = 2*inter or model_dim)
+    const float* sx;            // one scale per row of x
+    const float* sw;            // [experts * rows_per_expert]
+    const int32_t* sorted_ids;  // (slot << 24) | token per sorted row; padding rows hold token >= tokens
+    const int32_t* expert_ids;  // expert of each block of block_m sorted rows
+    const float* sorted_w;      // routing weight per sorted row
+    const int32_t* num_valid;   // [0] = number of sorted rows in use (a multiple of block_m)
+    int tokens, topk, experts;
+    int n_out;                  // inter_dim (stage 1) or model_dim (stage 2)
+    int K;                      // model_dim (stage 1) or inter_dim (stage 2)
+    int sorted_size;            // entries of sorted_ids / sorted_w
+    int out_dtype;              // OUT_BF16 / OUT_FP16 / OUT_F32 (stage 2 with accumulate only)
+    int doweight;               // multiply by the routing weight in this stage
+    int accumulate;             // stage 2: atomic add into out[token] (else one row per (token, slot))
+};
+
 // bias + activation + 16-bit conversion of four consecutive columns.  The variant is chosen at run time
 // (the epilogue is a vanishing part of any launch, so it is not worth a kernel instantiation per variant).
 template <int OUT, int EPI>

@@ -27,6 +27,8 @@
  *                       tiled kernel uses); psg_debug_tile_order runs the same function on the device
  *   psg_gemm_a8w8_static, psg_init, psg_static_scratch_bytes
  *                       no counterpart in the reference: for callers that cannot allocate (see below)
+ *   psg_moe_gemm        kernels/moe/moe_gemm_2stage/gemm1.py, gemm2.py (launch_moe_gemm1 / launch_moe_gemm2), fp8 and int8
+ *   psg_moe_reduce      kernels/moe/moe_gemm_2stage/moe_reduce.py:164 (compile_moe_reduction)
  *   psg_quant_pertoken  device version of the host quantiser tests/utils.py:29-73
  *   psg_quant_mxfp4     device version of tests/kernels/utils/gemm_common_utils.py:675-704 (+ :645-672)
  */
@@ -40,12 +42,12 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 3
+#define PSG_ABI_VERSION 4
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
 /* output element types of C */
-enum psg_out_dtype { PSG_OUT_BF16 = 0, PSG_OUT_FP16 = 1 };
+enum psg_out_dtype { PSG_OUT_BF16 = 0, PSG_OUT_FP16 = 1, PSG_OUT_F32 = 2 /* psg_moe_gemm stage 2 with accumulate only */ };
 /* fused epilogue, as the reference's `epilogue` keyword (kernels/gemm/preshuffle_gemm.py:118) */
 enum psg_epilogue {
     PSG_EPI_NONE = 0,
@@ -229,6 +231,54 @@ int psg_quant_pertoken(const void *x, int32_t x_dtype, void *y, float *scale, in
  * shuffle_scale_w4 layout the GEMM reads (shuffled = 1, needs K % 256 == 0).  K % 32 == 0. */
 int psg_quant_mxfp4(const void *x, int32_t x_dtype, void *packed, void *scales, int32_t M, int32_t K, int32_t shuffled,
                     void *stream);
+
+/*
+ * MoE grouped GEMMs over expert-sorted token blocks: the two stages of the reference's 2-stage MoE
+ * (kernels/moe/moe_gemm_2stage/gemm1.py:367-381,502-537 launch_moe_gemm1; gemm2.py launch_moe_gemm2), int8 or e4m3fn
+ * operands with one fp32 scale per row of x and per weight row.
+ *   stage 1: out[t, slot, n] = silu(g) * u (* routing weight when doweight), g = x[t] . W1[e, n], u = x[t] . W1[e, inter + n];
+ *            x [tokens, model_dim], w = shuffle_weight of W1 [experts * 2*inter_dim, model_dim], out [tokens, topk, inter_dim]
+ *   stage 2: y = x[t*topk + slot] . W2[e, n] (* routing weight when doweight); accumulate = 1 adds y atomically into
+ *            out[t, n] (out [tokens, model_dim], bf16 / fp16 / fp32, zeroed by the caller; the order of the additions is
+ *            not fixed), accumulate = 0 writes out[t*topk + slot, n] (bf16 / fp16) for psg_moe_reduce;
+ *            x [tokens*topk, inter_dim], w = shuffle_weight of W2 [experts * model_dim, inter_dim]
+ *   sorted_token_ids  (slot << 24) | token for every sorted row, experts in ascending order, every expert padded to
+ *                     whole blocks of block_m rows with entries whose token is >= tokens (tests/kernels/
+ *                     test_moe_gemm_2stage.py:99-137); sorted_weights the routing weight of each sorted row;
+ *                     sorted_expert_ids one expert per block (entries < 0 are skipped); num_valid_ids[0] = sorted rows
+ *                     in use (read on the device, so the grid does not depend on the routing)
+ *   block_m in {16, 32, 64, 128}; model_dim % 128 == 0 and inter_dim % 128 == 0 for the K side of each stage;
+ *   the output width of each stage a multiple of 16; tokens < 2^24; rows of x times K below 4 GiB.
+ */
+typedef struct psg_moe_args {
+    void *out;
+    const void *x;
+    const void *w;
+    const float *scale_x;
+    const float *scale_w;
+    const int32_t *sorted_token_ids;
+    const int32_t *sorted_expert_ids;
+    const float *sorted_weights;
+    const int32_t *num_valid_ids;
+    int32_t tokens, topk, experts;
+    int32_t model_dim, inter_dim;
+    int32_t sorted_size; /* entries of sorted_token_ids / sorted_weights */
+    int32_t blocks;      /* entries of sorted_expert_ids = grid size along the sorted rows */
+    int32_t block_m;
+    int32_t in_dtype;    /* PSG_IN_INT8 or PSG_IN_FP8_E4M3FN */
+    int32_t out_dtype;   /* enum psg_out_dtype */
+    int32_t stage;       /* 1 or 2 */
+    int32_t doweight;
+    int32_t accumulate;  /* stage 2 only */
+    int32_t pad0;        /* 0 */
+} psg_moe_args;
+
+int psg_moe_gemm(const psg_moe_args *args, void *stream);
+
+/* y[t, :] = sum over the topk slots of x[t, slot, :] (fp32 sum in slot order), the pass after stage 2 with accumulate = 0
+ * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203, without its expert mask).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16;
+ * model_dim % 4 == 0. */
+int psg_moe_reduce(const void *x, void *y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void *stream);
 
 #ifdef __cplusplus
 }

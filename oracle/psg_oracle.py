@@ -475,6 +475,89 @@ def run_torch_mx(a_q, b_q, scale_a, scale_b, a_fmt: str = "fp4", b_fmt: str = "f
 
 
 # ----------------------------------------------------------------------------------------------
+# MoE 2-stage (tests/kernels/test_moe_gemm_2stage.py, tests/kernels/test_ref.py)
+# ----------------------------------------------------------------------------------------------
+
+
+def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int, block_size: int):
+    """Expert sorting of routed (token, slot) pairs (tests/kernels/test_moe_gemm_2stage.py:99-137): experts in
+    ascending order, each expert's pairs in row-major (token, slot) order and padded to whole blocks with
+    ``(topk << 24) | tokens``; one expert id per block, -1 for unused blocks.  Returns ``(sorted_ids int32,
+    sorted_weights fp32 (0 in padding rows; the reference leaves them uninitialised), sorted_expert_ids int32,
+    num_tokens_post_pad int32[2])``.  Pinned by invariants (every pair exactly once and inside its expert's blocks,
+    padding values, block count) and a hand-worked example."""
+    ids = np.asarray(topk_ids)
+    wts = np.asarray(topk_weights, dtype=np.float32)
+    tokens, topk = ids.shape
+    max_padded = int(ids.size + num_experts * block_size - topk)
+    max_blocks = (max_padded + block_size - 1) // block_size
+    sorted_ids = np.full(max_padded, (topk << 24) | tokens, dtype=np.int32)
+    sorted_w = np.zeros(max_padded, dtype=np.float32)
+    sorted_e = np.full(max_blocks, -1, dtype=np.int32)
+    begin = blk = 0
+    for e in range(num_experts):
+        t, s = np.nonzero(ids == e)
+        n = t.size
+        nb = (n + block_size - 1) // block_size
+        sorted_ids[begin : begin + n] = (s.astype(np.int32) << 24) | t.astype(np.int32)
+        sorted_w[begin : begin + n] = wts[t, s]
+        begin += nb * block_size
+        sorted_e[blk : blk + nb] = e
+        blk += nb
+    return sorted_ids, sorted_w, sorted_e, np.array([begin, tokens], dtype=np.int32)
+
+
+def moe_gemm1(x_q, w1_q, scale_x, scale_w1, topk_ids, topk_weights, inter_dim: int, doweight_stage1: bool, kind: str = "fp8"):
+    """Stage 1 of the 2-stage MoE (tests/kernels/test_ref.py:91-161, per-row scales): for every routed (token, slot)
+    with expert e, ``y = W1[e] @ x[token]`` over the dequantised operands, ``out[token, slot] = silu(y[:inter]) *
+    y[inter:]`` (times the routing weight when ``doweight_stage1``).  ``x_q [tokens, model_dim]``, ``w1_q
+    [experts*2*inter, model_dim]`` bit patterns (``kind`` "fp8" / "int8"), scales fp32 per row.  Returns fp32
+    ``[tokens, topk, inter_dim]``.  Pinned by scalar float64 loops on tiny inputs."""
+    x = _as_f32_operand(np.asarray(x_q), kind) * np.asarray(scale_x, dtype=np.float32).reshape(-1, 1)
+    w = _as_f32_operand(np.asarray(w1_q), kind) * np.asarray(scale_w1, dtype=np.float32).reshape(-1, 1)
+    ids = np.asarray(topk_ids)
+    tokens, topk = ids.shape
+    w = w.reshape(-1, 2 * inter_dim, x.shape[1])
+    out = np.zeros((tokens, topk, inter_dim), dtype=np.float32)
+    for e in range(w.shape[0]):
+        t, s = np.nonzero(ids == e)
+        if t.size == 0:
+            continue
+        y2 = (x[t] @ w[e].T).astype(np.float32)
+        g, u = y2[:, :inter_dim], y2[:, inter_dim:]
+        with np.errstate(over="ignore"):
+            y = (g / (np.float32(1.0) + np.exp(-g))).astype(np.float32) * u
+        if doweight_stage1:
+            y = y * np.asarray(topk_weights, dtype=np.float32)[t, s][:, None]
+        out[t, s] = y
+    return out
+
+
+def moe_gemm2(a2_q, w2_q, scale_a2, scale_w2, topk_ids, topk_weights, model_dim: int, doweight_stage2: bool, kind: str = "fp8",
+              reduce_slots: bool = True):
+    """Stage 2 of the 2-stage MoE (tests/kernels/test_ref.py:164-240, per-row scales): ``y = W2[e] @ a2[token, slot]``
+    (times the routing weight when ``doweight_stage2``), summed over the slots into ``[tokens, model_dim]`` fp32
+    (``reduce_slots=False`` keeps ``[tokens, topk, model_dim]``, what the non-accumulating kernel writes).  ``a2_q
+    [tokens, topk, inter]``, ``w2_q [experts*model_dim, inter]``.  Pinned by scalar float64 loops on tiny inputs."""
+    ids = np.asarray(topk_ids)
+    tokens, topk = ids.shape
+    a = _as_f32_operand(np.asarray(a2_q).reshape(tokens * topk, -1), kind) * np.asarray(scale_a2, dtype=np.float32).reshape(-1, 1)
+    a = a.reshape(tokens, topk, -1)
+    w = _as_f32_operand(np.asarray(w2_q).reshape(-1, a.shape[2]), kind) * np.asarray(scale_w2, dtype=np.float32).reshape(-1, 1)
+    w = w.reshape(-1, model_dim, a.shape[2])
+    out = np.zeros((tokens, topk, model_dim), dtype=np.float32)
+    for e in range(w.shape[0]):
+        t, s = np.nonzero(ids == e)
+        if t.size == 0:
+            continue
+        y = (a[t, s] @ w[e].T).astype(np.float32)
+        if doweight_stage2:
+            y = y * np.asarray(topk_weights, dtype=np.float32)[t, s][:, None]
+        out[t, s] = y
+    return out.sum(axis=1).astype(np.float32) if reduce_slots else out
+
+
+# ----------------------------------------------------------------------------------------------
 # Epilogue (kernels/gemm/preshuffle_gemm.py:672-714)
 # ----------------------------------------------------------------------------------------------
 

@@ -1,0 +1,230 @@
+"""GPU parity of the 2-stage MoE grouped GEMMs (fp8 / int8) against the CPU oracle, through the reference's call shapes.
+
+Mirrors tests/kernels/test_moe_gemm_2stage.py: test_moe_gemm1_numeric (:382-408), test_moe_gemm2_numeric (:608-642),
+the ragged-M fast shapes (:982-996), the output canaries (:1350-1450) and test_moe_gemm2_rejects_f32_reduce (:894).
+The reference accepts cosine similarity > 0.99; here stage 1 and the non-accumulating stage 2 must also be within
+|out-ref| <= 1e-2*|ref| + 1e-2*max|ref|, and the atomic stage 2 (whose 16-bit additions round in arrival order) within
+3e-2*max|ref|."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from flydsl_amd import layout, quant
+from flydsl_amd.kernels.moe.moe_sorting import moe_sorting
+from oracle import psg_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = dict(model_dim=256, inter_dim=128, experts=4, topk=2)
+TDT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+QDT = {"fp8": torch.float8_e4m3fn, "int8": torch.int8}
+
+
+def _cos(a, b):
+    a, b = a.reshape(-1).astype(np.float64), b.reshape(-1).astype(np.float64)
+    return float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b)))
+
+
+def _routing(tokens, experts, topk, tile_m, seed):
+    g = torch.Generator().manual_seed(seed)
+    score = torch.rand(tokens, experts, generator=g)
+    vals, ids = torch.topk(score, k=topk, dim=1)
+    w = torch.softmax(vals, dim=1).float()
+    sid, sw, se, npp = moe_sorting(ids.int(), w, num_experts=experts, block_size=tile_m)
+    return ids.int(), w, (sid, sw, se, npp[:1].contiguous(), int(se.numel()))
+
+
+def _launch(exe, out, x, w, sx, sw, routing, dim0, dim1, tokens):
+    dev = torch.device("cuda")
+    sid, swt, se, nv, blocks = routing
+    exe(out, x.to(dev).view(-1), w.to(dev).view(-1), sx.to(dev).view(-1).contiguous(), sw.to(dev).view(-1).contiguous(), sid.to(dev), se.to(dev),
+        swt.to(dev), nv.to(dev), tokens, dim0, dim1, blocks, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+
+
+def _stage1(tokens, model_dim, inter_dim, experts, topk, tile_m, tile_n, tile_k, out_dtype, in_dtype, seed=0, doweight=False, canary=None):
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1
+
+    g = torch.Generator().manual_seed(seed + 100)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, seed)
+    x = torch.randn(tokens, model_dim, generator=g)
+    w1 = torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim)
+    xq, sx = quant.pertoken_quant(x, quant_dtype=QDT[in_dtype])
+    w1q, sw1 = quant.pertoken_quant(w1, quant_dtype=QDT[in_dtype])
+    w1s = layout.shuffle_weight(w1q).view(experts * 2 * inter_dim, model_dim).contiguous()
+    out = torch.empty(tokens, topk, inter_dim, dtype=TDT[out_dtype], device="cuda")
+    if canary is not None:
+        out.fill_(canary)
+    exe = compile_moe_gemm1(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=tile_n, tile_k=tile_k,
+                            doweight_stage1=doweight, out_dtype=out_dtype, in_dtype=in_dtype)
+    _launch(exe, out, xq, w1s, sx, sw1.view(-1, 1), routing, inter_dim, model_dim, tokens)
+    ref = O.moe_gemm1(xq.view(torch.uint8).numpy(), w1q.view(torch.uint8).numpy().reshape(-1, model_dim), sx.numpy(), sw1.numpy().reshape(-1),
+                      ids.numpy(), wts.numpy(), inter_dim, doweight, in_dtype)
+    return out.float().cpu().numpy(), ref
+
+
+def _stage2(tokens, model_dim, inter_dim, experts, topk, tile_m, tile_n, tile_k, out_dtype, accumulate, in_dtype, seed=0, doweight=True, guard=0):
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm2
+
+    g = torch.Generator().manual_seed(seed + 200)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, seed)
+    a2 = torch.randn(tokens, topk, inter_dim, generator=g)
+    a2 = torch.nn.functional.silu(a2) * torch.randn(tokens, topk, inter_dim, generator=g)  # shaped like a stage-1 output
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    a2q, sa2 = quant.pertoken_quant(a2, quant_dtype=QDT[in_dtype])
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=QDT[in_dtype])
+    w2s = layout.shuffle_weight(w2q).view(experts * model_dim, inter_dim).contiguous()
+    rows = tokens if accumulate else tokens * topk
+    out = torch.zeros(rows + guard, model_dim, dtype=TDT[out_dtype], device="cuda")
+    exe = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=tile_n, tile_k=tile_k,
+                            doweight_stage2=doweight, out_dtype=out_dtype, accumulate=accumulate, in_dtype=in_dtype)
+    _launch(exe, out, a2q, w2s, sa2, sw2.view(-1, 1), routing, model_dim, inter_dim, tokens)
+    ref = O.moe_gemm2(a2q.view(torch.uint8).numpy(), w2q.view(torch.uint8).numpy().reshape(-1, inter_dim), sa2.numpy().reshape(-1),
+                      sw2.numpy().reshape(-1), ids.numpy(), wts.numpy(), model_dim, doweight, in_dtype, reduce_slots=accumulate)
+    return out, ref.reshape(rows, model_dim)
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
+@pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile_m,tokens", [(64, 128), (16, 8)])
+def test_moe_gemm1_numeric(in_dtype, out_dtype, tile_m, tokens):
+    out, ref = _stage1(tokens, **SHAPE, tile_m=tile_m, tile_n=64, tile_k=128, out_dtype=out_dtype, in_dtype=in_dtype)
+    assert _cos(out, ref) > 0.99
+    ok, ratio = O.within_north_star_tolerance(out, ref, 1e-2)
+    assert ok, f"outside tolerance (worst ratio {ratio:.3f})"
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
+@pytest.mark.parametrize("accumulate,out_dtype", [(True, "f16"), (True, "bf16"), (True, "f32"), (False, "f16"), (False, "bf16")])
+@pytest.mark.parametrize("tile_m,tokens", [(16, 8), (64, 128)])
+def test_moe_gemm2_numeric(accumulate, out_dtype, tile_m, tokens, in_dtype):
+    out, ref = _stage2(tokens, **SHAPE, tile_m=tile_m, tile_n=64, tile_k=128, out_dtype=out_dtype, accumulate=accumulate, in_dtype=in_dtype, guard=4)
+    got = out[: ref.shape[0]].float().cpu().numpy()
+    assert (out[ref.shape[0]:] == 0).all()
+    assert _cos(got, ref) > 0.99
+    if accumulate and out_dtype != "f32":
+        assert np.abs(got - ref).max() <= 3e-2 * np.abs(ref).max()
+    else:
+        ok, ratio = O.within_north_star_tolerance(got, ref, 1e-2)
+        assert ok, f"outside tolerance (worst ratio {ratio:.3f})"
+
+
+# ragged M against the block size, several experts / topk / tiles (tests/kernels/test_moe_gemm_2stage.py:982-996, :1005-1011)
+FAST = [(3, 4, 2, 16, 64, 128), (7, 8, 2, 32, 64, 128), (33, 8, 2, 64, 128, 128), (17, 8, 2, 16, 64, 256), (31, 32, 6, 16, 64, 128), (129, 16, 8, 128, 256, 256),
+        (1, 8, 1, 16, 64, 128)]
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
+@pytest.mark.parametrize("tokens,experts,topk,tile_m,tile_n,tile_k", FAST)
+def test_moe_gemm1_shapes(in_dtype, tokens, experts, topk, tile_m, tile_n, tile_k):
+    out, ref = _stage1(tokens, 512, 256, experts, topk, tile_m, tile_n, tile_k, "bf16", in_dtype, seed=tokens, doweight=bool(tokens % 2))
+    ok, ratio = O.within_north_star_tolerance(out, ref, 1e-2)
+    assert ok, f"outside tolerance (worst ratio {ratio:.3f})"
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
+@pytest.mark.parametrize("accumulate", [True, False])
+@pytest.mark.parametrize("tokens,experts,topk,tile_m,tile_n,tile_k", FAST)
+def test_moe_gemm2_shapes(in_dtype, accumulate, tokens, experts, topk, tile_m, tile_n, tile_k):
+    out, ref = _stage2(tokens, 512, 256, experts, topk, tile_m, tile_n, tile_k, "f32" if accumulate else "bf16", accumulate, in_dtype, seed=tokens,
+                       doweight=not (tokens % 2 == 0 and accumulate))
+    got = out.float().cpu().numpy()
+    ok, ratio = O.within_north_star_tolerance(got, ref, 1e-2)
+    assert ok, f"outside tolerance (worst ratio {ratio:.3f})"
+
+
+def test_stage1_writes_every_routed_row_and_nothing_else():
+    # every (token, slot) is routed, so a canary must survive nowhere; with the accumulate-free stage 2 the same holds
+    out, ref = _stage1(7, **SHAPE, tile_m=16, tile_n=64, tile_k=128, out_dtype="f16", in_dtype="fp8", canary=777.0)
+    assert not (out == 777.0).any()
+    ok, _ = O.within_north_star_tolerance(out, ref, 1e-2)
+    assert ok
+
+
+def test_padding_rows_do_not_touch_token_zero():
+    # all routes go to ONE expert with 3 tokens and blocks of 64: 61 padding rows per block must neither read nor write
+    # row 0 (the reference's sentinel regression, tests/kernels/test_moe_gemm_2stage.py:1687-1760)
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm2
+
+    tokens, model_dim, inter_dim, experts, topk, tile_m = 3, 256, 128, 4, 1, 64
+    g = torch.Generator().manual_seed(5)
+    ids = torch.full((tokens, topk), 2, dtype=torch.int32)
+    wts = torch.ones(tokens, topk)
+    sid, swt, se, npp = moe_sorting(ids, wts, num_experts=experts, block_size=tile_m)
+    a2 = torch.randn(tokens, topk, inter_dim, generator=g)
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    a2q, sa2 = quant.pertoken_quant(a2, quant_dtype=torch.int8)
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=torch.int8)
+    out = torch.zeros(tokens, model_dim, dtype=torch.float32, device="cuda")
+    exe = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128,
+                            doweight_stage2=True, out_dtype="f32", accumulate=True, in_dtype="int8")
+    _launch(exe, out, a2q, layout.shuffle_weight(w2q).view(experts * model_dim, inter_dim).contiguous(), sa2, sw2.view(-1, 1),
+            (sid, swt, se, npp[:1].contiguous(), int(se.numel())), model_dim, inter_dim, tokens)
+    ref = O.moe_gemm2(a2q.numpy(), w2q.numpy().reshape(-1, inter_dim), sa2.numpy().reshape(-1), sw2.numpy().reshape(-1), ids.numpy(), wts.numpy(),
+                      model_dim, True, "int8")
+    assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-5 * np.abs(ref).max())  # one addition per element: exact up to fp32 rounding
+
+
+def test_two_stages_end_to_end_with_reduction():
+    # gemm1 -> per-token requantisation -> gemm2 (one row per slot) -> slot reduction, against the same chain in the oracle
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2, compile_moe_reduction
+
+    tokens, model_dim, inter_dim, experts, topk, tile_m = 129, 1024, 256, 8, 2, 32
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(11)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, 11)
+    x = torch.randn(tokens, model_dim, generator=g)
+    w1 = torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim)
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    xq, sx = quant.pertoken_quant(x, quant_dtype=torch.float8_e4m3fn)
+    w1q, sw1 = quant.pertoken_quant(w1, quant_dtype=torch.float8_e4m3fn)
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=torch.float8_e4m3fn)
+    out1 = torch.empty(tokens, topk, inter_dim, dtype=torch.bfloat16, device=dev)
+    e1 = compile_moe_gemm1(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128,
+                           doweight_stage1=False, out_dtype="bf16", in_dtype="fp8")
+    _launch(e1, out1, xq, layout.shuffle_weight(w1q).view(-1, model_dim).contiguous(), sx, sw1.view(-1, 1), routing, inter_dim, model_dim, tokens)
+    a2q, sa2 = quant.pertoken_quant(out1.float().cpu(), quant_dtype=torch.float8_e4m3fn)  # the harness's requantisation (:293-305)
+    out2 = torch.zeros(tokens * topk, model_dim, dtype=torch.bfloat16, device=dev)
+    e2 = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128,
+                           doweight_stage2=True, out_dtype="bf16", accumulate=False, in_dtype="fp8")
+    _launch(e2, out2, a2q, layout.shuffle_weight(w2q).view(-1, inter_dim).contiguous(), sa2, sw2.view(-1, 1), routing, model_dim, inter_dim, tokens)
+    y = torch.empty(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+    compile_moe_reduction(topk=topk, model_dim=model_dim, dtype_str="bf16")(out2, y, None, None, tokens, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    ref1 = O.moe_gemm1(xq.view(torch.uint8).numpy(), w1q.view(torch.uint8).numpy().reshape(-1, model_dim), sx.numpy(), sw1.numpy().reshape(-1),
+                       ids.numpy(), wts.numpy(), inter_dim, False, "fp8")
+    ok, ratio = O.within_north_star_tolerance(out1.float().cpu().numpy(), ref1, 1e-2)
+    assert ok, f"stage 1 outside tolerance ({ratio:.3f})"
+    per_slot = O.moe_gemm2(a2q.view(torch.uint8).numpy(), w2q.view(torch.uint8).numpy().reshape(-1, inter_dim), sa2.numpy().reshape(-1),
+                           sw2.numpy().reshape(-1), ids.numpy(), wts.numpy(), model_dim, True, "fp8", reduce_slots=False)
+    ok, ratio = O.within_north_star_tolerance(out2.float().cpu().numpy(), per_slot.reshape(tokens * topk, model_dim), 1e-2)
+    assert ok, f"stage 2 outside tolerance ({ratio:.3f})"
+    # the reduction adds what stage 2 wrote, in slot order, in fp32, and rounds once
+    want = out2.float().view(tokens, topk, model_dim).sum(dim=1).to(torch.bfloat16)
+    assert torch.equal(y, want)
+
+
+def test_moe_argument_errors():
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2, compile_moe_reduction
+
+    with pytest.raises(ValueError):  # f32 output is atomic-only (tests/kernels/test_moe_gemm_2stage.py:894-906)
+        compile_moe_gemm2(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage2=True, out_dtype="f32", accumulate=False)
+    with pytest.raises(ValueError):
+        compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, out_dtype="f32")
+    with pytest.raises(AssertionError):
+        compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=64, doweight_stage1=False)
+    with pytest.raises(AssertionError):  # model_dim must be an EVEN multiple of tile_k in stage 1
+        compile_moe_gemm1(model_dim=384, inter_dim=128, experts=4, topk=2, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False)
+    with pytest.raises(NotImplementedError):
+        compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, in_dtype="int4")
+    with pytest.raises(ValueError):
+        compile_moe_gemm1(**SHAPE, tile_m=48, tile_n=64, tile_k=128, doweight_stage1=False)
+    with pytest.raises(NotImplementedError):
+        compile_moe_reduction(topk=2, model_dim=256, dtype_str="f32")
+    exe = compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False)
+    z = torch.zeros(16, device="cuda")
+    with pytest.raises(ValueError, match="built for dims"):
+        exe(z, z, z, z, z, z, z, z, z, 8, 256, 128, 1, None)

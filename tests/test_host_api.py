@@ -140,6 +140,27 @@ def test_mx_c_abi_validation_codes():
     assert handle.psg_gemm_mxfp4(ctypes.byref(m), None) == -2
 
 
+def test_moe_c_abi_validation_codes():
+    handle = _lib.lib()
+    m = _lib.MoeArgs()
+    assert handle.psg_moe_gemm(ctypes.byref(m), None) == -1
+    for f in ("out", "x", "w", "scale_x", "scale_w", "sorted_token_ids", "sorted_expert_ids", "sorted_weights", "num_valid_ids"):
+        setattr(m, f, 0x1000)
+    m.tokens, m.topk, m.experts, m.model_dim, m.inter_dim = 8, 2, 4, 256, 128
+    m.sorted_size, m.blocks, m.block_m, m.in_dtype, m.out_dtype, m.stage = 76, 5, 16, 1, 0, 1
+    for field, val, code, word in (("stage", 3, -2, b"stage"), ("in_dtype", 2, -3, b"in_dtype"), ("out_dtype", 2, -3, b"fp32 output"),
+                                   ("block_m", 48, -2, b"block_m"), ("model_dim", 192, -2, b"K=192"), ("inter_dim", 24, -2, b"output width"),
+                                   ("tokens", 1 << 24, -2, b"tokens"), ("blocks", 0, -2, b"blocks"), ("x", 0x1004, -6, b"aligned"), ("pad0", 1, -2, b"pad0")):
+        old = getattr(m, field)
+        setattr(m, field, val)
+        assert handle.psg_moe_gemm(ctypes.byref(m), None) == code, field
+        assert word in handle.psg_last_error(), (field, handle.psg_last_error())
+        setattr(m, field, old)
+    assert handle.psg_moe_reduce(None, None, 1, 1, 4, 0, None) == -1
+    assert handle.psg_moe_reduce(0x1000, 0x1000, 4, 2, 6, 0, None) == -2
+    assert handle.psg_moe_reduce(0x1000, 0x1000, 4, 2, 8, 2, None) == -3
+
+
 def test_mx_quantisers_match_the_oracle_byte_for_byte():
     from flydsl_amd import quant
     from oracle import psg_oracle as O
@@ -334,6 +355,8 @@ def test_struct_layouts_match_header():
         printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(psg_mxfp4_args), offsetof(psg_mxfp4_args, M), offsetof(psg_mxfp4_args, out_dtype),
                offsetof(psg_mxfp4_args, force_path), offsetof(psg_mxfp4_args, a_dtype), offsetof(psg_mxfp4_args, batch),
                offsetof(psg_mxfp4_args, a_row_stride), offsetof(psg_mxfp4_args, scale_a_batch_stride));
+        printf("%zu %zu %zu %zu\n", sizeof(psg_moe_args), offsetof(psg_moe_args, num_valid_ids), offsetof(psg_moe_args, tokens),
+               offsetof(psg_moe_args, accumulate));
         return 0;
     }'''
     with tempfile.TemporaryDirectory() as d:
@@ -346,6 +369,8 @@ def test_struct_layouts_match_header():
     want = [ctypes.sizeof(a), a.workspace_bytes.offset, a.M.offset, a.epilogue.offset, a.force_path.offset, a.bias.offset,
             a.b_layout.offset, ctypes.sizeof(m), m.M.offset, m.out_dtype.offset, m.force_path.offset,
             m.a_dtype.offset, m.batch.offset, m.a_row_stride.offset, m.scale_a_batch_stride.offset]
+    e = _lib.MoeArgs
+    want += [ctypes.sizeof(e), e.num_valid_ids.offset, e.tokens.offset, e.accumulate.offset]
     assert [int(v) for v in out] == want
 
 

@@ -1,0 +1,95 @@
+"""Pins of the MoE oracle functions: sorting by invariants and a hand-worked example, the two stage references by scalar
+float64 loops on tiny inputs, and the product's vectorised sorter against the oracle's loop."""
+
+import math
+
+import numpy as np
+import torch
+
+from oracle import psg_oracle as O
+
+
+def _routing(tokens, experts, topk, seed):
+    g = torch.Generator().manual_seed(seed)
+    score = torch.rand(tokens, experts, generator=g)
+    vals, ids = torch.topk(score, k=topk, dim=1)
+    return ids.numpy().astype(np.int32), torch.softmax(vals, dim=1).numpy().astype(np.float32)
+
+
+def test_moe_sorting_hand_worked_example():
+    # 3 tokens, top-2, 3 experts, blocks of 4: expert 0 <- (t0,s0),(t2,s1); expert 1 <- (t0,s1),(t1,s0),(t2,s0); expert 2 <- (t1,s1)
+    ids = np.array([[0, 1], [1, 2], [1, 0]], dtype=np.int32)
+    w = np.array([[.6, .4], [.7, .3], [.8, .2]], dtype=np.float32)
+    sid, sw, se, npp = O.moe_sorting(ids, w, 3, 4)
+    pad = (2 << 24) | 3
+    assert sid.tolist() == [0, (1 << 24) | 2, pad, pad, (1 << 24) | 0, 1, 2, pad, (1 << 24) | 1, pad, pad, pad, pad, pad, pad, pad]
+    assert se.tolist() == [0, 1, 2, -1]
+    assert npp.tolist() == [12, 3]
+    assert np.allclose(sw[[0, 1, 4, 5, 6, 8]], [.6, .2, .4, .7, .8, .3])
+    assert len(sid) == 3 * 2 + 3 * 4 - 2
+
+
+def test_moe_sorting_invariants_and_product_sorter():
+    from flydsl_amd.kernels.moe.moe_sorting import moe_sorting
+
+    for tokens, experts, topk, bm, seed in [(8, 4, 2, 16, 0), (129, 8, 2, 32, 1), (33, 8, 2, 64, 2), (1, 8, 1, 16, 3), (333, 17, 9, 64, 4), (7, 8, 2, 128, 5)]:
+        ids, w = _routing(tokens, experts, topk, seed)
+        sid, sw, se, npp = O.moe_sorting(ids, w, experts, bm)
+        valid = int(npp[0])
+        assert valid % bm == 0 and npp[1] == tokens
+        blocks = valid // bm
+        assert (se[:blocks] >= 0).all() and (np.diff(se[:blocks]) >= 0).all() and (se[blocks:] == -1).all()
+        seen = set()
+        for i in range(valid):
+            t, s = int(sid[i]) & 0xFFFFFF, int(sid[i]) >> 24
+            if t >= tokens:
+                assert (t, s) == (tokens, topk)
+                continue
+            assert ids[t, s] == se[i // bm] and sw[i] == w[t, s] and (t, s) not in seen
+            seen.add((t, s))
+        assert len(seen) == tokens * topk
+        assert (sid[valid:] == ((topk << 24) | tokens)).all()
+        got = moe_sorting(torch.from_numpy(ids), torch.from_numpy(w), num_experts=experts, block_size=bm)
+        for a, b in zip(got, (sid, sw, se, npp)):
+            assert np.array_equal(a.numpy(), b)
+
+
+def test_moe_stage_references_against_scalar_loops():
+    rng = np.random.default_rng(3)
+    tokens, experts, topk, model_dim, inter = 5, 3, 2, 32, 16
+    ids, w = _routing(tokens, experts, topk, 7)
+    for kind in ("int8", "fp8"):
+        if kind == "int8":
+            xq = rng.integers(-127, 128, (tokens, model_dim)).astype(np.int8)
+            w1q = rng.integers(-127, 128, (experts * 2 * inter, model_dim)).astype(np.int8)
+            w2q = rng.integers(-127, 128, (experts * model_dim, inter)).astype(np.int8)
+            a2q = rng.integers(-127, 128, (tokens, topk, inter)).astype(np.int8)
+            dec = lambda q: q.astype(np.float64)  # noqa: E731
+        else:
+            codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+            xq, w1q = rng.choice(codes, (tokens, model_dim)), rng.choice(codes, (experts * 2 * inter, model_dim))
+            w2q, a2q = rng.choice(codes, (experts * model_dim, inter)), rng.choice(codes, (tokens, topk, inter))
+            dec = lambda q: O.e4m3fn_to_f32(q).astype(np.float64)  # noqa: E731
+        sx = rng.uniform(0.01, 0.02, tokens).astype(np.float32)
+        sw1 = rng.uniform(0.001, 0.002, experts * 2 * inter).astype(np.float32)
+        sa2 = rng.uniform(0.01, 0.02, tokens * topk).astype(np.float32)
+        sw2 = rng.uniform(0.001, 0.002, experts * model_dim).astype(np.float32)
+        for dow in (False, True):
+            want1 = np.zeros((tokens, topk, inter))
+            want2 = np.zeros((tokens, model_dim))
+            for t in range(tokens):
+                for s in range(topk):
+                    e = int(ids[t, s])
+                    for n in range(inter):
+                        g = sum(dec(xq)[t, k] * sx[t] * dec(w1q)[e * 2 * inter + n, k] * sw1[e * 2 * inter + n] for k in range(model_dim))
+                        u = sum(dec(xq)[t, k] * sx[t] * dec(w1q)[e * 2 * inter + inter + n, k] * sw1[e * 2 * inter + inter + n] for k in range(model_dim))
+                        want1[t, s, n] = g / (1 + math.exp(-g)) * u * (w[t, s] if dow else 1.0)
+                    for n in range(model_dim):
+                        y = sum(dec(a2q)[t, s, k] * sa2[t * topk + s] * dec(w2q)[e * model_dim + n, k] * sw2[e * model_dim + n] for k in range(inter))
+                        want2[t, n] += y * (w[t, s] if dow else 1.0)
+            got1 = O.moe_gemm1(xq, w1q, sx, sw1, ids, w, inter, dow, kind)
+            got2 = O.moe_gemm2(a2q, w2q, sa2, sw2, ids, w, model_dim, dow, kind)
+            assert np.allclose(got1, want1, rtol=2e-5, atol=1e-6 * np.abs(want1).max())
+            assert np.allclose(got2, want2, rtol=2e-5, atol=1e-6 * np.abs(want2).max())
+            per_slot = O.moe_gemm2(a2q, w2q, sa2, sw2, ids, w, model_dim, dow, kind, reduce_slots=False)
+            assert np.allclose(per_slot.sum(1), got2, rtol=1e-6, atol=1e-7)
