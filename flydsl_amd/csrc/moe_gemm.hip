@@ -84,7 +84,8 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     for (int s = 0; s < NSET; s++)
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
-            const int n = n0 + (wave * NR + ni) * 16;                 // first column of the block
+            const int n = n0 + (ni * 4 + wave) * 16;                  // first column of the block: the four wavefronts of pass ni
+                                                                      // cover 64 consecutive columns
             const int nb = (n + s * p.n_out) >> 4;
             b_voff[s][ni] = n < p.n_out ? (uint32_t)nb * 16u * (uint32_t)K + (uint32_t)lane * 16u : 0xFFFFFFF0u;
         }
@@ -159,62 +160,75 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
     }
 
-    // epilogue: lane owns rows mi*16 + li, columns n0 + (wave*NR + ni)*16 + lg*4 + 0..3
-    static_for<MR>([&](auto MI) {
-        constexpr int mi = decltype(MI)::value;
-        const int r = mi * 16 + li;
-        const int xr = x_row(r);
-        if (xr >= 0) {
+    // Epilogue, one pass per ni (64 consecutive columns of the tile): every lane finishes its own fragments (rows
+    // mi*16 + li, columns ni*64 + wave*16 + lg*4 + 0..3) into an LDS tile of BM rows (free after the loop's last
+    // barrier; 16-byte granules XOR-swizzled by the row), then the workgroup walks the tile row by row so that one
+    // store or atomic instruction covers whole 128- or 256-byte rows of the output instead of 16 rows x 16 bytes.
+    const bool f32_out = p.out_dtype == OUT_F32;
+    const int esize = f32_out ? 4 : 2;
+    const int row_bytes = 64 * esize;                  // one pass's row in LDS: 128 or 256 bytes (both stages hold BM*256)
+    const int gmask = (row_bytes >> 4) - 1;            // granules per row - 1 (7 or 15)
+    uint8_t* stage = &lds[0][0];
+    static_for<NR>([&](auto NI) {
+        constexpr int ni = decltype(NI)::value;
+        const int ncol = n0 + ni * 64 + wave * 16 + lg * 4;   // first of the lane's four columns
+        v4f swa = {0.f, 0.f, 0.f, 0.f}, swb = {0.f, 0.f, 0.f, 0.f};
+        if (ncol < p.n_out) {
+            swa = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + ncol);
+            if constexpr (STAGE == 1) swb = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + p.n_out + ncol);
+        }
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            const int r = mi * 16 + li;
+            const int xr = x_row(r);
+            const float sx = xr >= 0 ? p.sx[xr] : 0.f;
+            const float rw = (p.doweight && xr >= 0) ? p.sorted_w[blk * BM + r] : 1.0f;
+            v4f y;
+            if constexpr (STAGE == 1) {
+                const acc_t ag = acc[mi][0][ni], au = acc[mi][NSET - 1][ni];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float g = ((float)ag[v] * sx) * swa[v], u = ((float)au[v] * sx) * swb[v];
+                    y[v] = silu(g) * u * rw;
+                }
+            } else {
+                const acc_t a = acc[mi][0][ni];
+#pragma unroll
+                for (int v = 0; v < 4; v++) y[v] = (((float)a[v] * sx) * swa[v]) * rw;
+            }
+            const int cb = (wave * 16 + lg * 4) * esize;      // byte column inside the pass's row
+            uint8_t* dst = stage + r * row_bytes + ((((cb >> 4) ^ r) & gmask) << 4) + (cb & 15);
+            if (f32_out) {
+                *reinterpret_cast<v4f*>(dst) = y;
+            } else {
+                *reinterpret_cast<v2i*>(dst) = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(y[0], y[1], y[2], y[3]) : pack4_out16<OUT_FP16>(y[0], y[1], y[2], y[3]);
+            }
+        });
+        __syncthreads();
+        const bool atomic = STAGE == 2 && p.accumulate;
+        const int unit = atomic ? 4 : 16;                      // bytes one thread moves per trip
+        const int upr = row_bytes / unit;                      // units per row
+        for (int q = tid; q < BM * upr; q += 256) {
+            const int r = q / upr, cb = (q % upr) * unit;
+            const int n = n0 + ni * 64 + cb / esize;
             const uint32_t sid = (uint32_t)ids[r];
             const int t = (int)(sid & 0xFFFFFFu), slot = (int)(sid >> 24);
-            const float sx = p.sx[xr];
-            const float rw = p.doweight ? p.sorted_w[blk * BM + r] : 1.0f;
-            static_for<NR>([&](auto NI) {
-                constexpr int ni = decltype(NI)::value;
-                const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-                if (n < p.n_out) {
-                    v4f y;
-                    if constexpr (STAGE == 1) {
-                        const v4f swg = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + n);
-                        const v4f swu = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + p.n_out + n);
-                        const acc_t ag = acc[mi][0][ni], au = acc[mi][NSET - 1][ni];
-#pragma unroll
-                        for (int v = 0; v < 4; v++) {
-                            const float g = ((float)ag[v] * sx) * swg[v], u = ((float)au[v] * sx) * swu[v];
-                            y[v] = silu(g) * u * rw;
-                        }
-                        const size_t idx = ((size_t)t * p.topk + slot) * (size_t)p.n_out + n;
-                        const v2i o = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(y[0], y[1], y[2], y[3]) : pack4_out16<OUT_FP16>(y[0], y[1], y[2], y[3]);
-                        *reinterpret_cast<v2i*>(static_cast<uint16_t*>(p.out) + idx) = o;
-                    } else {
-                        const v4f sw = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + n);
-                        const acc_t a = acc[mi][0][ni];
-#pragma unroll
-                        for (int v = 0; v < 4; v++) y[v] = (((float)a[v] * sx) * sw[v]) * rw;
-                        if (!p.accumulate) {
-                            const size_t idx = ((size_t)t * p.topk + slot) * (size_t)p.n_out + n;
-                            const v2i o = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(y[0], y[1], y[2], y[3]) : pack4_out16<OUT_FP16>(y[0], y[1], y[2], y[3]);
-                            *reinterpret_cast<v2i*>(static_cast<uint16_t*>(p.out) + idx) = o;
-                        } else {
-                            const size_t idx = (size_t)t * (size_t)p.n_out + n;
-                            if (p.out_dtype == OUT_F32) {
-                                float* o = static_cast<float*>(p.out) + idx;
-#pragma unroll
-                                for (int v = 0; v < 4; v++) unsafeAtomicAdd(o + v, y[v]);
-                            } else if (p.out_dtype == OUT_FP16) {
-                                auto* o = (__attribute__((address_space(1))) v2h*)(static_cast<uint16_t*>(p.out) + idx);
-                                __builtin_amdgcn_global_atomic_fadd_v2f16(o, (v2h){(__fp16)y[0], (__fp16)y[1]});
-                                __builtin_amdgcn_global_atomic_fadd_v2f16(o + 1, (v2h){(__fp16)y[2], (__fp16)y[3]});
-                            } else {
-                                auto* o = (__attribute__((address_space(1))) v2b*)(static_cast<uint16_t*>(p.out) + idx);
-                                __builtin_amdgcn_global_atomic_fadd_v2bf16(o, (v2b){(__bf16)y[0], (__bf16)y[1]});
-                                __builtin_amdgcn_global_atomic_fadd_v2bf16(o + 1, (v2b){(__bf16)y[2], (__bf16)y[3]});
-                            }
-                        }
-                    }
+            if (t < p.tokens && slot < p.topk && n < p.n_out) {
+                const uint8_t* src = stage + r * row_bytes + ((((cb >> 4) ^ r) & gmask) << 4) + (cb & 15);
+                const size_t orow = atomic ? (size_t)t : (size_t)t * p.topk + slot;
+                uint8_t* o = static_cast<uint8_t*>(p.out) + (orow * (size_t)p.n_out + n) * esize;
+                if (!atomic) {
+                    *reinterpret_cast<v4i*>(o) = *reinterpret_cast<const v4i*>(src);
+                } else if (f32_out) {
+                    unsafeAtomicAdd(reinterpret_cast<float*>(o), *reinterpret_cast<const float*>(src));
+                } else if (p.out_dtype == OUT_FP16) {
+                    __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) v2h*)o, *reinterpret_cast<const v2h*>(src));
+                } else {
+                    __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) v2b*)o, *reinterpret_cast<const v2b*>(src));
                 }
-            });
+            }
         }
+        if constexpr (ni + 1 < NR) __syncthreads();
     });
 }
 
