@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
+typedef float v16f __attribute__((ext_vector_type(16)));
 #define CK(x) do{hipError_t e=(x); if(e!=hipSuccess){printf("HIP error %s at %d\n",hipGetErrorString(e),__LINE__); exit(1);} }while(0)
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -45,23 +46,26 @@ __global__ void __launch_bounds__(512) k_lds(int iters, unsigned long long* out)
   if(acc[0]+acc[1]+acc[2]+acc[3]==12345) out[0]=1;
 }
 // ---- MFMA only: 8 independent accumulators per wavefront, operands random or zero ----
-// KIND 0: fp8 16x16x128 (65536 flop), 1: int8 16x16x64 (32768 op), 2: fp4 16x16x128 with e8m0 scales (65536 flop)
+// KIND 0: fp8 16x16x128 (65536 flop), 1: int8 16x16x64 (32768 op), 2: fp4 16x16x128 with e8m0 scales (65536 flop),
+// 3: fp8 32x32x64 (131072 flop, four accumulators of 16 registers)
 template<int KIND>
 __global__ void __launch_bounds__(512) k_mfma(int iters, const int* src, unsigned long long* out){
   v8i a, b; for(int i=0;i<8;i++){ a[i]=src[(threadIdx.x*8+i)&4095]; b[i]=src[(threadIdx.x*8+i+2048)&4095]; }
   v4i a4={a[0],a[1],a[2],a[3]}, b4={b[0],b[1],b[2],b[3]};
   v4f c[8]; v4i ci[8]; for(int i=0;i<8;i++){ c[i]=(v4f){0,0,0,0}; ci[i]=(v4i){0,0,0,0}; }
+  v16f cw[4]; for(int i=0;i<4;i++) for(int j=0;j<16;j++) cw[i][j]=0.f;
   unsigned long long w0=wall_clock64(); long long t0=clock64();
   for(int it=0;it<iters;it++){
 #pragma unroll
     for(int i=0;i<8;i++){
-      if constexpr (KIND==0) c[i]=__builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a,b,c[i],0,0,0,0,0,0);
+      if constexpr (KIND==3) cw[i&3]=__builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a,b,cw[i&3],0,0,0,0,0,0);
+      else if constexpr (KIND==0) c[i]=__builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a,b,c[i],0,0,0,0,0,0);
       else if constexpr (KIND==1) ci[i]=__builtin_amdgcn_mfma_i32_16x16x64_i8(a4,b4,ci[i],0,0,0);
       else c[i]=__builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a,b,c[i],4,4,0,0x7f7f7f7f,0,0x7f7f7f7f);
     }
   }
   long long t1=clock64(); unsigned long long w1=wall_clock64();
-  float s=0; for(int i=0;i<8;i++) s+=c[i][0]+(float)ci[i][0];
+  float s=0; for(int i=0;i<8;i++) s+=c[i][0]+(float)ci[i][0]+cw[i&3][i];
   if((threadIdx.x&63)==0){ int w=blockIdx.x*(blockDim.x/64)+(threadIdx.x>>6); out[w*2]=t1-t0; out[w*2+1]=w1-w0; }
   if(s==12345.f) out[0]=1;
 }
@@ -112,12 +116,17 @@ int main(){
     k_lds<1><<<256,th>>>(iters,d); snprintf(nm,96,"LDS ds_read_b128 A-fragment pattern, %d waves/CU",th/64); report(nm,256*th/64,(double)iters*8*1024,"B",1e12);
   }
   int* src; CK(hipMalloc(&src,4096*4)); std::vector<int> hs(4096);
-  for(int mode=0;mode<2;mode++){ for(auto&x:hs) x= mode? 0 : (rand()&0x77777777); CK(hipMemcpy(src,hs.data(),4096*4,hipMemcpyHostToDevice));
-    const char* dn = mode ? "zero" : "random";
+  // operand data: "random" = random bytes with the top bit of every nibble clear (all fp8 values positive), "zero",
+  // "signed" = fp8 bytes with random sign, exponent field 4..10 and random mantissa (what quantised GEMM operands look like)
+  for(int mode=0;mode<3;mode++){
+    for(auto&x:hs){ if(mode==0) x=rand()&0x77777777; else if(mode==1) x=0; else { unsigned v=0; for(int b=0;b<4;b++) v|=(unsigned)(((rand()&1)<<7)|(((rand()%7)+4)<<3)|(rand()&7))<<(8*b); x=(int)v; } }
+    CK(hipMemcpy(src,hs.data(),4096*4,hipMemcpyHostToDevice));
+    const char* dn = mode==0 ? "random" : (mode==1 ? "zero" : "signed");
     for(int th: {256,512}){ char nm[96]; int w=256*th/64;
       k_mfma<0><<<256,th>>>(100000,src,d); snprintf(nm,96,"MFMA only fp8 16x16x128, %s operands, %d waves/SIMD",dn,th/256); report(nm,w,(double)100000*8*65536,"flop",1e12);
       k_mfma<1><<<256,th>>>(200000,src,d); snprintf(nm,96,"MFMA only int8 16x16x64, %s operands, %d waves/SIMD",dn,th/256); report(nm,w,(double)200000*8*32768,"flop",1e12);
       k_mfma<2><<<256,th>>>(200000,src,d); snprintf(nm,96,"MFMA only fp4 16x16x128 scaled, %s operands, %d waves/SIMD",dn,th/256); report(nm,w,(double)200000*8*65536,"flop",1e12);
+      k_mfma<3><<<256,th>>>(50000,src,d); snprintf(nm,96,"MFMA only fp8 32x32x64, %s operands, %d waves/SIMD",dn,th/256); report(nm,w,(double)50000*8*131072,"flop",1e12);
     } }
   v4i* big; CK(hipMalloc(&big,(size_t)64*4096*16)); CK(hipMemset(big,1,(size_t)64*4096*16));
   k_l2<<<256,256>>>(4000,big,d); report("vector loads 16 B/lane hitting L2 (4 MB footprint), 4 waves/CU",1024,(double)4000*8*1024,"B",1e12);
