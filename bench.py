@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the preshuffle quantized GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu] [--next-rows]
 
 A step is one GEMM launch on one set of synthetic operands (seed 0; activations N(0,1), weights
 N(0,0.02), quantised and preshuffled on the host, resident in HBM before the timed region).
@@ -252,6 +252,79 @@ def run_quant_workload(name, steps=50, warmup=5):
                          "traffic": None, "algorithmic_bytes": nbytes}}
 
 
+def run_next_row_workloads():
+    """Timings of the kernels of the rows next to the hot path (``--next-rows``): the general MX kernel on the reference's
+    test shapes and the two MoE stages.  HIP events around plain launch loops (every kernel here runs for >= 15 us, so
+    launch gaps hide behind the previous kernel); weights sized beyond the Infinity Cache where the shape allows."""
+    import math as _m
+
+    import torch
+
+    from flydsl_amd import layout, quant
+    from flydsl_amd.kernels.moe.moe_sorting import moe_sorting
+    from flydsl_amd.synthetic import make_mx
+    from kernels.gemm.mxfp4_preshuffle import launch_gemm
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+
+    dev = torch.device("cuda:0")
+
+    def timed(f, iters=20):
+        for _ in range(3):
+            f()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                f()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e-3 / iters)
+        return best
+
+    out = []
+    for af, bf in (("fp8", "fp8"), ("fp6", "fp4"), ("fp8", "fp4")):
+        for M in (1024, 64, 32):
+            N = K = 8192
+            d = make_mx(min(M, 256), 512, K, af, bf, seed=0)
+            rep = lambda t, n: t.repeat((n + t.shape[0] - 1) // t.shape[0], 1)[:n].contiguous().to(dev)  # noqa: E731
+            a, b = rep(d["a_q"], M), rep(d["b_shuf"].view(512, -1), N)
+            sa = d["sa_shuf"].view(-1).repeat((M + 255) // 256 + 1).contiguous().to(dev)
+            sb = d["sb_shuf"].view(-1).repeat(N // 512).contiguous().to(dev)
+            c = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+            sec = timed(lambda: launch_gemm(c, a, b, sa, sb, M, N, None, N, K, 64, 256, 256, af, "bf16", bf, 1, -1, -1, -1, -1, -1, -1, 0, 0))
+            wbytes = N * K // (2 if bf == "fp4" else 1)
+            out.append({"workload": f"mx_{af}x{bf}_m{M}_n8192_k8192", "us_per_launch_events": sec * 1e6, "tflops": 2.0 * M * N * K / sec / 1e12,
+                        "weight_gb_per_s": wbytes / sec / 1e9})
+    for tokens, model_dim, inter_dim, experts, topk, tile_m in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 16), (333, 4096, 2048, 17, 9, 64)):
+        g = torch.Generator().manual_seed(0)
+        vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
+        sid, swt, se, npp = [t.to(dev) for t in moe_sorting(ids.int(), torch.softmax(vals, 1), num_experts=experts, block_size=tile_m)]
+        qd = torch.float8_e4m3fn
+        xq, sx = quant.pertoken_quant(torch.randn(tokens, model_dim, generator=g), quant_dtype=qd)
+        w1q = layout.shuffle_weight((torch.randn(experts * 2 * inter_dim, model_dim, generator=g) / _m.sqrt(model_dim) * 40).to(qd))
+        w2q = layout.shuffle_weight((torch.randn(experts * model_dim, inter_dim, generator=g) / _m.sqrt(inter_dim) * 40).to(qd))
+        a2q, sa2 = quant.pertoken_quant(torch.randn(tokens * topk, inter_dim, generator=g), quant_dtype=qd)
+        sw1 = torch.full((experts * 2 * inter_dim,), 0.025, device=dev)
+        sw2 = torch.full((experts * model_dim,), 0.025, device=dev)
+        xq, w1q, w2q, a2q, sx, sa2 = [t.to(dev).contiguous().view(-1) for t in (xq, w1q, w2q, a2q, sx, sa2)]
+        out1 = torch.empty(tokens, topk, inter_dim, dtype=torch.bfloat16, device=dev)
+        out2 = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+        nv, blocks = npp[:1].contiguous(), int(se.numel())
+        kw = dict(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128, in_dtype="fp8")
+        e1 = compile_moe_gemm1(doweight_stage1=False, out_dtype="bf16", **kw)
+        e2 = compile_moe_gemm2(doweight_stage2=True, out_dtype="bf16", accumulate=True, **kw)
+        s1 = timed(lambda: e1(out1, xq, w1q, sx, sw1, sid, se, swt, nv, tokens, inter_dim, model_dim, blocks, None))
+        s2 = timed(lambda: e2(out2, a2q, w2q, sa2, sw2, sid, se, swt, nv, tokens, model_dim, inter_dim, blocks, None))
+        tag = f"tokens{tokens}_e{experts}_top{topk}_model{model_dim}_inter{inter_dim}_block{tile_m}"
+        out.append({"workload": f"moe_fp8_stage1_{tag}", "us_per_launch_events": s1 * 1e6, "tflops": 2.0 * tokens * topk * 2 * inter_dim * model_dim / s1 / 1e12,
+                    "weight_gb_per_s": experts * 2 * inter_dim * model_dim / s1 / 1e9})
+        out.append({"workload": f"moe_fp8_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
+                    "weight_gb_per_s": experts * model_dim * inter_dim / s2 / 1e9})
+    return out
+
+
 def cpu_baseline(name, host, budget_s=12.0):  # budget_s bounds the CPU work of one workload
     """The reference's torch CPU path (dequantise to fp32 + torch.mm) on the same seeded operands,
     timed on this box's host cores.  For workloads whose single pass exceeds the budget a row sample of
@@ -311,6 +384,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--next-rows", action="store_true",
+                    help="also time the general MX kernel and the MoE stages (rows next to the hot path); adds a next_rows list")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy a few times (the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against)")
@@ -363,6 +438,7 @@ def main():
             others.append(r)
         for name in ("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"):
             others.append(run_quant_workload(name))
+    next_rows = run_next_row_workloads() if args.next_rows else None
 
     line = {
         "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",
@@ -392,6 +468,8 @@ def main():
         "cpu_baseline": cpu,
         "per_config": others,
     }
+    if next_rows is not None:
+        line["next_rows"] = next_rows
     # the metric names two operating points; the second one (MFMA-bound prefill) is lifted out of the table for convenience
     for r in others:
         if r["workload"] == "fp8_prefill_m8192":
