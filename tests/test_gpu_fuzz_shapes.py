@@ -77,3 +77,22 @@ def test_fuzz_mxfp4():
         ref = O.run_torch_w4(d["a_q"].numpy(), d["b_q"].numpy(), d["sa"].numpy(), d["sb"].numpy())
         ok, ratio = O.within_north_star_tolerance(c.float().cpu().numpy(), ref)
         assert ok, (M, N, K, ratio)
+
+
+@pytest.mark.parametrize("a_dtype,b_dtype", [("fp8", "fp8"), ("fp6", "fp4"), ("fp8", "fp4"), ("fp4", "fp8")])
+def test_fuzz_mx_formats(a_dtype, b_dtype):
+    # the general MX kernel through the automatic dispatcher (split-K plan included), ragged M, any N % 32, K % 256
+    from helpers import make_mx
+    from kernels.gemm.mxfp4_preshuffle import launch_gemm
+
+    dev = torch.device("cuda")
+    for i, (M, N, K) in enumerate(_shapes(7, 10, 256, 32, 2048) + [(32, 512, 8192), (64, 1024, 4096)]):
+        d = make_mx(M, N, K, a_dtype, b_dtype, seed=300 + i)
+        c = torch.full((M + 3, N), -8192.0, dtype=torch.bfloat16, device=dev)
+        launch_gemm(c, d["a_q"].to(dev), d["b_shuf"].to(dev), d["sa_shuf"].to(dev), d["sb_shuf"].to(dev), M, N, None, N, K, 64, 128, 256,
+                    a_dtype, "bf16", b_dtype, 1, -1, -1, -1, -1, -1, -1, 0, 0)
+        torch.cuda.synchronize()
+        assert (c[M:] == -8192.0).all(), (M, N, K)
+        ref = O.run_torch_mx(d["a_q"].numpy(), d["b_q"].numpy(), d["sa"].numpy(), d["sb"].numpy(), a_dtype, b_dtype)
+        ok, ratio = O.within_north_star_tolerance(c[:M].float().cpu().numpy(), ref)
+        assert ok, (M, N, K, ratio)

@@ -228,3 +228,51 @@ def test_moe_argument_errors():
     z = torch.zeros(16, device="cuda")
     with pytest.raises(ValueError, match="built for dims"):
         exe(z, z, z, z, z, z, z, z, z, 8, 256, 128, 1, None)
+
+
+def test_moe_stages_replay_from_a_graph():
+    # both stages record into a HIP graph (no allocation, no host read of the routing); the accumulating stage 2 is
+    # cleared by a fill kernel inside the graph; every replay must reproduce the eager result
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+
+    tokens, model_dim, inter_dim, experts, topk, tile_m = 40, 512, 256, 8, 2, 32
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(21)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, 21)
+    sid, swt, se, nv, blocks = [t.to(dev) if torch.is_tensor(t) else t for t in routing]
+    xq, sx = quant.pertoken_quant(torch.randn(tokens, model_dim, generator=g), quant_dtype=torch.int8)
+    w1q, sw1 = quant.pertoken_quant(torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim), quant_dtype=torch.int8)
+    w2q, sw2 = quant.pertoken_quant(torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim), quant_dtype=torch.int8)
+    a2q, sa2 = quant.pertoken_quant(torch.randn(tokens * topk, inter_dim, generator=g), quant_dtype=torch.int8)
+    dv = lambda t: t.to(dev).contiguous().view(-1)  # noqa: E731
+    xq, sx, sw1, sw2, a2q, sa2 = dv(xq), dv(sx), dv(sw1), dv(sw2), dv(a2q), dv(sa2)
+    w1s, w2s = dv(layout.shuffle_weight(w1q)), dv(layout.shuffle_weight(w2q))
+    kw = dict(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128, in_dtype="int8")
+    e1 = compile_moe_gemm1(doweight_stage1=False, out_dtype="bf16", **kw)
+    e2 = compile_moe_gemm2(doweight_stage2=True, out_dtype="f32", accumulate=True, **kw)
+    out1 = torch.empty(tokens, topk, inter_dim, dtype=torch.bfloat16, device=dev)
+    out2 = torch.empty(tokens, model_dim, dtype=torch.float32, device=dev)
+
+    def run():
+        s = torch.cuda.current_stream()
+        e1(out1, xq, w1s, sx, sw1, sid, se, swt, nv, tokens, inter_dim, model_dim, blocks, s)
+        out2.zero_()
+        e2(out2, a2q, w2s, sa2, sw2, sid, se, swt, nv, tokens, model_dim, inter_dim, blocks, s)
+
+    run()
+    torch.cuda.synchronize()
+    want1, want2 = out1.clone(), out2.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run()
+    for _ in range(3):
+        out1.fill_(7.0)
+        out2.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out1, want1)
+        # fp32 atomics: one addition per slot, order not fixed -> equal up to fp32 rounding
+        assert torch.allclose(out2, want2, rtol=1e-5, atol=1e-5 * float(want2.abs().max()))
