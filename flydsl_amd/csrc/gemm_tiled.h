@@ -22,6 +22,10 @@
 //             shuffled e8m0 scale layout; two v_mfma_scale_f32_16x16x128_f8f6f4 per step (one per 64-byte
 //             half = one preshuffled block), each lane's 16 bytes are 32 consecutive K elements sharing one
 //             scale byte, selected from the lane's scale dword with op_sel (byte = 2*half + 16-row half).
+//       mxfp8: e4m3fn x e4m3fn with one e8m0 scale per 32 K elements: the data path of fp8 (one 16x16x128 MFMA per
+//             128-byte step, both 64-byte halves), the scale path of mxfp4 with two K steps per 256-element scale
+//             chunk (op_sel byte = 2*(step parity) + 16-row half; a lane's scale applies to elements [32g, 32g+32)
+//             while its data are [16g, 16g+16) and [64+16g, 64+16g+16): the hardware pairs them up by K index).
 //   * Workgroup ids are remapped so that the ids the hardware deals to one XCD cover a compact
 //     group_m x tiles_n patch of tiles (A and B panels stay in that XCD's L2).
 #pragma once
@@ -66,6 +70,15 @@ __device__ __forceinline__ void mfma_mx(v4f& c, const v4i& a, const v4i& b, int 
                  : "v"(a), "v"(b), "v"(s0), "v"(s1), "n"(LO0), "n"(LO1), "n"(HI));
 }
 
+// fp8 x fp8 with per-lane e8m0 scales (MXFP8): one MFMA covers the whole 128-element step; HI = its parity in the
+// 256-element scale chunk
+template <int HI, int LO0, int LO1>
+__device__ __forceinline__ void mfma_mx8(v4f& c, const v8i& a, const v8i& b, int s0, int s1) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%7,0]"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "v"(s0), "v"(s1), "n"(LO0), "n"(LO1), "n"(HI));
+}
+
 // LDS byte offset of 16-byte chunk `kc` (0..7) of row `row` inside one A stage
 __device__ __forceinline__ int lds_off(int row, int kc) { return row * TK + ((kc ^ ((row >> 1) & 7)) << 4); }
 
@@ -73,10 +86,14 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
     psg_tile_order(id, tiles_m, tiles_n, group_m, &tm, &tn);
 }
 
+// Two workgroups per CU are asked for where 128 + 128 registers per lane suffice; the 128x256 tile of the MX kinds
+// (scale dwords on top of the operands) does not fit that and is left to the register allocator (it spilled 172 bytes per
+// lane into the K loop when forced: MXFP4 4096x7168x2048 82 us).
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
 template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4>
-__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 : 1)) k_a8w8_tiled(A8W8Params p) {
+__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 && !((KIND == KIND_MXFP4 || KIND == KIND_MXFP8) && MR * NR == 32) ? 2 : 1))
+k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr int WN = WAVES / WM;
     constexpr int TM = 16 * MR * WM;
@@ -103,6 +120,7 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
     // K counts BYTES of one operand row from here on (two fp4 elements per byte)
     constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
     constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;  // per-token x per-channel fp32 scales in the epilogue
+    constexpr bool MX = KIND == KIND_MXFP4 || KIND == KIND_MXFP8;   // e8m0 scales applied by the MFMA
     const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : (IS16 ? (p.K << 1) : p.K);
     const int KT = (K + TK - 1) / TK;
     // split-K: workgroup blockIdx.y of p.splits covers K steps [kt_begin, kt_end) and (STORE_ACC only) writes its
@@ -125,9 +143,10 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
     constexpr int MP = MR / 2 > 0 ? MR / 2 : 1, NP = NR / 2 > 0 ? NR / 2 : 1;
     __amdgpu_buffer_rsrc_t rsa = ra, rsb = ra;
     uint32_t chunk_bytes = 0;
-    if constexpr (KIND == KIND_MXFP4) {
-        static_assert(KIND != KIND_MXFP4 || (MR % 2 == 0 && NR % 2 == 0), "scale chunks cover 32 rows");
-        chunk_bytes = (uint32_t)KT * 256u;
+    if constexpr (MX) {
+        static_assert(!MX || (MR % 2 == 0 && NR % 2 == 0), "scale chunks cover 32 rows");
+        // one 256-byte block of scale dwords per 256 K elements: every K step for mxfp4, every second one for mxfp8
+        chunk_bytes = KIND == KIND_MXFP4 ? (uint32_t)KT * 256u : (uint32_t)(p.K >> 8) * 256u;
         const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5), sa_first = (uint64_t)((m0 >> 5) + wm * MP);
         rsa = make_rsrc(p.mx_sa + (sa_first < sa_chunks ? sa_first : sa_chunks) * chunk_bytes,
                         sa_first < sa_chunks ? (sa_chunks - sa_first) * chunk_bytes : 0);
@@ -171,7 +190,7 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
     // MXFP4: load number 2*NR + q fetches scale dword q of the step (A-side chunks first, then W-side)
     auto load_sc1 = [&](int kt, int q, int* sa_dst, int* sb_dst) {
         const bool has = kt < kt_end;
-        const uint32_t soff = has ? (uint32_t)kt * 256u : 0u;
+        const uint32_t soff = has ? (uint32_t)(KIND == KIND_MXFP8 ? (kt >> 1) : kt) * 256u : 0u;
         if (q < MP) {
             sa_dst[q] = buf_load4(rsa, has ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, soff);
         } else {
@@ -207,7 +226,7 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
     auto step = [&](int kt, auto SP) {
         constexpr int S = decltype(SP)::value;
         constexpr int HALF = MR / 2;
-        constexpr int N_LOADS = 2 * NR + (KIND == KIND_MXFP4 ? MP + NP : 0);  // W fragments (+ scale dwords)
+        constexpr int N_LOADS = 2 * NR + (MX ? MP + NP : 0);  // W fragments (+ scale dwords)
         constexpr int B_PER = (N_LOADS + HALF - 1) / HALF;
         // A fragments are read FRAG_AHEAD m-blocks ahead of the MFMAs that use them (register ring buffer)
         constexpr int FRAG_AHEAD = MR >= 4 ? 2 : 1;
@@ -264,6 +283,15 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
                     constexpr int ni = decltype(NI)::value;
                     mfma_mx<1, ni & 1, mi & 1>(acc[mi][ni], bhi[S][ni], ahi, sbv[S][ni / 2], sav[S][mi / 2]);
                 });
+            } else if constexpr (KIND == KIND_MXFP8) {
+                // step parity S = 128-element half of the scale chunk: K ranges start at even steps (no split-K here)
+                const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    const v8i bf = {blo[S][ni][0], blo[S][ni][1], blo[S][ni][2], blo[S][ni][3],
+                                    bhi[S][ni][0], bhi[S][ni][1], bhi[S][ni][2], bhi[S][ni][3]};
+                    mfma_mx8<S, ni & 1, mi & 1>(acc[mi][ni], bf, af, sbv[S][ni / 2], sav[S][mi / 2]);
+                });
             } else {
                 const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
 #pragma unroll
@@ -290,7 +318,7 @@ __global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 ? 2 :
     for (int j = 0; j < A_LOADS; j++) load_a1(kt_begin, j, areg[j]);
 #pragma unroll
     for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin, idx, blo[0], bhi[0]);
-    if constexpr (KIND == KIND_MXFP4) {
+    if constexpr (MX) {
 #pragma unroll
         for (int q = 0; q < MP + NP; q++) load_sc1(kt_begin, q, sav[0], sbv[0]);
     }
@@ -435,7 +463,7 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
     PSG_CASE(8, 4, 1)
     PSG_CASE(4, 4, 1)
     PSG_CASE(2, 4, 1)
-    if constexpr (KIND == KIND_MXFP4) {
+    if constexpr (KIND == KIND_MXFP4 || KIND == KIND_MXFP8) {
         PSG_CASE(4, 2, 1)
         PSG_CASE(2, 2, 1)
     } else {

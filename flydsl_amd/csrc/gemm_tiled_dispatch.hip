@@ -1,6 +1,6 @@
 // Host entry of the tiled MFMA mainloop used by the C-ABI layer.  kind: KIND_INT8 / KIND_FP8 / KIND_FP16 / KIND_BF16 /
-// KIND_MXFP4.  tile_m x tile_n must be one of the instantiated shapes: 256x256, 128x512, 128x256, 64x256, 32x256, then
-// 128x128 and 64x64 (8- and 16-bit) or 64x128 and 32x128 (MXFP4).
+// KIND_MXFP4 / KIND_MXFP8.  tile_m x tile_n must be one of the instantiated shapes: 256x256, 128x512, 128x256, 64x256, 32x256, then
+// 128x128 and 64x64 (8- and 16-bit) or 64x128 and 32x128 (MXFP4, MXFP8).
 #include "psg_common.h"
 #include "tile_order.h"
 
@@ -9,6 +9,7 @@ hipError_t psg_launch_tiled_fp8(const A8W8Params& p, int store, int tile_m, int 
 hipError_t psg_launch_tiled_fp16(const A8W8Params& p, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_tiled_bf16(const A8W8Params& p, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_tiled_mxfp4(const A8W8Params& p, int store, int tile_m, int tile_n, hipStream_t stream);
+hipError_t psg_launch_tiled_mxfp8(const A8W8Params& p, int store, int tile_m, int tile_n, hipStream_t stream);
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream) {
     // the plain bf16 store without bias/activation has its own instantiation; everything else is the generic epilogue
@@ -19,6 +20,7 @@ hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int t
         case KIND_FP16: return psg_launch_tiled_fp16(p, store, tile_m, tile_n, stream);
         case KIND_BF16: return psg_launch_tiled_bf16(p, store, tile_m, tile_n, stream);
         case KIND_MXFP4: return psg_launch_tiled_mxfp4(p, store, tile_m, tile_n, stream);
+        case KIND_MXFP8: return psg_launch_tiled_mxfp8(p, store, tile_m, tile_n, stream);
     }
     return hipErrorInvalidValue;
 }

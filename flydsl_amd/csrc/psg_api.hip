@@ -70,8 +70,8 @@ struct Tile {
 // tile of eight wavefronts side by side along N loads every W fragment once per CU and moves the least data per flop:
 // on real data the chip is power-limited, so that is what decides (fp8 8192x4096x4096: 117 us against 134 us for
 // the 128x256 tile that runs two workgroups per CU; int8 4096x28672x8192: 775 against 940).  MXFP4 4096x7168x2048:
-// 45 us with eight wavefronts against 52 with four, and 82 for the 128x256 tile, whose two workgroups per CU ask the
-// L2 for 47 bytes per clock at fp4 MFMA speed.  The score multiplies the efficiency by
+// 46 us with eight wavefronts against 52 with four, 58 for the 128x256 tile (one workgroup per CU: with two it spilled) and
+// 48 for 64x256; MXFP4 1024x8192x8192, where 256x256 gives only 128 tiles: 40 us with 128x256 against 59.  The score multiplies the efficiency by
 // how evenly the tiles fill the CUs' workgroup slots and by the fraction of each tile that is not padding.
 Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     struct Shape {
@@ -80,7 +80,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     };
     static const Shape shapes8[] = {{256, 256, 8, 1, 1.17}, {128, 256, 4, 2, 1.00}, {64, 256, 4, 2, 0.62}, {32, 256, 4, 3, 0.36},
                                     {128, 128, 4, 2, 0.70}, {64, 64, 4, 5, 0.25}};
-    static const Shape shapesx[] = {{256, 256, 8, 1, 1.00}, {128, 256, 4, 2, 0.86}, {64, 256, 4, 2, 0.80}, {32, 256, 4, 3, 0.40},
+    static const Shape shapesx[] = {{256, 256, 8, 1, 1.00}, {128, 256, 4, 1, 0.80}, {64, 256, 4, 2, 0.75}, {32, 256, 4, 3, 0.40},
                                     {64, 128, 4, 3, 0.40}, {32, 128, 4, 4, 0.25}};
     const Shape* shapes = mx ? shapesx : shapes8;
     if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n, 4};  // forced by the caller; the launcher rejects unknown shapes
@@ -365,9 +365,38 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     if (a->force_path < 0 || a->force_path > 3) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
     const bool dense = a_rs == a_row && c_rs == (uint64_t)a->N && sa_cs == chunk;
     const bool fp4_fast = a->a_dtype == PSG_MX_FP4 && a->b_dtype == PSG_MX_FP4 && batch == 1 && dense;
-    if ((a->force_path == 1 || a->force_path == 2) && !fp4_fast)
-        return fail(PSG_E_SHAPE, "force_path=%d is for dense, unbatched fp4 x fp4 only", a->force_path);
+    // fp8 x fp8 (MXFP8) also runs on the tiled mainloop when the problem has enough 128x256 tiles to fill the GPU (that
+    // kernel has no split-K for this format; decode-like shapes go to the general kernel and its split-K plan)
+    const bool fp8_pair = a->a_dtype == PSG_MX_FP8 && a->b_dtype == PSG_MX_FP8 && batch == 1 && dense;
+    const bool fp8_tiled = fp8_pair && a->force_path != 3 &&
+                           (a->force_path == 1 || (a->M > kSmallM && (long)((a->M + 127) / 128) * (long)((a->N + 255) / 256) >= 192));
+    if (a->force_path == 2 && !fp4_fast) return fail(PSG_E_SHAPE, "force_path=2 is for dense, unbatched fp4 x fp4 only");
+    if (a->force_path == 1 && !fp4_fast && !fp8_pair)
+        return fail(PSG_E_SHAPE, "force_path=1 is for dense, unbatched fp4 x fp4 or fp8 x fp8 only");
     if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    if (fp8_tiled) {
+        const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
+        const Tile t = forced ? Tile{a->tile_m, a->tile_n, 4} : pick_tile(a->M, a->N, true, 0, 0);
+        A8W8Params q{};
+        q.c = out;
+        q.a = static_cast<const uint8_t*>(a->a);
+        q.b = static_cast<const uint8_t*>(a->b);
+        q.mx_sa = static_cast<const uint8_t*>(a->scale_a);
+        q.mx_sb = static_cast<const uint8_t*>(a->scale_b);
+        q.M = a->M;
+        q.N = a->N;
+        q.K = a->K;
+        q.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;
+        q.ksplit = 1;
+        q.wave_layout = a->reserved >= 2 ? a->reserved : 1;  // four wavefronts: 8192x4096x4096 117 us against 130 with eight
+        q.splits = 1;
+        q.epi = EPI_NONE;
+        q.out = a->out_dtype;
+        const hipError_t te = psg_launch_a8w8_tiled(q, KIND_MXFP8, store, t.m, t.n, static_cast<hipStream_t>(stream));
+        if (te != hipSuccess) return hip_fail(te, "psg_gemm_mxfp4 launch");
+        g_err[0] = 0;
+        return 0;
+    }
     if (a->force_path == 3 || !fp4_fast) {
         MxGenParams g;
         g.c = out;

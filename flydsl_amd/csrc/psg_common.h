@@ -12,7 +12,7 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3, KIND_MXFP4 = 4 };
+enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3, KIND_MXFP4 = 4, KIND_MXFP8 = 5 };
 enum { OUT_BF16 = 0, OUT_FP16 = 1 };
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_RELU = 2, EPI_BIAS_SILU = 3, EPI_BIAS_GELU = 4 };
 // what a kernel writes: the scaled/activated C, or the raw accumulators

@@ -225,3 +225,46 @@ def test_bad_arguments_are_rejected():
     with pytest.raises(ValueError, match="c_row_stride"):  # a row stride below N comes back from the C ABI
         launch_gemm(c, d["a_q"].to(dev), d["b_shuf"].to(dev), d["sa_shuf"].to(dev), d["sb_shuf"].to(dev), 32, 128,
                     torch.cuda.current_stream(), 128, 256, 32, 128, 256, "fp8", "bf16", "fp8", 1, -1, -1, -1, -1, 64, -1, 0, 0)
+
+
+# ---- fp8 x fp8 on the tiled mainloop (problems with enough tiles; forced here on small shapes) -------------------------
+@pytest.mark.parametrize("tile", [(256, 256), (128, 512), (128, 256), (64, 256), (32, 256), (64, 128), (32, 128)])
+@pytest.mark.parametrize("M,N,K", [(64, 512, 512), (133, 288, 768), (300, 1056, 256)])
+def test_mxfp8_tiled_shapes(tile, M, N, K):
+    from kernels.gemm.mxfp4_preshuffle import launch_gemm
+
+    d = make_mx(M, N, K, "fp8", "fp8", seed=8)
+    ref = _ref(d)
+    dev = torch.device("cuda")
+    ops = [d[k].to(dev) for k in ("a_q", "b_shuf", "sa_shuf", "sb_shuf")]
+    for wave_layout in ((0, 8, 2) if tile == (256, 256) else (0,)):
+        c = torch.full((M + 40, N), SENTINEL, dtype=torch.bfloat16, device=dev)
+        launch_gemm(c, *ops, M, N, torch.cuda.current_stream(), N, K, 64, 128, 256, "fp8", "bf16", "fp8", 1, -1, -1, -1, -1, -1, -1, 0, 0,
+                    _force_path=1, _tile=tile, _wave_layout=wave_layout)
+        torch.cuda.synchronize()
+        _check(c[:M].float().cpu().numpy(), ref)
+        assert (c[M:] == SENTINEL).all()
+        # same K order as the general kernel (one MFMA per 128-element step, ascending): the same accumulator bits
+        acc = torch.zeros(M, N, dtype=torch.float32, device=dev)
+        launch_gemm(0, *ops, M, N, torch.cuda.current_stream(), N, K, 64, 128, 256, "fp8", "bf16", "fp8", 1, -1, -1, -1, -1, -1, -1, 0, 0,
+                    _acc=acc, _force_path=1, _tile=tile, _wave_layout=wave_layout)
+        torch.cuda.synchronize()
+        assert np.array_equal(acc.cpu().numpy(), _launch(d, M, N, K, acc=True, force_path=3)), (tile, wave_layout)
+
+
+def test_mxfp8_large_problem_takes_the_tiled_path_and_scale_extremes_hold():
+    from flydsl_amd import layout
+
+    M, N, K = 1024, 8192, 512  # 8 x 32 tiles of 128x256: routed to the tiled mainloop
+    d = make_mx(M, N, K, "fp8", "fp8", seed=12, w_std=1.0)
+    g = torch.Generator().manual_seed(12)
+    d["sa"] = torch.randint(115, 135, d["sa"].shape, generator=g, dtype=torch.uint8)
+    d["sb"] = torch.randint(115, 135, d["sb"].shape, generator=g, dtype=torch.uint8)
+    d["sa_shuf"], d["sb_shuf"] = layout.shuffle_scale_w4(d["sa"], 1, False), layout.shuffle_scale_w4(d["sb"], 1, False)
+    ref = _ref(d)
+    for out_dtype in ("bf16", "fp16"):
+        if out_dtype == "fp16" and np.abs(ref).max() > 6e4:
+            continue
+        c = _launch(d, M, N, K, out_dtype=out_dtype)
+        _check(c.float().cpu().numpy(), ref)
+    assert np.array_equal(_launch(d, M, N, K, acc=True), _launch(d, M, N, K, acc=True, force_path=3))
