@@ -91,8 +91,12 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 // lane into the K loop when forced: MXFP4 4096x7168x2048 82 us).
 // STORE: STORE_ACC dumps raw accumulators; STORE_C writes bf16 with no bias/activation (the common case, kept
 // free of run-time epilogue switches); STORE_C_GENERIC handles fp16 output and the fused bias/activation variants.
-template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4>
-__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && MR * NR <= 32 && !((KIND == KIND_MXFP4 || KIND == KIND_MXFP8) && MR * NR == 32) ? 2 : 1))
+// OCC > 0 overrides that rule: the 128x256 tile of the 8- and 16-bit kinds spills 20-50 bytes per lane when held to two
+// workgroups per CU, which only pays when there are more tiles than CUs (fp8 8192x4096x4096: 127 us against 150 with one
+// workgroup per CU); with at most one tile per CU the unconstrained build is faster (int8 1024x8192x8192: 68 us against
+// 106, fp8 67 against 76), so the launcher picks per problem.
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0>
+__global__ void __launch_bounds__(WAVES * 64, (OCC > 0 ? OCC : (WAVES == 4 && MR * NR <= 32 && !((KIND == KIND_MXFP4 || KIND == KIND_MXFP8) && MR * NR == 32) ? 2 : 1)))
 k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr int WN = WAVES / WM;
@@ -436,14 +440,14 @@ k_a8w8_tiled(A8W8Params p) {
     }
 }
 
-template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4>
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
     constexpr int TM = 16 * MR * WM, TN = 16 * NR * (WAVES / WM);
     const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     A8W8Params q = p;
     q.splits = splits;
-    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE, WAVES>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE, WAVES, OCC>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
     return hipGetLastError();
 }
 
@@ -460,6 +464,13 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
     }
     PSG_CASE(16, 4, 1)
     PSG_CASE(8, 8, 1)
+    if constexpr (KIND != KIND_MXFP4 && KIND != KIND_MXFP8) {
+        // 128x256 with at most one tile per CU: the build that is not held to two workgroups per CU
+        if (tile_m == 128 && tile_n == 256) {
+            const long tiles = (long)((p.M + 127) / 128) * (long)((p.N + 255) / 256) * (STORE == STORE_ACC && p.splits > 1 ? p.splits : 1);
+            if (tiles <= 256) return launch_one<KIND, 8, 4, 1, STORE, 4, 1>(p, stream);
+        }
+    }
     PSG_CASE(8, 4, 1)
     PSG_CASE(4, 4, 1)
     PSG_CASE(2, 4, 1)
