@@ -199,11 +199,14 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
 
 template <int AF, int BF, int STORE>
 hipError_t launch_fmt(const MxGenParams& p, int batch, hipStream_t stream) {
-    // 64x128 tiles (32x128 when M <= 32)
+    // 32x128 tiles for M <= 32, 128x256 when those alone give every CU a workgroup, else 64x128
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     if (p.M <= 32) {
         const int tiles = ((p.M + 31) / 32) * ((p.N + 127) / 128);
         hipLaunchKernelGGL((k_mx_generic<AF, BF, 2, 2, STORE>), dim3(tiles, splits, batch), dim3(256), 0, stream, p);
+    } else if ((long)((p.M + 127) / 128) * (long)((p.N + 255) / 256) * batch >= 256 && splits == 1) {
+        const int tiles = ((p.M + 127) / 128) * ((p.N + 255) / 256);
+        hipLaunchKernelGGL((k_mx_generic<AF, BF, 8, 4, STORE>), dim3(tiles, 1, batch), dim3(256), 0, stream, p);
     } else {
         const int tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
         hipLaunchKernelGGL((k_mx_generic<AF, BF, 4, 2, STORE>), dim3(tiles, splits, batch), dim3(256), 0, stream, p);

@@ -268,3 +268,17 @@ def test_mxfp8_large_problem_takes_the_tiled_path_and_scale_extremes_hold():
         c = _launch(d, M, N, K, out_dtype=out_dtype)
         _check(c.float().cpu().numpy(), ref)
     assert np.array_equal(_launch(d, M, N, K, acc=True), _launch(d, M, N, K, acc=True, force_path=3))
+
+
+@pytest.mark.parametrize("a_dtype,b_dtype", [("fp6", "fp4"), ("fp8", "fp4"), ("fp4", "fp8")])
+def test_general_kernel_large_tile(a_dtype, b_dtype):
+    # enough 128x256 tiles to give every CU one: the general kernel's large tile, ragged in M and N
+    M, N, K = 1000, 8224, 256
+    d = make_mx(M, N, K, a_dtype, b_dtype, seed=14)
+    ref = _ref(d)
+    c = _launch(d, M, N, K, guard_rows=8)
+    _check(c[:M].float().cpu().numpy(), ref)
+    assert (c[M:] == SENTINEL).all()
+    # the small tile through the same kernel (forced by a batch of one narrow problem) gives the same accumulators
+    acc = _launch(d, M, N, K, acc=True)
+    assert np.allclose(acc, ref, rtol=1e-4, atol=_acc_atol(d, ref))
