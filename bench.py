@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the preshuffle quantized GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu] [--next-rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu] [--next-rows] [--reference-shapes]
 
 A step is one GEMM launch on one set of synthetic operands (seed 0; activations N(0,1), weights
 N(0,0.02), quantised and preshuffled on the host, resident in HBM before the timed region).
@@ -325,6 +325,86 @@ def run_next_row_workloads():
     return out
 
 
+def run_reference_test_shapes():
+    """The shapes of the reference's own tests for this path (tests/kernels/test_preshuffle_gemm.py:118-126 for the 8- and
+    16-bit GEMM, :346-353 for MXFP4), through the automatic dispatcher (``--reference-shapes``).  Each shape is recorded
+    20 times into a HIP graph over rotating operand sets; the graph is replayed until 50 ms are timed."""
+    import torch
+
+    from flydsl_amd.synthetic import make_a8w8, make_a16w16, make_mxfp4
+
+    dev = torch.device("cuda:0")
+    out = []
+
+    def graph_time(launch, sets, steps=20):
+        for i in range(3):
+            launch(sets[i % len(sets)])
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(steps):
+                launch(sets[i % len(sets)])
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        replays = max(1, math.ceil(MIN_TIMED_S / max(e0.elapsed_time(e1) * 1e-3, 1e-7)))
+        e0.record()
+        for _ in range(replays):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / (steps * replays)
+
+    def tile(t, rows, unit):  # rows of a host tensor repeated to `rows` (weights of the large shapes are built from a slab)
+        return t.repeat((rows + unit - 1) // unit, *([1] * (t.dim() - 1)))[:rows].contiguous()
+
+    shapes8 = [(16, 5120, 8192), (33, 1024, 2048), (5120, 5120, 8320), (5120, 2048, 8320), (9728, 8192, 8320), (5133, 5120, 8320)]
+    for kind in ("fp8", "int8", "bf16"):
+        for M, N, K in shapes8:
+            mh, nh = min(M, 512), min(N, 512)
+            family = "a16w16" if kind == "bf16" else "a8w8"
+            host = make_a16w16(mh, nh, K, kind, seed=0, w_std=0.02) if kind == "bf16" else make_a8w8(mh, nh, K, kind, seed=0)
+            nbytes = algorithmic_bytes(family, M, N, K)
+            n_sets = max(2, min(16, math.ceil(2 * MALL_BYTES / nbytes)))
+            sets = []
+            for _ in range(n_sets):
+                none = torch.empty(0, dtype=torch.float32, device=dev)
+                s = {"a": tile(host["a_q"], M, mh).to(dev), "b": tile(host["b_shuf"].view(nh, -1), N, nh).to(dev),
+                     "sa": none if kind == "bf16" else tile(host["sa"].view(-1), M, mh).to(dev),
+                     "sb": none if kind == "bf16" else tile(host["sb"].view(-1), N, nh).to(dev),
+                     "c": torch.zeros(M, N, dtype=torch.bfloat16, device=dev)}
+                sets.append(s)
+            sec = graph_time(make_launcher(family, kind, M, N, K), sets)
+            out.append({"workload": f"{kind}_m{M}_n{N}_k{K}", "us_per_launch_events": sec * 1e6, "tflops": 2.0 * M * N * K / sec / 1e12,
+                        "gb_per_s": nbytes / sec / 1e9, "operand_sets": n_sets})
+            del sets
+            torch.cuda.empty_cache()
+    for M, N, K in [(64, 8192, 8192), (32, 8192, 8192), (128, 8192, 8192), (1024, 8192, 8192), (5133, 8192, 8192)]:
+        mh, nh = min(M, 512), 512
+        host = make_mxfp4(mh, nh, K, seed=0)
+        nbytes = algorithmic_bytes("mxfp4", M, N, K)
+        n_sets = max(2, min(16, math.ceil(2 * MALL_BYTES / nbytes)))
+        sets = []
+        for _ in range(n_sets):
+            sets.append({"a": tile(host["a_q"], M, mh).to(dev), "b": tile(host["b_shuf"].view(nh, -1), N, nh).to(dev),
+                         "sa": host["sa_shuf"].view(-1).repeat((M + mh - 1) // mh + 1).contiguous().to(dev),
+                         "sb": host["sb_shuf"].view(-1).repeat(N // nh).contiguous().to(dev),
+                         "c": torch.zeros(M, N, dtype=torch.bfloat16, device=dev)})
+        sec = graph_time(make_launcher("mxfp4", "fp4", M, N, K), sets)
+        out.append({"workload": f"mxfp4_m{M}_n{N}_k{K}", "us_per_launch_events": sec * 1e6, "tflops": 2.0 * M * N * K / sec / 1e12,
+                    "gb_per_s": nbytes / sec / 1e9, "operand_sets": n_sets})
+        del sets
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(name, host, budget_s=12.0):  # budget_s bounds the CPU work of one workload
     """The reference's torch CPU path (dequantise to fp32 + torch.mm) on the same seeded operands,
     timed on this box's host cores.  For workloads whose single pass exceeds the budget a row sample of
@@ -384,6 +464,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--reference-shapes", action="store_true",
+                    help="also time the shapes of the reference's own tests for this path; adds a reference_test_shapes list")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the general MX kernel and the MoE stages (rows next to the hot path); adds a next_rows list")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -439,6 +521,7 @@ def main():
         for name in ("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"):
             others.append(run_quant_workload(name))
     next_rows = run_next_row_workloads() if args.next_rows else None
+    ref_shapes = run_reference_test_shapes() if args.reference_shapes else None
 
     line = {
         "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",
@@ -470,6 +553,8 @@ def main():
     }
     if next_rows is not None:
         line["next_rows"] = next_rows
+    if ref_shapes is not None:
+        line["reference_test_shapes"] = ref_shapes
     # the metric names two operating points; the second one (MFMA-bound prefill) is lifted out of the table for convenience
     for r in others:
         if r["workload"] == "fp8_prefill_m8192":
