@@ -233,7 +233,9 @@ k_a8w8_tiled(A8W8Params p) {
         constexpr int N_LOADS = 2 * NR + (MX ? MP + NP : 0);  // W fragments (+ scale dwords)
         constexpr int B_PER = (N_LOADS + HALF - 1) / HALF;
         // A fragments are read FRAG_AHEAD m-blocks ahead of the MFMAs that use them (register ring buffer)
-        constexpr int FRAG_AHEAD = MR >= 4 ? 2 : 1;
+        // (one block ahead for the int8 128x256 tile held to two workgroups per CU: with two the build spilled 48 bytes per
+        // lane, int8 5120x2048x8320 123 us against 95; the fp8 build of the same tile is the other way round)
+        constexpr int FRAG_AHEAD = (MR >= 4 && !(KIND == KIND_INT8 && WAVES == 4 && MR * NR == 32 && OCC == 0)) ? 2 : 1;
         constexpr int FRAG_BUFS = FRAG_AHEAD + 1;
         v4i flo[FRAG_BUFS], fhi[FRAG_BUFS];
         static_for<FRAG_AHEAD>([&](auto I) {
