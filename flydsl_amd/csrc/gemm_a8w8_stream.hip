@@ -53,16 +53,17 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     const int li = lane & 15;
     const int lg = lane >> 4;
     const int K = IS16 ? (p.K << 1) : p.K;   // BYTES per operand row from here on
-    const int ks = p.ksplit;                 // K slices per workgroup: 1, 2, 4 or 8
-    const int gpw = NWAVES / ks;             // column groups per workgroup
+    const int ks = p.ksplit;                 // K slices per workgroup: 1, 2, 4 or 8 (a power of two: shifts, no divisions,
+    const int ksh = __builtin_ctz(ks);       // which cost tens of instructions each in front of the first load)
+    const int gpw = NWAVES >> ksh;           // column groups per workgroup
     const int tg = p.splits;                 // column groups in the whole launch
     // 8-column units are dealt out evenly: group g starts at unit g*uq + min(g, ur) (the first ur groups hold one more)
     const int uq = p.group_m, ur = p.wave_layout;
     auto unit_begin = [&](int g) { return g * uq + (g < ur ? g : ur); };
-    const int my_ks = wave % ks;
-    const int grp = (int)blockIdx.x * gpw + wave / ks;
+    const int my_ks = wave & (ks - 1);
+    const int grp = (int)blockIdx.x * gpw + (wave >> ksh);
     const int steps = (K + 127) >> 7;
-    const int per = (steps + ks - 1) / ks;
+    const int per = (steps + ks - 1) >> ksh;
     const int s_begin = my_ks * per;
     const int s_end = (s_begin + per) < steps ? (s_begin + per) : steps;
     const int nchunks = s_end > s_begin ? (s_end - s_begin + CH - 1) / CH : 0;
