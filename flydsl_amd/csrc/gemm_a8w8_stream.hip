@@ -61,7 +61,11 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     const int uq = p.group_m, ur = p.wave_layout;
     auto unit_begin = [&](int g) { return g * uq + (g < ur ? g : ur); };
     const int my_ks = wave & (ks - 1);
-    const int grp = (int)blockIdx.x * gpw + (wave >> ksh);
+    // Workgroups go round-robin over the 8 XCDs, so workgroup b of a grid that is a multiple of 8 takes the column groups
+    // of position (b % 8) * grid/8 + b / 8: each XCD then owns one contiguous range of columns and the partial lines of
+    // C that neighbouring workgroups share are merged in one L2 instead of being written back from several.
+    const int bid = (gridDim.x & 7) == 0 ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+    const int grp = bid * gpw + (wave >> ksh);
     const int steps = (K + 127) >> 7;
     const int per = (steps + ks - 1) >> ksh;
     const int s_begin = my_ks * per;
@@ -87,7 +91,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     auto item_coords = [&](int t, int& g, int& frag, int& m, int& n, bool& live) {
         g = (t >> 6) / (NWIN * MB);
         frag = (t >> 6) % (NWIN * MB);
-        const int gq = (int)blockIdx.x * gpw + g;
+        const int gq = bid * gpw + g;
         const int nb = gq < tg ? unit_begin(gq) << 3 : 0;
         const int ne = gq < tg ? unit_begin(gq + 1) << 3 : 0;
         m = (frag % MB) * 16 + li;
