@@ -51,10 +51,14 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
     const int lg = lane >> 4;
     const int KP = p.K >> 1;
     const int KT = p.K >> 8;
-    const int ks = p.ksplit;
+    // four wavefronts are always four K slices: a compile-time constant spares the run-time divisions in front of the loads
+    const int ks = NW == 4 ? 4 : p.ksplit;
     const int npw = NW / ks;  // n-pairs per workgroup
     const int my_ks = wave % ks;
-    const int my_np = (int)blockIdx.x * npw + wave / ks;
+    // workgroups go round-robin over the 8 XCDs: give each XCD one contiguous range of n-pairs, so the 128-byte lines of C
+    // that two neighbouring n-pairs share are completed in one L2
+    const int bid = (gridDim.x & 7) == 0 ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+    const int my_np = bid * npw + wave / ks;
     const int n_pairs = p.N >> 5;
     const int per = (KT + ks - 1) / ks;
     const int s_begin = my_ks * per;
@@ -130,7 +134,7 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
         const int npi = t / (MB * 2 * 64);
         const int f = (t / 64) % (MB * 2);
         const int mb = f >> 1, nb = f & 1;
-        const int np = (int)blockIdx.x * npw + npi;
+        const int np = bid * npw + npi;
         // all partial sums are read in one batch (no wait between them), then added in slice order
         v4f part[NW];
 #pragma unroll
