@@ -4,18 +4,16 @@
 //   MFMA-only rates (fp8 16x16x128, int8 16x16x64, fp4 16x16x128 scaled) on random and on zero operands, with one
 //   and with two wavefronts per SIMD, L2-hit vector load bandwidth per CU, HBM write bandwidth,
 //   a plain read of a decode-sized weight (25.2 MB) rotating through 25 copies and from the Infinity Cache,
-//   and the launch floor of an empty kernel.
+//   the launch floor of an empty kernel, and the small-M streaming GEMM (fp8, M=16, N=6144, K=4096) as the library
+//   launches it, with its parts switched off one at a time (what A, the in-workgroup reduction and the store cost).
 // Build: make -C flydsl_amd/csrc ../psg_ceilings      Run: flydsl_amd/psg_ceilings
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
+#include "gemm_a8w8_stream.hip"  // the library's small-M kernel (and the vector typedefs of psg_common.h)
 typedef float v16f __attribute__((ext_vector_type(16)));
 #define CK(x) do{hipError_t e=(x); if(e!=hipSuccess){printf("HIP error %s at %d\n",hipGetErrorString(e),__LINE__); exit(1);} }while(0)
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v2i __attribute__((ext_vector_type(2)));
-typedef float v4f __attribute__((ext_vector_type(4)));
 
 // ---- LDS read bandwidth: every wavefront of every CU reads its own 8 KB window, 8 independent reads in flight ----
 // PAT 0: lane l reads 16 bytes at l*16 (+1 KB per read): contiguous.  PAT 1: the A-fragment pattern of the tiled
@@ -145,7 +143,20 @@ int main(){
     for(int r=0;r<4;r++){ CK(hipEventRecord(e0,st)); CK(hipGraphLaunch(ge,st)); CK(hipEventRecord(e1,st)); CK(hipEventSynchronize(e1)); float ms; CK(hipEventElapsedTime(&ms,e0,e1)); if(ms<best)best=ms; }
     printf("%-58s %.2f us per launch (graph of %d)  %.0f GB/s\n",name,best*1e3/steps,steps,bbytes/(best*1e-3/steps)/1e9); };
   run("plain read of 25.2 MB, rotating 25 sets, 24 KB per wave", [&](int i){ int nw=bbytes/(24*1024); k_read<24><<<(nw+3)/4,256,0,st>>>(bs[i],nw,dout); });
+  run("plain read of 25.2 MB, rotating 25 sets, 12 KB per wave", [&](int i){ int nw=bbytes/(12*1024); k_read<12><<<(nw+3)/4,256,0,st>>>(bs[i],nw,dout); });
   run("plain read of 25.2 MB, one set (Infinity Cache hot)", [&](int i){ int nw=bbytes/(24*1024); k_read<24><<<(nw+3)/4,256,0,st>>>(bs[0],nw,dout); });
   run("empty kernel, 256 x 512 threads", [&](int i){ k_empty<<<256,512,0,st>>>(); });
+  { // the streaming GEMM of the decode shape, launched like the library does (256 workgroups x 8 wavefronts, 8 K slices,
+    // 768 eight-column units dealt out 3 per workgroup, chunks of 2 K steps); A, scales and C stay fixed, W rotates
+    const int M=16,N=6144,K=4096; uint8_t* a; float *sa,*sb; uint16_t* c;
+    CK(hipMalloc(&a,(size_t)32*K)); CK(hipMemset(a,0x38,(size_t)32*K)); CK(hipMalloc(&sa,4*32)); CK(hipMalloc(&sb,4*N)); CK(hipMemset(sa,0,4*32)); CK(hipMemset(sb,0,4*N)); CK(hipMalloc(&c,(size_t)32*N*2));
+    A8W8Params p{}; p.c=c; p.a=a; p.sa=sa; p.sb=sb; p.M=M; p.N=N; p.K=K; p.epi=EPI_NONE; p.out=OUT_BF16; p.ksplit=8; p.splits=256; p.group_m=(N/8)/256; p.wave_layout=(N/8)%256;
+#define GEMM_DIAG(D,TXT) run(TXT, [&](int i){ A8W8Params q=p; q.b=(const uint8_t*)bs[i]; hipLaunchKernelGGL((k_a8w8_stream<KIND_FP8,1,2,8,2,STORE_C,D>),dim3(256),dim3(512),0,st,q); });
+    GEMM_DIAG(0,"fp8 GEMM M=16 6144x4096, streaming kernel as shipped")
+    GEMM_DIAG(1,"  same, A loads redirected past the bound")
+    GEMM_DIAG(2,"  same, wavefronts end after their MFMAs")
+    GEMM_DIAG(3,"  same, neither A nor reduction / store")
+    GEMM_DIAG(4,"  same, reduction kept, nothing stored")
+  }
   return 0;
 }

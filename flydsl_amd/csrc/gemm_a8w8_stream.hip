@@ -36,7 +36,10 @@ struct Acc<KIND_INT8> {
 
 // MB = 16-row blocks of A (1 or 2); NWIN = 16-column windows per wavefront group (1 or 2).
 // CH = 128-byte K steps per chunk; NWAVES = wavefronts per workgroup.
-template <int KIND, int MB, int NWIN, int NWAVES, int CH, int STORE>
+// DIAG is 0 in the library.  The hardware-ceilings probe instantiates the kernel with parts switched off to price them
+// (results are then wrong on purpose): bit 0 = A loads redirected past the buffer bound, bit 1 = wavefronts end after
+// their MFMAs (no reduction, no store), bit 2 = reduction kept but nothing stored.
+template <int KIND, int MB, int NWIN, int NWAVES, int CH, int STORE, int DIAG = 0>
 __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
@@ -135,7 +138,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
         auto load_chunk = [&](int c, v4i (&at)[PASSES], v4i (&wlo)[NWIN][CH], v4i (&whi)[NWIN][CH]) {
             const int s0 = s_begin + c * CH;
             const uint32_t kbyte = (uint32_t)s0 * 128u + (uint32_t)st_c * 16u;
-            const bool a_ok = c < nchunks && kbyte < slice_end;
+            const bool a_ok = !(DIAG & 1) && c < nchunks && kbyte < slice_end;
 #pragma unroll
             for (int ps = 0; ps < PASSES; ps++) {
                 const int r = st_r0 + ps * RPP;
@@ -208,6 +211,15 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
         fetch_scales();  // wavefronts without work still finish outputs
     }
 
+    if constexpr ((DIAG & 2) != 0) {  // keep the MFMAs alive without a reduction or a store
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWIN; w++)
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) t += (float)acc[w][mb][0] + (float)acc[w][mb][1] + (float)acc[w][mb][2] + (float)acc[w][mb][3];
+        if (t == 12345.678f) reinterpret_cast<float*>(p.c)[0] = t;
+        return;
+    }
     // split-K reduction through LDS, fixed order
 #pragma unroll
     for (int w = 0; w < NWIN; w++)
@@ -242,7 +254,11 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
                     x = (v4f){((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
                               ((float)sum[3] * sa) * sb[3]};
                 }
-                store_c4(p, idx, n, x);
+                if constexpr ((DIAG & 4) != 0) {
+                    if (x[0] == 12345.678f) store_c4(p, idx, n, x);
+                } else {
+                    store_c4(p, idx, n, x);
+                }
             }
         }
     }
