@@ -261,7 +261,7 @@ def run_next_row_workloads():
     import torch
 
     from flydsl_amd import layout, quant
-    from flydsl_amd.kernels.moe.moe_sorting import moe_sorting
+    from flydsl_amd.kernels.moe.moe_sorting import moe_sorting, moe_sorting_flydsl, moe_sorting_get_workspace_size, sorted_sizes
     from flydsl_amd.synthetic import make_mx
     from kernels.gemm.mxfp4_preshuffle import launch_gemm
     from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
@@ -300,7 +300,7 @@ def run_next_row_workloads():
     for tokens, model_dim, inter_dim, experts, topk, tile_m in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 16), (333, 4096, 2048, 17, 9, 64)):
         g = torch.Generator().manual_seed(0)
         vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
-        sid, swt, se, npp = [t.to(dev) for t in moe_sorting(ids.int(), torch.softmax(vals, 1), num_experts=experts, block_size=tile_m)]
+        sid, swt, se, npp = moe_sorting(ids.int().to(dev), torch.softmax(vals, 1).to(dev), num_experts=experts, block_size=tile_m)  # device sorter
         qd = torch.float8_e4m3fn
         xq, sx = quant.pertoken_quant(torch.randn(tokens, model_dim, generator=g), quant_dtype=qd)
         w1q = layout.shuffle_weight((torch.randn(experts * 2 * inter_dim, model_dim, generator=g) / _m.sqrt(model_dim) * 40).to(qd))
@@ -322,6 +322,19 @@ def run_next_row_workloads():
                     "weight_gb_per_s": experts * 2 * inter_dim * model_dim / s1 / 1e9})
         out.append({"workload": f"moe_fp8_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
                     "weight_gb_per_s": experts * model_dim * inter_dim / s2 / 1e9})
+    # the device-side expert sorter in front of the stages (outputs pre-allocated, accumulate buffer cleared by the same launch)
+    for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)):
+        g = torch.Generator().manual_seed(0)
+        vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
+        d_ids, d_w = ids.int().to(dev), torch.softmax(vals, 1).to(dev)
+        rows, blocks = sorted_sizes(tokens, topk, experts, tile_m)
+        bufs = (torch.empty(rows, dtype=torch.int32, device=dev), torch.empty(rows, dtype=torch.float32, device=dev),
+                torch.empty(blocks, dtype=torch.int32, device=dev), torch.empty(2, dtype=torch.int32, device=dev))
+        acc = torch.empty(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(max(4, moe_sorting_get_workspace_size(tokens, experts, topk)), dtype=torch.uint8, device=dev)
+        sec = timed(lambda: moe_sorting_flydsl(d_ids, d_w, *bufs, acc, experts, tile_m, None, None, ws), iters=50)
+        out.append({"workload": f"moe_sorting_tokens{tokens}_e{experts}_top{topk}_block{tile_m}_clear{tokens}x{model_dim}bf16",
+                    "us_per_launch_events": sec * 1e6, "tflops": 0.0, "weight_gb_per_s": 0.0})
     return out
 
 

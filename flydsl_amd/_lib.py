@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -34,6 +34,8 @@ EXPORTS = (
     "psg_debug_tile_order",
     "psg_moe_gemm",
     "psg_moe_reduce",
+    "psg_moe_sorting",
+    "psg_moe_sorting_workspace_bytes",
 )
 
 
@@ -126,6 +128,29 @@ class MoeArgs(ctypes.Structure):
         ("pad0", ctypes.c_int32),
     ]
 
+
+class MoeSortArgs(ctypes.Structure):
+    _fields_ = [
+        ("topk_ids", ctypes.c_void_p),
+        ("topk_weights", ctypes.c_void_p),
+        ("expert_mask", ctypes.c_void_p),
+        ("sorted_ids", ctypes.c_void_p),
+        ("sorted_weights", ctypes.c_void_p),
+        ("sorted_expert_ids", ctypes.c_void_p),
+        ("num_valid_ids", ctypes.c_void_p),
+        ("zero_buf", ctypes.c_void_p),
+        ("zero_bytes", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("tokens", ctypes.c_int32),
+        ("topk", ctypes.c_int32),
+        ("experts", ctypes.c_int32),
+        ("block_m", ctypes.c_int32),
+        ("sorted_size", ctypes.c_int32),
+        ("blocks", ctypes.c_int32),
+    ]
+
+
 _lib = None
 
 
@@ -155,9 +180,11 @@ def lib() -> ctypes.CDLL:
     handle.psg_tile_coords.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
     handle.psg_debug_tile_order.restype = ctypes.c_int
     handle.psg_debug_tile_order.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
+    handle.psg_moe_sorting_workspace_bytes.restype = ctypes.c_uint64
+    handle.psg_moe_sorting_workspace_bytes.argtypes = [ctypes.c_int32] * 3
     handle.psg_moe_reduce.restype = ctypes.c_int
     handle.psg_moe_reduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int32] * 4 + [ctypes.c_void_p]
-    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm"):
+    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm", "psg_moe_sorting"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]

@@ -1,0 +1,288 @@
+// Expert sorting of routed (token, slot) pairs on the device: the step in front of the MoE grouped GEMMs.
+//
+// Output layout (the one the MoE stage kernels read): experts in ascending order, each expert's pairs in row-major
+// (token, slot) order, padded to whole blocks of block_m rows with (topk << 24) | tokens; one expert id per block.
+// No atomics on global memory and a stable order inside every expert, so the output never depends on timing.
+//
+// Small routings (decode): ONE launch, one workgroup per expert.
+//   1. every workgroup builds the whole histogram of expert ids in LDS (4 bytes per routed pair, read from L2), which
+//      gives it its own start row (padded rows of all experts below it), the total and, with an expert mask, its local
+//      expert number;
+//   2. it walks the pairs again in order and compacts those of its expert with wavefront ballots and a prefix over the
+//      wavefronts of the workgroup;
+//   3. it fills its padding rows, its block ids and its share of the unused tails.
+// Large routings (prefill) with a caller workspace: THREE launches, because E workgroups that each count all pairs
+// spend their time in LDS atomics (4096 tokens x top-8 on 32 experts: 109 us in one launch).
+//   1. the pairs are cut into slices; one workgroup per slice writes the slice's histogram to the workspace;
+//   2. one workgroup turns the histograms into per-(slice, expert) offsets, the start row and local number of every
+//      expert, the total, the block ids;
+//   3. one workgroup per (expert, slice) compacts that slice's pairs of that expert straight to their final rows.
+// Either way extra workgroups of the first launch clear the caller's accumulate buffer at full memory bandwidth.
+#include "psg_common.h"
+
+namespace {
+
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_WAVES = SORT_THREADS / 64;
+constexpr int SORT_MAX_EXPERTS = 4096;
+constexpr int SORT_ONESHOT_PAIRS = 4096;   // routings up to this many pairs always take the single launch
+constexpr int SORT_SLICE = 2048;           // pairs per slice of the three-launch path (more when there are > 64 slices)
+constexpr int SORT_MAX_SLICES = 64;
+
+__device__ __forceinline__ int pack_id(int slot, int token) { return (int)(((unsigned)slot << 24) | (unsigned)token); }
+
+// workgroups past the sorting ones clear the caller's buffer, 16 bytes per lane, grid-stride
+__device__ __forceinline__ void clear_share(const MoeSortParams& p, int wg, int wgs) {
+    for (int64_t i = (int64_t)wg * SORT_THREADS + threadIdx.x; i < p.zero_vec; i += (int64_t)wgs * SORT_THREADS)
+        p.zero_buf[i] = (v4i){0, 0, 0, 0};
+}
+
+// rows [total, sorted_size) and blocks [total / block_m, blocks): padding value, weight 0, expert -1; share `wg` of `wgs`
+__device__ __forceinline__ void fill_tails(const MoeSortParams& p, int total, int wg, int wgs) {
+    const int sentinel = pack_id(p.topk, p.tokens);
+    const int tail = p.sorted_size - total, per = (tail + wgs - 1) / wgs;
+    const int lo = total + wg * per, hi = lo + per < p.sorted_size ? lo + per : p.sorted_size;
+    for (int i = lo + (int)threadIdx.x; i < hi; i += SORT_THREADS) {
+        p.sorted_ids[i] = sentinel;
+        p.sorted_weights[i] = 0.f;
+    }
+    const int used = total / p.block_m, btail = p.blocks - used, bper = (btail + wgs - 1) / wgs;
+    const int blo = used + wg * bper, bhi = blo + bper < p.blocks ? blo + bper : p.blocks;
+    for (int i = blo + (int)threadIdx.x; i < bhi; i += SORT_THREADS) p.sorted_expert_ids[i] = -1;
+}
+
+// Stable compaction of the pairs [q_begin, q_end) whose expert is e into rows dst, dst + 1, ...: every wavefront takes a
+// contiguous quarter, counts its matches, and after one barrier writes them behind the wavefronts before it.
+__device__ __forceinline__ void compact_range(const MoeSortParams& p, int e, int q_begin, int q_end, int dst, int (&wcount)[SORT_WAVES]) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int len = q_end - q_begin, per = ((len + SORT_WAVES - 1) / SORT_WAVES + 63) & ~63;
+    const int lo = q_begin + wave * per, hi = lo + per < q_end ? lo + per : q_end;
+    int mine = 0;
+#pragma unroll 4
+    for (int q0 = lo; q0 < hi; q0 += 64) {
+        const int q = q0 + lane;
+        mine += __popcll(__ballot(q < hi && p.topk_ids[q] == e));
+    }
+    if (lane == 0) wcount[wave] = mine;
+    __syncthreads();
+    int row = dst;
+    for (int w = 0; w < wave; w++) row += wcount[w];
+    for (int q0 = lo; q0 < hi; q0 += 64) {
+        const int q = q0 + lane;
+        const bool hit = q < hi && p.topk_ids[q] == e;
+        const unsigned long long ballot = __ballot(hit);
+        if (hit) {
+            const int r = row + __popcll(ballot & ((1ull << lane) - 1ull));
+            const int token = q / p.topk, slot = q - token * p.topk;
+            p.sorted_ids[r] = pack_id(slot, token);
+            p.sorted_weights[r] = p.topk_weights[q];
+        }
+        row += __popcll(ballot);
+    }
+}
+
+__device__ __forceinline__ void fill_padding(const MoeSortParams& p, int start, int cnt, int local) {
+    const int B = p.block_m, padded = (cnt + B - 1) / B * B, sentinel = pack_id(p.topk, p.tokens);
+    for (int i = cnt + (int)threadIdx.x; i < padded; i += SORT_THREADS) {
+        p.sorted_ids[start + i] = sentinel;
+        p.sorted_weights[start + i] = 0.f;
+    }
+    for (int b = threadIdx.x; b < padded / B; b += SORT_THREADS) p.sorted_expert_ids[start / B + b] = local;
+}
+
+// ---- single launch: grid = experts sorting workgroups + clearing workgroups ----
+__global__ void __launch_bounds__(SORT_THREADS) k_moe_sort(MoeSortParams p) {
+    __shared__ int hist[SORT_MAX_EXPERTS];
+    __shared__ int wcount[SORT_WAVES];
+    __shared__ int red[3][SORT_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int e = (int)blockIdx.x;
+    if (e >= p.experts) {
+        clear_share(p, e - p.experts, (int)gridDim.x - p.experts);
+        return;
+    }
+    const int P = p.tokens * p.topk, B = p.block_m;
+    for (int i = tid; i < p.experts; i += SORT_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int q = tid; q < P; q += SORT_THREADS) {
+        const int id = p.topk_ids[q];
+        if ((unsigned)id < (unsigned)p.experts) atomicAdd(&hist[id], 1);  // ids outside [0, experts) are dropped
+    }
+    __syncthreads();
+    // padded rows of the enabled experts below e, of all enabled experts, and the number of enabled experts below e
+    int below = 0, total = 0, local = 0;
+    for (int j = tid; j < p.experts; j += SORT_THREADS) {
+        const bool on = !p.expert_mask || p.expert_mask[j] != 0;
+        const int padded = on ? (hist[j] + B - 1) / B * B : 0;
+        total += padded;
+        if (j < e) {
+            below += padded;
+            local += on ? 1 : 0;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        below += __shfl_xor(below, o);
+        total += __shfl_xor(total, o);
+        local += __shfl_xor(local, o);
+    }
+    if (lane == 0) {
+        red[0][wave] = below;
+        red[1][wave] = total;
+        red[2][wave] = local;
+    }
+    __syncthreads();
+    below = total = local = 0;
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; w++) {
+        below += red[0][w];
+        total += red[1][w];
+        local += red[2][w];
+    }
+    const bool enabled = !p.expert_mask || p.expert_mask[e] != 0;
+    const int cnt = enabled ? hist[e] : 0;
+    if (cnt > 0) compact_range(p, e, 0, P, below, wcount);  // cnt is uniform over the workgroup
+    fill_padding(p, below, cnt, local);
+    fill_tails(p, total, e, p.experts);
+    if (e == 0 && tid == 0) {
+        p.num_valid[0] = total;
+        p.num_valid[1] = p.tokens;
+    }
+}
+
+// ---- three launches.  Workspace (ints): off[(slices + 1) * experts] | start[experts] | local[experts] | total ----
+struct SortPlan {
+    int slices, slice_len;
+};
+
+// launch 1: histogram of one slice -> off[g][*]; clearing workgroups behind the slices
+__global__ void __launch_bounds__(SORT_THREADS) k_moe_sort_count(MoeSortParams p, SortPlan plan, int* ws) {
+    __shared__ int hist[SORT_MAX_EXPERTS];
+    const int tid = threadIdx.x, g = (int)blockIdx.x;
+    if (g >= plan.slices) {
+        clear_share(p, g - plan.slices, (int)gridDim.x - plan.slices);
+        return;
+    }
+    const int P = p.tokens * p.topk;
+    for (int i = tid; i < p.experts; i += SORT_THREADS) hist[i] = 0;
+    __syncthreads();
+    const int lo = g * plan.slice_len, hi = lo + plan.slice_len < P ? lo + plan.slice_len : P;
+    for (int q = lo + tid; q < hi; q += SORT_THREADS) {
+        const int id = p.topk_ids[q];
+        if ((unsigned)id < (unsigned)p.experts) atomicAdd(&hist[id], 1);
+    }
+    __syncthreads();
+    for (int i = tid; i < p.experts; i += SORT_THREADS) ws[g * p.experts + i] = hist[i];
+}
+
+// launch 2 (one workgroup): counts per slice -> running offsets per expert; start row, local number, block ids, total
+__global__ void __launch_bounds__(1024) k_moe_sort_plan(MoeSortParams p, SortPlan plan, int* ws) {
+    __shared__ int padded[SORT_MAX_EXPERTS];
+    __shared__ int on[SORT_MAX_EXPERTS];
+    __shared__ int s_start[SORT_MAX_EXPERTS];
+    __shared__ int s_local[SORT_MAX_EXPERTS];
+    const int tid = threadIdx.x, E = p.experts, B = p.block_m;
+    int* off = ws;
+    int* start = ws + (plan.slices + 1) * E;
+    int* local = start + E;
+    for (int j = tid; j < E; j += 1024) {
+        int acc = 0;
+        for (int g = 0; g < plan.slices; g++) {  // neighbouring threads walk neighbouring columns: coalesced
+            const int c = off[g * E + j];
+            off[g * E + j] = acc;
+            acc += c;
+        }
+        const int enabled = !p.expert_mask || p.expert_mask[j] != 0;
+        off[plan.slices * E + j] = enabled ? acc : 0;  // row `slices` = pairs of the expert that are kept
+        on[j] = enabled;
+        padded[j] = enabled ? (acc + B - 1) / B * B : 0;
+    }
+    __syncthreads();
+    if (tid == 0) {  // E <= 4096 serial steps: a few microseconds, once per routing
+        int row = 0, loc = 0;
+        for (int j = 0; j < E; j++) {
+            s_start[j] = row;
+            s_local[j] = loc;
+            row += padded[j];
+            loc += on[j];
+        }
+        start[2 * E] = row;  // the total, behind start[] and local[]
+        p.num_valid[0] = row;
+        p.num_valid[1] = p.tokens;
+    }
+    __syncthreads();
+    for (int j = tid; j < E; j += 1024) {
+        start[j] = s_start[j];
+        local[j] = s_local[j];
+        for (int b = 0; b < padded[j] / B; b++) p.sorted_expert_ids[s_start[j] / B + b] = s_local[j];
+    }
+}
+
+// launch 3: grid (slices, experts + 1): workgroup (g, e) moves slice g's pairs of expert e; row `experts` fills the tails
+__global__ void __launch_bounds__(SORT_THREADS) k_moe_sort_scatter(MoeSortParams p, SortPlan plan, const int* ws) {
+    __shared__ int wcount[SORT_WAVES];
+    const int g = (int)blockIdx.x, e = (int)blockIdx.y, E = p.experts;
+    const int* off = ws;
+    const int* start = ws + (plan.slices + 1) * E;
+    if (e == E) {
+        fill_tails(p, start[2 * E], g, plan.slices);
+        return;
+    }
+    const int kept = off[plan.slices * E + e];  // 0 for a masked expert
+    if (g == 0) {  // padding rows of the expert
+        const int B = p.block_m, padded = (kept + B - 1) / B * B, sentinel = pack_id(p.topk, p.tokens);
+        for (int i = kept + (int)threadIdx.x; i < padded; i += SORT_THREADS) {
+            p.sorted_ids[start[e] + i] = sentinel;
+            p.sorted_weights[start[e] + i] = 0.f;
+        }
+    }
+    if (kept == 0) return;
+    const int first = off[g * E + e];
+    const int next = g + 1 < plan.slices ? off[(g + 1) * E + e] : kept;
+    if (next == first) return;  // uniform over the workgroup
+    const int P = p.tokens * p.topk;
+    const int lo = g * plan.slice_len, hi = lo + plan.slice_len < P ? lo + plan.slice_len : P;
+    compact_range(p, e, lo, hi, start[e] + first, wcount);
+}
+
+int clear_wgs(const MoeSortParams& p) {
+    if (!p.zero_buf || p.zero_vec <= 0) return 0;
+    const int64_t want = (p.zero_vec * 16 + (128 << 10) - 1) / (128 << 10);  // 128 KB per workgroup, at most 4 per CU
+    return (int)(want < 1 ? 1 : (want > 1024 ? 1024 : want));
+}
+
+SortPlan make_plan(int64_t pairs) {
+    SortPlan plan;
+    int64_t slices = (pairs + SORT_SLICE - 1) / SORT_SLICE;
+    if (slices > SORT_MAX_SLICES) slices = SORT_MAX_SLICES;
+    plan.slices = (int)slices;
+    plan.slice_len = (int)(((pairs + slices - 1) / slices + 63) / 64 * 64);
+    return plan;
+}
+
+}  // namespace
+
+int psg_moe_sort_max_experts() { return SORT_MAX_EXPERTS; }
+
+// bytes of workspace the three-launch path wants for this routing (0: the single launch is used anyway)
+uint64_t psg_moe_sort_workspace(int64_t pairs, int experts) {
+    if (pairs <= SORT_ONESHOT_PAIRS) return 0;
+    const SortPlan plan = make_plan(pairs);
+    return ((uint64_t)(plan.slices + 1) * experts + 2ull * experts + 4) * sizeof(int);
+}
+
+hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream) {
+    const int64_t pairs = (int64_t)p.tokens * p.topk;
+    const uint64_t want = psg_moe_sort_workspace(pairs, p.experts);
+    const int zwgs = clear_wgs(p);
+    if (want == 0 || !workspace || workspace_bytes < want) {
+        hipLaunchKernelGGL(k_moe_sort, dim3(p.experts + zwgs), dim3(SORT_THREADS), 0, stream, p);
+        return hipGetLastError();
+    }
+    const SortPlan plan = make_plan(pairs);
+    int* ws = static_cast<int*>(workspace);
+    hipLaunchKernelGGL(k_moe_sort_count, dim3(plan.slices + zwgs), dim3(SORT_THREADS), 0, stream, p, plan, ws);
+    hipLaunchKernelGGL(k_moe_sort_plan, dim3(1), dim3(1024), 0, stream, p, plan, ws);
+    hipLaunchKernelGGL(k_moe_sort_scatter, dim3(plan.slices, p.experts + 1), dim3(SORT_THREADS), 0, stream, p, plan, (const int*)ws);
+    return hipGetLastError();
+}

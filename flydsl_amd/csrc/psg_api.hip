@@ -13,6 +13,9 @@
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
 hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream);
+hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream);
+uint64_t psg_moe_sort_workspace(int64_t pairs, int experts);
+int psg_moe_sort_max_experts();
 hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, hipStream_t stream);
 hipError_t psg_launch_mx_generic(const MxGenParams& p, int af, int bf, int store, int batch, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
@@ -558,6 +561,50 @@ int psg_moe_reduce(const void* x, void* y, int32_t tokens, int32_t topk, int32_t
     if (!aligned(x, 8) || !aligned(y, 8)) return fail(PSG_E_ALIGN, "x and y must be 8-byte aligned");
     const hipError_t e = psg_launch_moe_reduce(x, y, tokens, topk, model_dim, dtype, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_reduce launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+uint64_t psg_moe_sorting_workspace_bytes(int32_t tokens, int32_t topk, int32_t experts) {
+    if (tokens < 1 || topk < 1 || experts < 1) return 0;
+    return psg_moe_sort_workspace((int64_t)tokens * topk, experts);
+}
+
+int psg_moe_sorting(const psg_moe_sort_args* a, void* stream) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!a->topk_ids || !a->topk_weights || !a->sorted_ids || !a->sorted_weights || !a->sorted_expert_ids || !a->num_valid_ids)
+        return fail(PSG_E_NULL, "topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids must be non-NULL");
+    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
+    if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
+    if (a->experts < 1 || a->experts > psg_moe_sort_max_experts()) return fail(PSG_E_SHAPE, "experts=%d outside [1, %d]", a->experts, psg_moe_sort_max_experts());
+    if (a->block_m < 1 || a->block_m > 4096) return fail(PSG_E_SHAPE, "block_m=%d outside [1, 4096]", a->block_m);
+    const int64_t pairs = (int64_t)a->tokens * a->topk;
+    const int64_t need = pairs + (int64_t)a->experts * a->block_m - a->topk;
+    if (need > 0x7FFFFFFF) return fail(PSG_E_SHAPE, "tokens*topk + experts*block_m must stay below 2^31");
+    if (a->sorted_size < need) return fail(PSG_E_SHAPE, "sorted_size=%d is below tokens*topk + experts*block_m - topk = %lld", a->sorted_size, (long long)need);
+    if ((int64_t)a->blocks * a->block_m < a->sorted_size)
+        return fail(PSG_E_SHAPE, "blocks=%d must cover sorted_size=%d rows in blocks of %d", a->blocks, a->sorted_size, a->block_m);
+    if (a->zero_buf && (a->zero_bytes < 0 || a->zero_bytes % 16 || !aligned(a->zero_buf, 16)))
+        return fail(PSG_E_ALIGN, "zero_buf must be 16-byte aligned and zero_bytes a multiple of 16");
+    MoeSortParams p;
+    p.topk_ids = a->topk_ids;
+    p.topk_weights = a->topk_weights;
+    p.expert_mask = a->expert_mask;
+    p.sorted_ids = a->sorted_ids;
+    p.sorted_weights = a->sorted_weights;
+    p.sorted_expert_ids = a->sorted_expert_ids;
+    p.num_valid = a->num_valid_ids;
+    p.zero_buf = a->zero_bytes > 0 ? static_cast<v4i*>(a->zero_buf) : nullptr;
+    p.zero_vec = a->zero_buf ? a->zero_bytes / 16 : 0;
+    p.tokens = a->tokens;
+    p.topk = a->topk;
+    p.experts = a->experts;
+    p.block_m = a->block_m;
+    p.sorted_size = a->sorted_size;
+    p.blocks = a->blocks;
+    if (a->workspace && !aligned(a->workspace, 4)) return fail(PSG_E_ALIGN, "workspace must be 4-byte aligned");
+    const hipError_t e = psg_launch_moe_sort(p, a->workspace, a->workspace ? a->workspace_bytes : 0, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_sorting launch");
     g_err[0] = 0;
     return 0;
 }

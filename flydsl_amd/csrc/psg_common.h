@@ -165,6 +165,20 @@ struct MoeParams {
     int accumulate;             // stage 2: atomic add into out[token] (else one row per (token, slot))
 };
 
+// Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).
+struct MoeSortParams {
+    const int32_t* topk_ids;     // [tokens, topk]
+    const float* topk_weights;   // [tokens, topk]
+    const int32_t* expert_mask;  // [experts] or nullptr: experts with mask 0 are dropped, the others renumbered densely
+    int32_t* sorted_ids;         // [sorted_size]
+    float* sorted_weights;       // [sorted_size]
+    int32_t* sorted_expert_ids;  // [blocks]
+    int32_t* num_valid;          // [2] = {padded rows in use, tokens}
+    v4i* zero_buf;               // nullptr or a buffer to clear
+    int64_t zero_vec;            // 16-byte vectors of zero_buf
+    int tokens, topk, experts, block_m, sorted_size, blocks;
+};
+
 // bias + activation + 16-bit conversion of four consecutive columns.  The variant is chosen at run time
 // (the epilogue is a vanishing part of any launch, so it is not worth a kernel instantiation per variant).
 template <int OUT, int EPI>

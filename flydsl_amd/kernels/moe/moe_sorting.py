@@ -1,13 +1,86 @@
 """Expert sorting of routed tokens, the layout the MoE stage kernels read.
 
-Same outputs as the reference's torch-native sorter (tests/kernels/test_moe_gemm_2stage.py:99-137, itself a mirror of
-aiter's ``moe_sorting``), computed without a Python loop over experts: one stable sort of the (token, slot) pairs by
-expert, then a scatter into the padded positions.
+Same outputs as the reference's sorters (kernels/moe/moe_sorting_kernel.py:2070-2215 ``moe_sorting_flydsl``; host
+restatements tests/kernels/test_moe_sorting.py:74-110 and tests/kernels/test_moe_gemm_2stage.py:99-137).  Device
+tensors go through the library's sorter kernel (``psg_moe_sorting``: one launch, no host synchronisation, records into
+a graph); host tensors are sorted with torch (one stable sort of the (token, slot) pairs by expert, then a scatter).
 """
 
 from __future__ import annotations
 
+import ctypes
+
 import torch
+
+from ... import _lib
+
+UNIT_SIZE = 32  # default rows per block, as in the reference (moe_sorting_kernel.py:43)
+
+
+def sorted_sizes(tokens: int, topk: int, num_experts: int, block_size: int):
+    """Upper bounds the reference sizes its buffers with: (rows of sorted_ids / sorted_weights, blocks)."""
+    max_padded = int(tokens * topk + num_experts * block_size - topk)
+    return max_padded, (max_padded + block_size - 1) // block_size
+
+
+def moe_sorting_get_workspace_size(M, num_experts, topk, unit_size=UNIT_SIZE):
+    """Bytes of workspace the sorter wants for ``M`` tokens (the reference's helper, moe_sorting_kernel.py:2030); 0 for
+    routings small enough for the single launch."""
+    return int(_lib.lib().psg_moe_sorting_workspace_bytes(int(M), int(topk), int(num_experts)))
+
+
+def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf,
+                       num_experts, unit_size=UNIT_SIZE, expert_mask=None, num_local_tokens=None, workspace=None, *,
+                       stream=None):
+    """The reference's call shape (moe_sorting_kernel.py:2070-2083): every output is pre-allocated by the caller and
+    ``moe_buf`` (the buffer stage 2 accumulates into; may be ``None`` here) is cleared by the same launch.  ``topk_ids``
+    int32 ``[tokens, topk]``, ``topk_weights`` fp32, ``expert_mask`` int32 ``[num_experts]`` or ``None``.  ``workspace``:
+    a device tensor of ``moe_sorting_get_workspace_size(...)`` bytes lets routings of more than 4096 pairs sort in three
+    short launches; ``None`` allocates one when it is needed (pass your own under graph capture or in serving loops),
+    ``False`` forces the single launch.  ``num_local_tokens`` (expert parallelism) is not implemented."""
+    if num_local_tokens is not None:
+        raise NotImplementedError("num_local_tokens (expert-parallel token count) is not implemented")
+    if topk_ids.dim() != 2 or topk_ids.shape != topk_weights.shape:
+        raise ValueError("topk_ids and topk_weights must both be [tokens, topk]")
+    tokens, topk = topk_ids.shape
+    E, B = int(num_experts), int(unit_size)
+    need_rows, _ = sorted_sizes(tokens, topk, E, B)
+    checks = [("topk_ids", topk_ids, torch.int32, tokens * topk), ("topk_weights", topk_weights, torch.float32, tokens * topk),
+              ("sorted_ids", sorted_ids, torch.int32, need_rows), ("sorted_weights", sorted_weights, torch.float32, need_rows),
+              ("sorted_expert_ids", sorted_expert_ids, torch.int32, (need_rows + B - 1) // B), ("num_valid_ids", num_valid_ids, torch.int32, 2)]
+    if expert_mask is not None:
+        checks.append(("expert_mask", expert_mask, torch.int32, E))
+    for name, t, dt, n in checks:
+        if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
+            raise ValueError(f"{name} must be a contiguous {dt} device tensor")
+        if t.numel() < n:
+            raise ValueError(f"{name} holds {t.numel()} elements, this call needs at least {n}")
+    if sorted_weights.numel() < sorted_ids.numel():
+        raise ValueError("sorted_weights must be as long as sorted_ids")
+    args = _lib.MoeSortArgs()
+    args.topk_ids, args.topk_weights = topk_ids.data_ptr(), topk_weights.data_ptr()
+    args.expert_mask = expert_mask.data_ptr() if expert_mask is not None else None
+    args.sorted_ids, args.sorted_weights = sorted_ids.data_ptr(), sorted_weights.data_ptr()
+    args.sorted_expert_ids, args.num_valid_ids = sorted_expert_ids.data_ptr(), num_valid_ids.data_ptr()
+    if moe_buf is not None and moe_buf.numel():
+        if not moe_buf.is_cuda or not moe_buf.is_contiguous():
+            raise ValueError("moe_buf must be a contiguous device tensor")
+        args.zero_buf, args.zero_bytes = moe_buf.data_ptr(), moe_buf.numel() * moe_buf.element_size()
+    want = int(_lib.lib().psg_moe_sorting_workspace_bytes(tokens, topk, E))
+    if workspace is None and want:
+        workspace = torch.empty(want, dtype=torch.uint8, device=topk_ids.device)
+    if workspace is not None and workspace is not False:
+        if not workspace.is_cuda or not workspace.is_contiguous():
+            raise ValueError("workspace must be a contiguous device tensor")
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    args.tokens, args.topk, args.experts, args.block_m = tokens, topk, E, B
+    args.sorted_size = sorted_ids.numel()
+    args.blocks = min(sorted_expert_ids.numel(), (sorted_ids.numel() + B - 1) // B)
+    handle = _lib.lib()
+    rc = handle.psg_moe_sorting(ctypes.byref(args), _lib.stream_handle(stream))
+    if rc != 0:
+        raise (ValueError if rc < 0 else RuntimeError)(handle.psg_last_error().decode())
+    return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf
 
 
 def moe_sorting(topk_ids: torch.Tensor, topk_weights: torch.Tensor, *, num_experts: int, block_size: int):
@@ -27,8 +100,13 @@ def moe_sorting(topk_ids: torch.Tensor, topk_weights: torch.Tensor, *, num_exper
     E, B = int(num_experts), int(block_size)
     if tokens >= 1 << 24:
         raise ValueError("token ids are packed into 24 bits")
-    max_padded = int(tokens * topk + E * B - topk)
-    max_blocks = (max_padded + B - 1) // B
+    max_padded, max_blocks = sorted_sizes(tokens, topk, E, B)
+    if topk_ids.is_cuda:
+        # the library's sorter kernel: no host synchronisation (expert ids outside [0, E) are dropped, not reported)
+        out = (torch.empty(max_padded, dtype=torch.int32, device=device), torch.empty(max_padded, dtype=torch.float32, device=device),
+               torch.empty(max_blocks, dtype=torch.int32, device=device), torch.empty(2, dtype=torch.int32, device=device))
+        moe_sorting_flydsl(topk_ids.to(torch.int32).contiguous(), topk_weights.to(torch.float32).contiguous(), *out, None, E, B)
+        return out
     flat = topk_ids.reshape(-1).to(torch.int64)
     if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= E):
         raise ValueError(f"expert ids must lie in [0, {E})")

@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 4
+#define PSG_ABI_VERSION 5
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
@@ -279,6 +279,45 @@ int psg_moe_gemm(const psg_moe_args *args, void *stream);
  * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203, without its expert mask).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16;
  * model_dim % 4 == 0. */
 int psg_moe_reduce(const void *x, void *y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void *stream);
+
+/*
+ * Expert sorting of the routed (token, slot) pairs on the device: what the reference's moe_sorting_flydsl
+ * (kernels/moe/moe_sorting_kernel.py:2070-2215, the aiter moe_sorting_fwd call shape) produces, in the layout
+ * psg_moe_gemm reads.  Same results as the reference's host restatements (tests/kernels/test_moe_sorting.py:74-110,
+ * tests/kernels/test_moe_gemm_2stage.py:99-137): experts ascending, the pairs of an expert in (token, slot) order,
+ * every expert padded to whole blocks of block_m rows with (topk << 24) | tokens, one expert id per block.
+ *   topk_ids [tokens, topk] int32 (ids outside [0, experts) are dropped), topk_weights [tokens, topk] fp32;
+ *   expert_mask NULL or [experts] int32: experts with 0 are dropped and the others numbered densely (test_moe_sorting.py:88-105);
+ *   sorted_size >= tokens*topk + experts*block_m - topk entries of sorted_ids / sorted_weights, blocks >=
+ *   ceil(sorted_size / block_m) entries of sorted_expert_ids; rows and blocks past the ones in use are written too
+ *   (padding value, weight 0, expert -1); num_valid_ids = {padded rows in use, tokens};
+ *   zero_buf NULL or a 16-byte aligned buffer of zero_bytes (a multiple of 16) that is cleared in the same launch (the
+ *   reference clears moe_buf, the accumulate target of stage 2, in its sorter).
+ *   workspace NULL or psg_moe_sorting_workspace_bytes(tokens, topk, experts) bytes of device memory (4-byte aligned;
+ *   nothing in it has to be initialised): routings of more than 4096 pairs are then sorted by three launches
+ *   (histograms per slice of the pairs, offsets, scatter) instead of one; without it they still sort correctly in one
+ *   launch, several times slower.  The reference's sorter takes a workspace in the same place (moe_sorting_kernel.py:2030).
+ * No atomics on global memory and a stable order: the output does not depend on timing.  experts <= 4096.
+ */
+typedef struct psg_moe_sort_args {
+    const int32_t *topk_ids;
+    const float *topk_weights;
+    const int32_t *expert_mask;
+    int32_t *sorted_ids;
+    float *sorted_weights;
+    int32_t *sorted_expert_ids;
+    int32_t *num_valid_ids;
+    void *zero_buf;
+    int64_t zero_bytes;
+    void *workspace;
+    uint64_t workspace_bytes;
+    int32_t tokens, topk, experts, block_m;
+    int32_t sorted_size;
+    int32_t blocks;
+} psg_moe_sort_args;
+
+uint64_t psg_moe_sorting_workspace_bytes(int32_t tokens, int32_t topk, int32_t experts);
+int psg_moe_sorting(const psg_moe_sort_args *args, void *stream);
 
 #ifdef __cplusplus
 }

@@ -479,13 +479,15 @@ def run_torch_mx(a_q, b_q, scale_a, scale_b, a_fmt: str = "fp4", b_fmt: str = "f
 # ----------------------------------------------------------------------------------------------
 
 
-def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int, block_size: int):
+def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int, block_size: int, expert_mask=None):
     """Expert sorting of routed (token, slot) pairs (tests/kernels/test_moe_gemm_2stage.py:99-137): experts in
     ascending order, each expert's pairs in row-major (token, slot) order and padded to whole blocks with
     ``(topk << 24) | tokens``; one expert id per block, -1 for unused blocks.  Returns ``(sorted_ids int32,
     sorted_weights fp32 (0 in padding rows; the reference leaves them uninitialised), sorted_expert_ids int32,
-    num_tokens_post_pad int32[2])``.  Pinned by invariants (every pair exactly once and inside its expert's blocks,
-    padding values, block count) and a hand-worked example."""
+    num_tokens_post_pad int32[2])``.  With ``expert_mask`` (one flag per expert) the experts whose flag is 0 are
+    dropped and the others numbered densely in ``sorted_expert_ids`` (tests/kernels/test_moe_sorting.py:74-110).
+    Pinned by invariants (every pair exactly once and inside its expert's blocks, padding values, block count) and
+    hand-worked examples, one of them with a mask."""
     ids = np.asarray(topk_ids)
     wts = np.asarray(topk_weights, dtype=np.float32)
     tokens, topk = ids.shape
@@ -494,15 +496,18 @@ def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int
     sorted_ids = np.full(max_padded, (topk << 24) | tokens, dtype=np.int32)
     sorted_w = np.zeros(max_padded, dtype=np.float32)
     sorted_e = np.full(max_blocks, -1, dtype=np.int32)
-    begin = blk = 0
+    begin = blk = skipped = 0
     for e in range(num_experts):
+        if expert_mask is not None and not int(expert_mask[e]):
+            skipped += 1
+            continue
         t, s = np.nonzero(ids == e)
         n = t.size
         nb = (n + block_size - 1) // block_size
         sorted_ids[begin : begin + n] = (s.astype(np.int32) << 24) | t.astype(np.int32)
         sorted_w[begin : begin + n] = wts[t, s]
         begin += nb * block_size
-        sorted_e[blk : blk + nb] = e
+        sorted_e[blk : blk + nb] = e - skipped
         blk += nb
     return sorted_ids, sorted_w, sorted_e, np.array([begin, tokens], dtype=np.int32)
 

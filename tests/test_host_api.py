@@ -357,6 +357,8 @@ def test_struct_layouts_match_header():
                offsetof(psg_mxfp4_args, a_row_stride), offsetof(psg_mxfp4_args, scale_a_batch_stride));
         printf("%zu %zu %zu %zu\n", sizeof(psg_moe_args), offsetof(psg_moe_args, num_valid_ids), offsetof(psg_moe_args, tokens),
                offsetof(psg_moe_args, accumulate));
+        printf("%zu %zu %zu %zu\n", sizeof(psg_moe_sort_args), offsetof(psg_moe_sort_args, workspace_bytes), offsetof(psg_moe_sort_args, tokens),
+               offsetof(psg_moe_sort_args, blocks));
         return 0;
     }'''
     with tempfile.TemporaryDirectory() as d:
@@ -371,6 +373,8 @@ def test_struct_layouts_match_header():
             m.a_dtype.offset, m.batch.offset, m.a_row_stride.offset, m.scale_a_batch_stride.offset]
     e = _lib.MoeArgs
     want += [ctypes.sizeof(e), e.num_valid_ids.offset, e.tokens.offset, e.accumulate.offset]
+    so = _lib.MoeSortArgs
+    want += [ctypes.sizeof(so), so.workspace_bytes.offset, so.tokens.offset, so.blocks.offset]
     assert [int(v) for v in out] == want
 
 

@@ -29,6 +29,21 @@ def test_moe_sorting_hand_worked_example():
     assert len(sid) == 3 * 2 + 3 * 4 - 2
 
 
+def test_moe_sorting_hand_worked_example_with_expert_mask():
+    # same routing, expert 1 switched off: its three pairs vanish, expert 2 becomes local expert 1
+    ids = np.array([[0, 1], [1, 2], [1, 0]], dtype=np.int32)
+    w = np.array([[.6, .4], [.7, .3], [.8, .2]], dtype=np.float32)
+    sid, sw, se, npp = O.moe_sorting(ids, w, 3, 4, expert_mask=np.array([1, 0, 1], dtype=np.int32))
+    pad = (2 << 24) | 3
+    assert sid.tolist() == [0, (1 << 24) | 2, pad, pad, (1 << 24) | 1] + [pad] * 11
+    assert se.tolist() == [0, 1, -1, -1]
+    assert npp.tolist() == [8, 3]
+    assert np.allclose(sw[[0, 1, 4]], [.6, .2, .3]) and (sw[[2, 3, 5, 6, 7]] == 0).all()
+    # an all-ones mask changes nothing
+    for a, b in zip(O.moe_sorting(ids, w, 3, 4, expert_mask=np.ones(3, dtype=np.int32)), O.moe_sorting(ids, w, 3, 4)):
+        assert np.array_equal(a, b)
+
+
 def test_moe_sorting_invariants_and_product_sorter():
     from flydsl_amd.kernels.moe.moe_sorting import moe_sorting
 
