@@ -34,7 +34,7 @@ struct Acc<KIND_INT8> {
     using type = v4i;
 };
 
-// MB = 16-row blocks of A (1 or 2); NWIN = 16-column windows per wavefront group (1 or 2).
+// MB = 16-row blocks of A (1 to 4); NWIN = 16-column windows per wavefront group (1 or 2).
 // CH = 128-byte K steps per chunk; NWAVES = wavefronts per workgroup.
 // DIAG is 0 in the library.  The hardware-ceilings probe instantiates the kernel with parts switched off to price them
 // (results are then wrong on purpose): bit 0 = A loads redirected past the buffer bound, bit 1 = wavefronts end after
@@ -48,7 +48,10 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     constexpr int PASSES = ROWS * CPR / 64;     // staging loads per lane per chunk
     constexpr int RPP = 64 / CPR;               // rows per staging pass
     __shared__ __attribute__((aligned(16))) v4i patch[NWAVES][ROWS * CPR];
-    __shared__ __attribute__((aligned(16))) acc_t red[NWAVES][NWIN * MB][64];
+    // the partial sums of the split-K reduction reuse the wavefront's own patch (it is done with it by then): with 64 rows
+    // patch and a separate array would not fit the LDS together
+    static_assert(ROWS * CPR >= NWIN * MB * 64, "the partial sums of a wavefront must fit its A patch");
+    auto red = [&](int w) { return reinterpret_cast<acc_t*>(patch[w]); };
 
     const int tid = threadIdx.x;
     const int wave = wave_id();
@@ -224,7 +227,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
 #pragma unroll
     for (int w = 0; w < NWIN; w++)
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) red[wave][w * MB + mb][lane] = acc[w][mb];
+        for (int mb = 0; mb < MB; mb++) red(wave)[(w * MB + mb) * 64 + lane] = acc[w][mb];
     __syncthreads();
 
 #pragma unroll
@@ -236,7 +239,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
             // all partial sums are read in one batch (no wait between them), then added in slice order
             acc_t part[NWAVES];
 #pragma unroll
-            for (int j = 0; j < NWAVES; j++) part[j] = red[g * ks + (j < ks ? j : 0)][frag][lane];
+            for (int j = 0; j < NWAVES; j++) part[j] = red(g * ks + (j < ks ? j : 0))[frag * 64 + lane];
             acc_t sum = part[0];
 #pragma unroll
             for (int j = 1; j < NWAVES; j++)
@@ -266,7 +269,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
 
 template <int KIND, int NWAVES, int CH, int STORE>
 hipError_t launch_kind(const A8W8Params& p, int nwin, int grid, hipStream_t stream) {
-    const int mb = p.M <= 16 ? 1 : 2;
+    const int mb = (p.M + 15) / 16;
 #define PSG_GO(MB_, NWIN_)                                                                                                   \
     {                                                                                                                        \
         hipLaunchKernelGGL((k_a8w8_stream<KIND, MB_, NWIN_, NWAVES, CH, STORE>), dim3(grid), dim3(NWAVES * 64), 0, stream, p); \
@@ -275,7 +278,13 @@ hipError_t launch_kind(const A8W8Params& p, int nwin, int grid, hipStream_t stre
     if (mb == 1) {
         if (nwin == 2) PSG_GO(1, 2) else PSG_GO(1, 1)
     }
-    if (nwin == 2) PSG_GO(2, 2) else PSG_GO(2, 1)
+    if (mb == 2) {
+        if (nwin == 2) PSG_GO(2, 2) else PSG_GO(2, 1)
+    }
+    if (mb == 3) {
+        if (nwin == 2) PSG_GO(3, 2) else PSG_GO(3, 1)
+    }
+    if (nwin == 2) PSG_GO(4, 2) else PSG_GO(4, 1)
 #undef PSG_GO
 }
 
@@ -306,7 +315,7 @@ hipError_t launch_planned(const A8W8Params& p0, int kbytes, hipStream_t stream) 
 
 }  // namespace
 
-// Host entry used by the C-ABI layer.  Requires 1 <= M <= 32.  Plans the launch: wavefronts per workgroup by the
+// Host entry used by the C-ABI layer.  Requires 1 <= M <= 64.  Plans the launch: wavefronts per workgroup by the
 // row length, K slices per workgroup so that a slice holds at least two K steps, then column groups dealt out
 // evenly over a multiple of the CU count (at most four 8-column units per group, at least one).
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream) {

@@ -56,6 +56,21 @@ int hip_fail(hipError_t e, const char* what) {
 bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int kSmallM = 32;      // rows the split-K path covers
+constexpr int kStreamMaxM = 64;  // rows the 8- / 16-bit streaming kernel can hold (four 16-row blocks)
+
+// Which regime an 8- / 16-bit problem takes when the caller does not force one.  Up to 32 rows always the streaming
+// kernel.  Above that every workgroup of the streaming kernel still reads all of A (M x K bytes through its texture
+// path), so it only wins while the weight is small enough that the split-K pair of the tiled kernel is bound by its
+// two launches rather than by bandwidth (measured, fp8, us streaming / tiled+split-K: M=33 1024x2048 4.3 / 8.0,
+// 6144x4096 9.2 / 14.1, 8192x8192 15.3 / 19.6, 28672x4096 31.7 / 32.3, 2048x16384 15.5 / 16.0; M=48 9.7 / 14.4,
+// 16.5 / 20.4, 33.0 / 31.3, 17.3 / 16.3; M=64 1024x2048 5.5 / 8.2, 6144x4096 13.9 / 15.0, 8192x8192 21.8 / 21.9, 28672x4096 47 / 32).
+bool takes_stream(int M, int N, int kbytes) {
+    if (M <= kSmallM) return true;
+    if (M > kStreamMaxM) return false;
+    const long w = (long)N * kbytes, a = (long)M * kbytes;
+    if (a > (384L << 10)) return false;
+    return M <= 48 ? w <= (80L << 20) : w <= (32L << 20);
+}
 constexpr int kTargetWaves = 1536;  // wavefronts wanted in flight for the streaming path (6 per CU)
 
 int pick_ksplit(int units, int steps) {
@@ -182,7 +197,7 @@ int validate_a8w8(const psg_a8w8_args* a, bool acc_only, const void* acc) {
     if (a->workspace && !aligned(a->workspace, 16)) return fail(PSG_E_ALIGN, "workspace must be 16-byte aligned");
     if (a->b_layout != 0 && a->b_layout != 1) return fail(PSG_E_DTYPE, "b_layout=%d unknown (0 preshuffled, 1 row-major)", a->b_layout);
     if (a->force_path < 0 || a->force_path > 2) return fail(PSG_E_SHAPE, "force_path=%d unknown", a->force_path);
-    if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    if (a->force_path == 2 && a->M > kStreamMaxM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kStreamMaxM, a->M);
     return 0;
 }
 
@@ -224,7 +239,7 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
     const int kinds[4] = {KIND_INT8, KIND_FP8, KIND_FP16, KIND_BF16};
     const int kind = kinds[a->in_dtype];
     const int kbytes = (kind == KIND_FP16 || kind == KIND_BF16) ? a->K * 2 : a->K;
-    const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
+    const bool small = a->force_path == 2 || (a->force_path == 0 && takes_stream(a->M, a->N, kbytes));
     hipError_t e;
     if (small) {
         e = psg_launch_a8w8_stream(p, kind, store, static_cast<hipStream_t>(stream));
@@ -270,6 +285,7 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) 
     if (M <= kSmallM || M < 1 || N < 16 || K < 64) return 0;
     const bool mx = in_dtype == 4;  // MXFP4 (psg_gemm_mxfp4)
     const int kbytes = mx ? K / 2 : ((in_dtype == PSG_IN_FP16 || in_dtype == PSG_IN_BF16) ? K * 2 : K);
+    if (!mx && takes_stream(M, N, kbytes)) return 0;  // the streaming kernel reduces inside its workgroups
     return splitk_bytes(M, N, plan_tiled(M, N, kbytes, mx).splits);
 }
 
@@ -293,7 +309,7 @@ int psg_gemm_a8w8_static(const psg_a8w8_args* args, void* stream) {
     uint64_t need = psg_workspace_bytes(args->M, args->N, args->K, args->in_dtype);
     if (args->force_path == 1 && args->tile_m > 0 && args->tile_n > 0)
         need = splitk_bytes(args->M, args->N, args->tile_k >= 1 && args->tile_k <= 16 ? args->tile_k : 1);
-    if (args->force_path == 2 || (args->force_path == 0 && args->M <= kSmallM)) need = 0;
+    if (args->force_path == 2) need = 0;  // (psg_workspace_bytes is already 0 for what the streaming kernel takes by itself)
     if (need > PSG_STATIC_SCRATCH_BYTES)
         return fail(PSG_E_WORKSPACE, "this problem's split-K plan needs %llu bytes of scratch, the static scratch holds %u; use "
                     "psg_gemm_a8w8 with a caller workspace", (unsigned long long)need, PSG_STATIC_SCRATCH_BYTES);

@@ -8,7 +8,7 @@ argument.  Underneath there is no JIT: the call fills a plain C struct and enter
 The reference's tuning keywords (``tile_*``, ``waves_per_eu``, ``enable_scheduler``,
 ``use_async_copy``, ``xcd_swizzle``, ``lds_stage``, ``preload``) are validated exactly as the
 reference validates them and then treated as hints: the native dispatcher picks its own tiling per
-regime (MFMA mainloop for M > 32, split-K streaming kernel for M <= 32).
+regime (split-K streaming kernel for M <= 32 and, while the weight is small, up to 64 rows; MFMA mainloop otherwise).
 """
 
 from __future__ import annotations

@@ -100,7 +100,7 @@ typedef struct psg_a8w8_args {
     int32_t epilogue;  /* enum psg_epilogue */
     int32_t tile_m, tile_n, tile_k;
     int32_t xcd_swizzle;
-    int32_t force_path; /* 0 = auto, 1 = tiled MFMA mainloop, 2 = small-M split-K (tests/benchmarks) */
+    int32_t force_path; /* 0 = auto, 1 = tiled MFMA mainloop, 2 = small-M streaming kernel, M <= 64 (tests/benchmarks) */
     int32_t reserved;   /* 0; tuning knob for a forced 256x256 tile: 2 = 2x2 wavefronts, 8 = eight wavefronts 1x8 (default 1x4) */
     int32_t b_layout;   /* 0 = b is preshuffled (above); 1 = b is plain row-major W[N,K], the b_preshuffled=False call
                            shape of the reference's row-scale fp8 GEMMs (kernels/gemm/fp8_gemm_8wave.py:148) */

@@ -65,8 +65,6 @@ def test_gpu_reproduces_a8w8_fixture(name, kind, force_path):
     g = _load(name)
     M, K = g["a_q"].shape
     N = g["b_q"].shape[0]
-    if force_path == 2 and M > 32:
-        pytest.skip("small-M path covers M <= 32")
     dev = torch.device("cuda")
     fn = compile_preshuffle_gemm(N=N, K=K, tile_m=64, tile_n=64, tile_k=64, in_dtype=kind)
     a = torch.from_numpy(g["a_q"]).to(dev)

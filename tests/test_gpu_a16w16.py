@@ -51,7 +51,7 @@ def test_a16w16_shapes(kind, M, N, K):
     d = make_a16w16(M, N, K, kind, seed=M, w_std=0.05)
     ref = _ref(d)
     paths = [(1, t) for t in ((256, 256), (128, 256), (64, 256), (32, 256), (128, 128), (64, 64))]
-    if M <= 32:
+    if M <= 64:
         paths.append((2, None))
     for force_path, tile in paths:
         c = _launch(d, M, N, K, force_path=force_path, tile=tile, guard_rows=40)

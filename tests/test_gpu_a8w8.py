@@ -74,7 +74,7 @@ def test_int8_config1_bit_exact(force_path, tile):
 
 
 @pytest.mark.parametrize("kind", ["int8", "fp8"])
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 47, 48, 49, 64])
 def test_small_m_paths(kind, M):
     N, K = 1024, 2048
     d = make_a8w8(M, N, K, kind, seed=M)
@@ -88,6 +88,22 @@ def test_small_m_paths(kind, M):
             assert np.array_equal(got, O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"])))
             cref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")
             assert np.array_equal(bf16_bits(c[:M]), cref["c_bf16_bits"])
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("M,N,K", [(33, 1040, 1088), (48, 272, 192), (50, 48, 64), (64, 528, 320), (41, 992, 4160), (64, 6144, 4096)])
+def test_streaming_kernel_above_32_rows_ragged(kind, M, N, K):
+    # three and four 16-row blocks, N % 128 != 0, K % 128 == 64, a single K step, the long-row plan (8 wavefronts)
+    d = make_a8w8(M, N, K, kind, seed=M + N)
+    c = _launch(d, M, N, K, force_path=2, guard_rows=24)
+    assert (c[M:] == SENTINEL).all(), "rows past M were written"
+    _check_fp(c[:M].float().cpu().numpy(), O.run_torch(np_bytes(d["a_q"]), np_bytes(d["b_q"]), d["sa"].numpy(), d["sb"].numpy(), kind))
+    if kind == "int8":
+        assert np.array_equal(_acc(d, M, N, K, force_path=2), O.int32_accumulators(np_bytes(d["a_q"]), np_bytes(d["b_q"])))
+        cref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")
+        assert np.array_equal(bf16_bits(c[:M]), cref["c_bf16_bits"])
+        # the automatic plan (streaming or tiled, whichever the planner takes for the shape) gives the same bits
+        assert np.array_equal(bf16_bits(_launch(d, M, N, K)[:M]), cref["c_bf16_bits"])
 
 
 def test_small_m_no_ksplit():
