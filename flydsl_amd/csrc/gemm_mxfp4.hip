@@ -35,7 +35,7 @@ __device__ __forceinline__ void store_mx4(const P& p, int store, size_t idx, v4f
 }
 
 // ------------------------------------------------------------------------------------------------
-// small-M kernel: M <= 32; wavefront = (n-pair of 32 columns, K slice of 256-K steps)
+// small-M kernel: M <= 64; wavefront = (n-pair of 32 columns, K slice of 256-K steps)
 // ------------------------------------------------------------------------------------------------
 constexpr int UNROLL = 2;
 
@@ -72,17 +72,20 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
         __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (uint64_t)my_np * 32ull * (uint64_t)KP, 32ull * (uint64_t)KP);
         __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)p.M * (uint64_t)KP);
         const uint64_t chunk_bytes = (uint64_t)KT * 256ull;
-        __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.sa, chunk_bytes);  // M <= 32: one chunk
+        constexpr int MC = (MB + 1) / 2;  // 32-row chunks of A scales
+        __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.sa, (uint64_t)((p.M + 31) >> 5) * chunk_bytes);
         __amdgpu_buffer_rsrc_t rsb = make_rsrc(p.sb + (uint64_t)my_np * chunk_bytes, chunk_bytes);
         const uint32_t a_voff = (uint32_t)li * (uint32_t)KP + (uint32_t)lg * 16u;
 
         for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
             v4i bq[UNROLL][2][2], aq[UNROLL][MB][2];
-            int sav[UNROLL], sbv[UNROLL];
+            int sav[UNROLL][(MB + 1) / 2], sbv[UNROLL];
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
                 const int s = s0 + u;
-                sav[u] = sbv[u] = 0;
+                sbv[u] = 0;
+#pragma unroll
+                for (int mc = 0; mc < (MB + 1) / 2; mc++) sav[u][mc] = 0;
 #pragma unroll
                 for (int nb = 0; nb < 2; nb++) bq[u][nb][0] = bq[u][nb][1] = (v4i){0, 0, 0, 0};
 #pragma unroll
@@ -100,7 +103,8 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
                         aq[u][mb][0] = buf_load16(ra, voff, (uint32_t)s * TKB);
                         aq[u][mb][1] = buf_load16(ra, voff, (uint32_t)s * TKB + 64u);
                     }
-                    sav[u] = buf_load4(rsa, (uint32_t)lane * 4u, (uint32_t)s * 256u);
+#pragma unroll
+                    for (int mc = 0; mc < MC; mc++) sav[u][mc] = buf_load4(rsa, (uint32_t)mc * (uint32_t)chunk_bytes + (uint32_t)lane * 4u, (uint32_t)s * 256u);
                     sbv[u] = buf_load4(rsb, (uint32_t)lane * 4u, (uint32_t)s * 256u);
                 }
             }
@@ -114,7 +118,7 @@ __global__ void __launch_bounds__(NW * 64) k_mxfp4_smallm(MxParams p) {
                         constexpr int nb = decltype(NB)::value;
                         static_for<MB>([&](auto MBI) {
                             constexpr int mb = decltype(MBI)::value;
-                            acc[mb][nb] = mx_mfma<kh * 2 + nb, kh * 2 + mb>(bq[u][nb][kh], aq[u][mb][kh], acc[mb][nb], sbv[u], sav[u]);
+                            acc[mb][nb] = mx_mfma<kh * 2 + nb, kh * 2 + (mb & 1)>(bq[u][nb][kh], aq[u][mb][kh], acc[mb][nb], sbv[u], sav[u][mb / 2]);
                         });
                     });
                 });
@@ -159,12 +163,14 @@ hipError_t launch_smallm(const MxParams& p, hipStream_t stream) {
 
 }  // namespace
 
-// requires 1 <= M <= 32, nw (wavefronts per workgroup) in {4,8} and p.ksplit a power of two <= nw
+// requires 1 <= M <= 64, nw (wavefronts per workgroup) in {4,8} and p.ksplit a power of two <= nw
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream) {
 #define PSG_GO(MB_)                                                                                             \
     if (nw == 4) return store == STORE_ACC ? launch_smallm<MB_, 4, STORE_ACC>(p, stream) : launch_smallm<MB_, 4, STORE_C>(p, stream); \
     return store == STORE_ACC ? launch_smallm<MB_, 8, STORE_ACC>(p, stream) : launch_smallm<MB_, 8, STORE_C>(p, stream);
     if (p.M <= 16) { PSG_GO(1) }
-    PSG_GO(2)
+    if (p.M <= 32) { PSG_GO(2) }
+    if (p.M <= 48) { PSG_GO(3) }
+    PSG_GO(4)
 #undef PSG_GO
 }

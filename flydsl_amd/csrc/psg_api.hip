@@ -56,7 +56,7 @@ int hip_fail(hipError_t e, const char* what) {
 bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int kSmallM = 32;      // rows the split-K path covers
-constexpr int kStreamMaxM = 64;  // rows the 8- / 16-bit streaming kernel can hold (four 16-row blocks)
+constexpr int kStreamMaxM = 64;  // rows the small-M kernels can hold (four 16-row blocks)
 
 // Which regime an 8- / 16-bit problem takes when the caller does not force one.  Up to 32 rows always the streaming
 // kernel.  Above that every workgroup of the streaming kernel still reads all of A (M x K bytes through its texture
@@ -64,6 +64,14 @@ constexpr int kStreamMaxM = 64;  // rows the 8- / 16-bit streaming kernel can ho
 // two launches rather than by bandwidth (measured, fp8, us streaming / tiled+split-K: M=33 1024x2048 4.3 / 8.0,
 // 6144x4096 9.2 / 14.1, 8192x8192 15.3 / 19.6, 28672x4096 31.7 / 32.3, 2048x16384 15.5 / 16.0; M=48 9.7 / 14.4,
 // 16.5 / 20.4, 33.0 / 31.3, 17.3 / 16.3; M=64 1024x2048 5.5 / 8.2, 6144x4096 13.9 / 15.0, 8192x8192 21.8 / 21.9, 28672x4096 47 / 32).
+// The same question for fp4 x fp4: the small-M kernel up to 32 rows; up to 64 rows while the weight is at most 40 MB and
+// K at least 2048 (measured, us small-M / tiled plan: M=33 7168x2048 4.9 / 6.5, 8192x8192 10.9 / 14.6, 1024x2048 4.3 / 5.3,
+// 4096x1024 4.8 / 4.1, 28672x4096 16.5 / 17.0; M=64 5.9 / 6.7, 13.2 / 15.8, 5.4 / 5.3, 5.8 / 4.2, 22.0 / 17.8).
+bool mx_takes_small(int M, int N, int K) {
+    if (M <= kSmallM) return true;
+    return M <= kStreamMaxM && K >= 2048 && (long)N * (K / 2) <= (40L << 20);
+}
+
 bool takes_stream(int M, int N, int kbytes) {
     if (M <= kSmallM) return true;
     if (M > kStreamMaxM) return false;
@@ -285,7 +293,7 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) 
     if (M <= kSmallM || M < 1 || N < 16 || K < 64) return 0;
     const bool mx = in_dtype == 4;  // MXFP4 (psg_gemm_mxfp4)
     const int kbytes = mx ? K / 2 : ((in_dtype == PSG_IN_FP16 || in_dtype == PSG_IN_BF16) ? K * 2 : K);
-    if (!mx && takes_stream(M, N, kbytes)) return 0;  // the streaming kernel reduces inside its workgroups
+    if (mx ? mx_takes_small(M, N, K) : takes_stream(M, N, kbytes)) return 0;  // the small-M kernels reduce inside their workgroups
     return splitk_bytes(M, N, plan_tiled(M, N, kbytes, mx).splits);
 }
 
@@ -392,7 +400,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     if (a->force_path == 2 && !fp4_fast) return fail(PSG_E_SHAPE, "force_path=2 is for dense, unbatched fp4 x fp4 only");
     if (a->force_path == 1 && !fp4_fast && !fp8_pair)
         return fail(PSG_E_SHAPE, "force_path=1 is for dense, unbatched fp4 x fp4 or fp8 x fp8 only");
-    if (a->force_path == 2 && a->M > kSmallM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kSmallM, a->M);
+    if (a->force_path == 2 && a->M > kStreamMaxM) return fail(PSG_E_SHAPE, "small-M path needs M <= %d, got %d", kStreamMaxM, a->M);
     if (fp8_tiled) {
         const bool forced = a->force_path == 1 && a->tile_m > 0 && a->tile_n > 0;
         const Tile t = forced ? Tile{a->tile_m, a->tile_n, 4} : pick_tile(a->M, a->N, true, 0, 0);
@@ -470,7 +478,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
     p.K = a->K;
     p.out = a->out_dtype;
     p.group_m = a->xcd_swizzle > 0 ? a->xcd_swizzle : 8;
-    const bool small = a->force_path == 2 || (a->force_path == 0 && a->M <= kSmallM);
+    const bool small = a->force_path == 2 || (a->force_path == 0 && mx_takes_small(a->M, a->N, a->K));
     hipError_t e;
     if (small) {
         // four wavefronts x four K slices per workgroup when every slice still holds two 256-K steps, else eight

@@ -46,7 +46,7 @@ def _check(out, ref):
     assert ok, f"outside tolerance (worst ratio {ratio:.3f})"
 
 
-@pytest.mark.parametrize("M", [1, 16, 31, 32])
+@pytest.mark.parametrize("M", [1, 16, 31, 32, 33, 47, 48, 49, 64])
 @pytest.mark.parametrize("N,K", [(256, 512), (7168, 2048)])
 def test_mxfp4_small_m(M, N, K):
     d = make_mxfp4(M, N, K, seed=M)
