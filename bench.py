@@ -487,7 +487,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
-              "the GEMM shards over N with no exchange, see DESIGN.md", file=sys.stderr)
+              "the GEMM would shard over N (disjoint column panels of C, no exchange between GPUs)", file=sys.stderr)
         sys.exit(2)
 
     import torch
