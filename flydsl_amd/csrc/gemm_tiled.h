@@ -95,7 +95,11 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 // workgroups per CU, which only pays when there are more tiles than CUs (fp8 8192x4096x4096: 127 us against 150 with one
 // workgroup per CU); with at most one tile per CU the unconstrained build is faster (int8 1024x8192x8192: 68 us against
 // 106, fp8 67 against 76), so the launcher picks per problem.
-template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0>
+// PFW = K steps the W fragments are fetched ahead of their MFMAs (PFW + 1 register sets).  1 for problems that fill the GPU
+// (the MFMAs of a step hide one memory latency).  3 for the few-tile / split-K regime, where a workgroup's MFMAs take no time
+// and the launch is bound by the bytes of W in flight: one 128x128 tile per CU with one step ahead keeps 16 KB per CU on
+// its way, far from what HBM needs (fp8 M=128, N=K=8192: 27 us for a 67 MB weight).
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0, int PFW = 1>
 __global__ void __launch_bounds__(WAVES * 64, (OCC > 0 ? OCC : (WAVES == 4 && MR * NR <= 32 && !((KIND == KIND_MXFP4 || KIND == KIND_MXFP8) && MR * NR == 32) ? 2 : 1)))
 k_a8w8_tiled(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
@@ -172,9 +176,15 @@ k_a8w8_tiled(A8W8Params p) {
         for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (acc_t){0, 0, 0, 0};
 
     // Register sets: areg holds the A tile of the next K step on its way to LDS (each register is written to
-    // LDS and immediately reloaded for the step after); blo/bhi[q] hold the W fragments of a step with parity q.
-    v4i areg[A_LOADS];
-    v4i blo[2][NR], bhi[2][NR];
+    // LDS and immediately reloaded for the step after); blo/bhi[q] hold the W fragments of the steps with kt % NB == q.
+    constexpr int NB = PFW + 1;
+    static_assert(NB == 2 || (NB == 4 && !MX), "W register sets: 2, or 4 for the kinds without MX scale dwords");
+    // With four W sets the A tile is fetched just as far ahead (loads return in order: a wait for A of the next step would
+    // otherwise also wait for every W fragment requested before it): four A register sets, A(j) in set j % 4, loaded five
+    // steps before its MFMAs and written to LDS one step before them.
+    constexpr int NA = NB == 4 ? 4 : 1;
+    v4i areg[NA][A_LOADS];
+    v4i blo[NB][NR], bhi[NB][NR];
 
     // Loads never sit under control flow: a K step past the end (prefetch of the last iterations) and an A
     // chunk past K (only when K % 128 == 64) are redirected past the descriptor bound, where the hardware
@@ -228,7 +238,9 @@ k_a8w8_tiled(A8W8Params p) {
     //                                each register reloaded at once with its part of the A tile of step kt+2
     //   every m-block              : LDS read of the next m-block's A fragment (register double buffer)
     auto step = [&](int kt, auto SP) {
-        constexpr int S = decltype(SP)::value;
+        constexpr int SB = decltype(SP)::value;  // W register set of this step
+        constexpr int S = SB & 1;                // LDS stage (and MX scale set) of this step
+        constexpr int SN = (SB + PFW) % NB;      // W register set the loads of this step fill
         constexpr int HALF = MR / 2;
         constexpr int N_LOADS = 2 * NR + (MX ? MP + NP : 0);  // W fragments (+ scale dwords)
         constexpr int B_PER = (N_LOADS + HALF - 1) / HALF;
@@ -249,7 +261,7 @@ k_a8w8_tiled(A8W8Params p) {
             if constexpr (mi < HALF) {
                 static_for<B_PER>([&](auto Q) {
                     constexpr int idx = mi * B_PER + decltype(Q)::value;
-                    if constexpr (idx < 2 * NR) load_b1(kt + 1, idx, blo[S ^ 1], bhi[S ^ 1]);
+                    if constexpr (idx < 2 * NR) load_b1(kt + PFW, idx, blo[SN], bhi[SN]);
                     else if constexpr (idx < N_LOADS) load_sc1(kt + 1, idx - 2 * NR, sav[S ^ 1], sbv[S ^ 1]);
                 });
             } else {
@@ -257,8 +269,9 @@ k_a8w8_tiled(A8W8Params p) {
                 static_for<A_PER>([&](auto Q) {
                     constexpr int j = (mi - HALF) * A_PER + decltype(Q)::value;
                     if constexpr (j < A_LOADS) {
-                        store_a1(S ^ 1, j, areg[j]);
-                        load_a1(kt + 2, j, areg[j]);
+                        constexpr int AS = NA == 4 ? (SB + 1) % 4 : 0;  // set of A(kt + 1)
+                        store_a1(S ^ 1, j, areg[AS][j]);
+                        load_a1(kt + (NA == 4 ? 5 : 2), j, areg[AS][j]);
                     }
                 });
             }
@@ -268,42 +281,42 @@ k_a8w8_tiled(A8W8Params p) {
             const v4i alo = flo[mi % FRAG_BUFS], ahi = fhi[mi % FRAG_BUFS];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
-                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[S][ni], alo);
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[SB][ni], alo);
 #pragma unroll
-                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[S][ni], ahi);
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[SB][ni], ahi);
             } else if constexpr (IS16) {
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
-                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], blo[S][ni], alo); else mfma_f16(acc[mi][ni], blo[S][ni], alo);
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], blo[SB][ni], alo); else mfma_f16(acc[mi][ni], blo[SB][ni], alo);
                 }
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
-                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], bhi[S][ni], ahi); else mfma_f16(acc[mi][ni], bhi[S][ni], ahi);
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], bhi[SB][ni], ahi); else mfma_f16(acc[mi][ni], bhi[SB][ni], ahi);
                 }
             } else if constexpr (KIND == KIND_MXFP4) {
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
-                    mfma_mx<0, ni & 1, mi & 1>(acc[mi][ni], blo[S][ni], alo, sbv[S][ni / 2], sav[S][mi / 2]);
+                    mfma_mx<0, ni & 1, mi & 1>(acc[mi][ni], blo[SB][ni], alo, sbv[S][ni / 2], sav[S][mi / 2]);
                 });
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
-                    mfma_mx<1, ni & 1, mi & 1>(acc[mi][ni], bhi[S][ni], ahi, sbv[S][ni / 2], sav[S][mi / 2]);
+                    mfma_mx<1, ni & 1, mi & 1>(acc[mi][ni], bhi[SB][ni], ahi, sbv[S][ni / 2], sav[S][mi / 2]);
                 });
             } else if constexpr (KIND == KIND_MXFP8) {
                 // step parity S = 128-element half of the scale chunk: K ranges start at even steps (no split-K here)
                 const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
-                    const v8i bf = {blo[S][ni][0], blo[S][ni][1], blo[S][ni][2], blo[S][ni][3],
-                                    bhi[S][ni][0], bhi[S][ni][1], bhi[S][ni][2], bhi[S][ni][3]};
+                    const v8i bf = {blo[SB][ni][0], blo[SB][ni][1], blo[SB][ni][2], blo[SB][ni][3],
+                                    bhi[SB][ni][0], bhi[SB][ni][1], bhi[SB][ni][2], bhi[SB][ni][3]};
                     mfma_mx8<S, ni & 1, mi & 1>(acc[mi][ni], bf, af, sbv[S][ni / 2], sav[S][mi / 2]);
                 });
             } else {
                 const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
-                    const v8i bf = {blo[S][ni][0], blo[S][ni][1], blo[S][ni][2], blo[S][ni][3],
-                                    bhi[S][ni][0], bhi[S][ni][1], bhi[S][ni][2], bhi[S][ni][3]};
+                    const v8i bf = {blo[SB][ni][0], blo[SB][ni][1], blo[SB][ni][2], blo[SB][ni][3],
+                                    bhi[SB][ni][0], bhi[SB][ni][1], bhi[SB][ni][2], bhi[SB][ni][3]};
                     mfma_f8(acc[mi][ni], bf, af);
                 }
             }
@@ -321,26 +334,48 @@ k_a8w8_tiled(A8W8Params p) {
 
     // prologue: A(0) -> LDS stage 0, A(1) -> registers, W(0) -> set 0
 #pragma unroll
-    for (int j = 0; j < A_LOADS; j++) load_a1(kt_begin, j, areg[j]);
+    for (int j = 0; j < A_LOADS; j++) load_a1(kt_begin, j, areg[0][j]);
+    static_for<PFW>([&](auto I) {
+        constexpr int i = decltype(I)::value;
 #pragma unroll
-    for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin, idx, blo[0], bhi[0]);
+        for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin + i, idx, blo[i], bhi[i]);
+        if constexpr (NA == 4) {
+#pragma unroll
+            for (int j = 0; j < A_LOADS; j++) load_a1(kt_begin + 1 + i, j, areg[1 + i][j]);
+        }
+    });
     if constexpr (MX) {
 #pragma unroll
         for (int q = 0; q < MP + NP; q++) load_sc1(kt_begin, q, sav[0], sbv[0]);
     }
 #pragma unroll
     for (int j = 0; j < A_LOADS; j++) {
-        store_a1(0, j, areg[j]);
-        load_a1(kt_begin + 1, j, areg[j]);
+        store_a1(0, j, areg[0][j]);
+        if constexpr (NA == 4) {
+            load_a1(kt_begin + 4, j, areg[0][j]);
+        } else {
+            load_a1(kt_begin + 1, j, areg[0][j]);
+        }
     }
     __syncthreads();
 
     // Two K steps per iteration (LDS / register ping-pong).  When the step count is odd the last "odd" step
     // multiplies zero operands (its loads were redirected past the bounds): harmless, and the loop body stays
     // free of control flow, which the software pipeline needs.
-    for (int kt = kt_begin; kt < kt_end; kt += 2) {
-        step(kt, std::integral_constant<int, 0>{});
-        step(kt + 1, std::integral_constant<int, 1>{});
+    if constexpr (NB == 2) {
+        for (int kt = kt_begin; kt < kt_end; kt += 2) {
+            step(kt, std::integral_constant<int, 0>{});
+            step(kt + 1, std::integral_constant<int, 1>{});
+        }
+    } else {
+        // four register sets: steps past the end are skipped (the condition is uniform over the workgroup) instead of run on
+        // zero operands; with 16 steps per workgroup three idle steps would be a fifth of the loop
+        for (int kt = kt_begin; kt < kt_end; kt += 4) {
+            step(kt, std::integral_constant<int, 0>{});
+            if (kt + 1 < kt_end) step(kt + 1, std::integral_constant<int, 1>{});
+            if (kt + 2 < kt_end) step(kt + 2, std::integral_constant<int, 2>{});
+            if (kt + 3 < kt_end) step(kt + 3, std::integral_constant<int, 3>{});
+        }
     }
 
     // epilogue operands, fetched in one batch (one memory latency for the whole tile, not one per fragment)
@@ -442,14 +477,14 @@ k_a8w8_tiled(A8W8Params p) {
     }
 }
 
-template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0>
+template <int KIND, int MR, int NR, int WM, int STORE, int WAVES = 4, int OCC = 0, int PFW = 1>
 hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
     constexpr int TM = 16 * MR * WM, TN = 16 * NR * (WAVES / WM);
     const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     A8W8Params q = p;
     q.splits = splits;
-    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE, WAVES, OCC>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
+    hipLaunchKernelGGL((k_a8w8_tiled<KIND, MR, NR, WM, STORE, WAVES, OCC, PFW>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
     return hipGetLastError();
 }
 
@@ -463,6 +498,13 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
     }
     if (p.wave_layout == 8) {  // eight wavefronts side by side along N: 256x256 tile, every W fragment loaded once
         if (tile_m == 256 && tile_n == 256) return launch_one<KIND, 16, 2, 1, STORE, 8>(p, stream);
+    }
+    if constexpr (KIND != KIND_MXFP4 && KIND != KIND_MXFP8) {
+        // few tiles (p.ksplit = 3: the planner's mark for launches of at most two workgroups per CU): W fetched three steps ahead
+        if (p.ksplit == 3) {
+            if (tile_m == 128 && tile_n == 128) return launch_one<KIND, 8, 2, 1, STORE, 4, 1, 3>(p, stream);
+            if (tile_m == 64 && tile_n == 64) return launch_one<KIND, 4, 1, 1, STORE, 4, 0, 3>(p, stream);
+        }
     }
     PSG_CASE(16, 4, 1)
     PSG_CASE(8, 8, 1)

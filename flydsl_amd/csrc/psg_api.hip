@@ -140,9 +140,13 @@ int pick_splits(int M, int N, int kbytes, Tile t) {
     const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
     const int steps = (kbytes + 127) / 128;
     if (tiles >= 192 || steps < 32) return 1;
-    // measured optimum: about 16 K steps per workgroup, at most ~1024 workgroups, partial traffic bounded
+    // measured optimum: about 16 K steps per workgroup, at most ~1024 workgroups, partial traffic bounded: a quarter of W
+    // once every CU has a workgroup; while CUs would stay idle the bound is five times looser, because an idle CU costs more
+    // than the partial sums (fp8 512x4096x14336, 128 tiles: 71 us unsplit, 49 us with two splits; 256x4096x14336: 45 -> 32 us)
     int s = 1;
-    while (s < 8 && steps / (s * 2) >= 16 && tiles * (s * 2) <= 1024 && (long)(s * 2) * M * 16 <= kbytes) s *= 2;
+    while (s < 8 && steps / (s * 2) >= 16 && tiles * (s * 2) <= 1024 &&
+           (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s < 256 ? 5 : 1))
+        s *= 2;
     return s;
 }
 
@@ -262,6 +266,11 @@ int run_a8w8(const psg_a8w8_args* a, void* out, int store, void* stream) {
         int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
         if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
         p.splits = splits;
+        // at most two workgroups per CU: the launch is bound by the bytes of W in flight, so the builds that fetch W three
+        // steps ahead run (ksplit doubles as that mark for the tiled kernel); reserved = 7 keeps the one-step builds (tests)
+        const long wgs = (long)((a->M + t.m - 1) / t.m) * (long)((a->N + t.n - 1) / t.n) * splits;
+        const int steps_per_wg = ((kbytes + 127) / 128 + splits - 1) / splits;
+        if (wgs <= 512 && steps_per_wg >= 6 && a->reserved != 7) p.ksplit = 3;
         if (splits > 1) {
             A8W8Params part = p;
             part.c = a->workspace;
