@@ -162,43 +162,65 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
         };
         // A through the private patch into fragment order, then the chunk's MFMAs as W arrives
         auto compute_chunk = [&](const v4i (&at)[PASSES], const v4i (&wlo)[NWIN][CH], const v4i (&whi)[NWIN][CH]) {
-            v4i alo[CH][MB], ahi[CH][MB];
 #pragma unroll
             for (int ps = 0; ps < PASSES; ps++) {
                 const int r = st_r0 + ps * RPP;
                 my_patch[r * CPR + (st_c ^ (r & 15))] = at[ps];
             }
-#pragma unroll
-            for (int t = 0; t < CH; t++)
+            // one K step's MFMAs on fragments alo / ahi (per 16-row block) and W registers wlo / whi (per window) of step t
+            auto mfma_step = [&](int t, const v4i (&alo_t)[MB], const v4i (&ahi_t)[MB], int w) {
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++) {
-                    const int r = mb * 16 + li;
-                    alo[t][mb] = my_patch[r * CPR + ((t * 8 + lg) ^ (r & 15))];
-                    ahi[t][mb] = my_patch[r * CPR + ((t * 8 + 4 + lg) ^ (r & 15))];
+                    if constexpr (KIND == KIND_INT8) {
+                        acc[w][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo[w][t], alo_t[mb], acc[w][mb], 0, 0, 0);
+                        acc[w][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi[w][t], ahi_t[mb], acc[w][mb], 0, 0, 0);
+                    } else if constexpr (KIND == KIND_BF16) {
+                        acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wlo[w][t]), __builtin_bit_cast(v8bf, alo_t[mb]), acc[w][mb], 0, 0, 0);
+                        acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, whi[w][t]), __builtin_bit_cast(v8bf, ahi_t[mb]), acc[w][mb], 0, 0, 0);
+                    } else if constexpr (KIND == KIND_FP16) {
+                        acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wlo[w][t]), __builtin_bit_cast(v8h, alo_t[mb]), acc[w][mb], 0, 0, 0);
+                        acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, whi[w][t]), __builtin_bit_cast(v8h, ahi_t[mb]), acc[w][mb], 0, 0, 0);
+                    } else {
+                        const v8i bf = {wlo[w][t][0], wlo[w][t][1], wlo[w][t][2], wlo[w][t][3],
+                                        whi[w][t][0], whi[w][t][1], whi[w][t][2], whi[w][t][3]};
+                        const v8i af = {alo_t[mb][0], alo_t[mb][1], alo_t[mb][2], alo_t[mb][3],
+                                        ahi_t[mb][0], ahi_t[mb][1], ahi_t[mb][2], ahi_t[mb][3]};
+                        acc[w][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[w][mb], 0, 0, 0, 0, 0, 0);
+                    }
                 }
-#pragma unroll
-            for (int w = 0; w < NWIN; w++)
+            };
+            if constexpr (MB <= 2) {
+                // all fragments of the chunk are read first, then window by window
+                v4i alo[CH][MB], ahi[CH][MB];
 #pragma unroll
                 for (int t = 0; t < CH; t++)
 #pragma unroll
                     for (int mb = 0; mb < MB; mb++) {
-                        if constexpr (KIND == KIND_INT8) {
-                            acc[w][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo[w][t], alo[t][mb], acc[w][mb], 0, 0, 0);
-                            acc[w][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi[w][t], ahi[t][mb], acc[w][mb], 0, 0, 0);
-                        } else if constexpr (KIND == KIND_BF16) {
-                            acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wlo[w][t]), __builtin_bit_cast(v8bf, alo[t][mb]), acc[w][mb], 0, 0, 0);
-                            acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, whi[w][t]), __builtin_bit_cast(v8bf, ahi[t][mb]), acc[w][mb], 0, 0, 0);
-                        } else if constexpr (KIND == KIND_FP16) {
-                            acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wlo[w][t]), __builtin_bit_cast(v8h, alo[t][mb]), acc[w][mb], 0, 0, 0);
-                            acc[w][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, whi[w][t]), __builtin_bit_cast(v8h, ahi[t][mb]), acc[w][mb], 0, 0, 0);
-                        } else {
-                            const v8i bf = {wlo[w][t][0], wlo[w][t][1], wlo[w][t][2], wlo[w][t][3],
-                                            whi[w][t][0], whi[w][t][1], whi[w][t][2], whi[w][t][3]};
-                            const v8i af = {alo[t][mb][0], alo[t][mb][1], alo[t][mb][2], alo[t][mb][3],
-                                            ahi[t][mb][0], ahi[t][mb][1], ahi[t][mb][2], ahi[t][mb][3]};
-                            acc[w][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[w][mb], 0, 0, 0, 0, 0, 0);
-                        }
+                        const int r = mb * 16 + li;
+                        alo[t][mb] = my_patch[r * CPR + ((t * 8 + lg) ^ (r & 15))];
+                        ahi[t][mb] = my_patch[r * CPR + ((t * 8 + 4 + lg) ^ (r & 15))];
                     }
+#pragma unroll
+                for (int w = 0; w < NWIN; w++)
+#pragma unroll
+                    for (int t = 0; t < CH; t++) mfma_step(t, alo[t], ahi[t], w);
+            } else {
+                // three and four 16-row blocks: step by step, so that only one step's fragments are live (the order of the
+                // additions into every accumulator is the same; all fragments at once spilled registers at 64 rows)
+#pragma unroll
+                for (int t = 0; t < CH; t++) {
+                    v4i alo[MB], ahi[MB];
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++) {
+                        const int r = mb * 16 + li;
+                        alo[mb] = my_patch[r * CPR + ((t * 8 + lg) ^ (r & 15))];
+                        ahi[mb] = my_patch[r * CPR + ((t * 8 + 4 + lg) ^ (r & 15))];
+                    }
+#pragma unroll
+                    for (int w = 0; w < NWIN; w++) mfma_step(t, alo, ahi, w);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         };
 
         v4i at[PASSES];

@@ -58,26 +58,26 @@ bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p
 constexpr int kSmallM = 32;      // rows the split-K path covers
 constexpr int kStreamMaxM = 64;  // rows the small-M kernels can hold (four 16-row blocks)
 
-// Which regime an 8- / 16-bit problem takes when the caller does not force one.  Up to 32 rows always the streaming
-// kernel.  Above that every workgroup of the streaming kernel still reads all of A (M x K bytes through its texture
-// path), so it only wins while the weight is small enough that the split-K pair of the tiled kernel is bound by its
-// two launches rather than by bandwidth (measured, fp8, us streaming / tiled+split-K: M=33 1024x2048 4.3 / 8.0,
-// 6144x4096 9.2 / 14.1, 8192x8192 15.3 / 19.6, 28672x4096 31.7 / 32.3, 2048x16384 15.5 / 16.0; M=48 9.7 / 14.4,
-// 16.5 / 20.4, 33.0 / 31.3, 17.3 / 16.3; M=64 1024x2048 5.5 / 8.2, 6144x4096 13.9 / 15.0, 8192x8192 21.8 / 21.9, 28672x4096 47 / 32).
-// The same question for fp4 x fp4: the small-M kernel up to 32 rows; up to 64 rows while the weight is at most 40 MB and
-// K at least 2048 (measured, us small-M / tiled plan: M=33 7168x2048 4.9 / 6.5, 8192x8192 10.9 / 14.6, 1024x2048 4.3 / 5.3,
+// Which regime an fp4 x fp4 problem takes: the small-M kernel up to 32 rows; up to 64 rows while the weight is at most 40 MB
+// and K at least 2048 (measured, us small-M / tiled plan: M=33 7168x2048 4.9 / 6.5, 8192x8192 10.9 / 14.6, 1024x2048 4.3 / 5.3,
 // 4096x1024 4.8 / 4.1, 28672x4096 16.5 / 17.0; M=64 5.9 / 6.7, 13.2 / 15.8, 5.4 / 5.3, 5.8 / 4.2, 22.0 / 17.8).
 bool mx_takes_small(int M, int N, int K) {
     if (M <= kSmallM) return true;
     return M <= kStreamMaxM && K >= 2048 && (long)N * (K / 2) <= (40L << 20);
 }
 
+// Which regime an 8- / 16-bit problem takes when the caller does not force one.  Up to 32 rows always the streaming
+// kernel.  Above that every workgroup of the streaming kernel still reads all of A (M x K bytes through its texture
+// path), so it only wins while the weight is small enough that the split-K pair of the tiled kernel is bound by its
+// two launches and its partial sums rather than by bandwidth (measured, fp8, us streaming / tiled+split-K: M=33 1024x2048
+// 4.3 / 8.0, 6144x4096 9.2 / 14.1, 8192x8192 15.3 / 19.6, 28672x4096 31.7 / 32.3, 2048x16384 15.5 / 16.0; M=48 9.7 / 14.4,
+// 16.5 / 20.4, 33.0 / 31.3, 17.3 / 16.3; M=64 1024x2048 5.5 / 8.2, 6144x4096 11.3 / 15.0, 8192x8192 18.3 / 22.2,
+// 5120x8192 15.8 / 19.0, 28672x4096 37.5 / 32.7, 2048x16384 20.0 / 15.6).
 bool takes_stream(int M, int N, int kbytes) {
     if (M <= kSmallM) return true;
     if (M > kStreamMaxM) return false;
     const long w = (long)N * kbytes, a = (long)M * kbytes;
-    if (a > (384L << 10)) return false;
-    return M <= 48 ? w <= (80L << 20) : w <= (32L << 20);
+    return a <= (512L << 10) && w <= (80L << 20);
 }
 constexpr int kTargetWaves = 1536;  // wavefronts wanted in flight for the streaming path (6 per CU)
 

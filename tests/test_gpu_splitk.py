@@ -70,7 +70,7 @@ def test_float_splitk(kind, epilogue):
 def test_automatic_plan_uses_and_survives_without_workspace():
     from flydsl_amd import _lib
 
-    M, N, K = 64, 2048, 8192  # few tiles, long K: the planner splits
+    M, N, K = 80, 2048, 8192  # few tiles, long K: the planner splits
     handle = _lib.lib()
     need = handle.psg_workspace_bytes(M, N, K, 0)
     assert need > 0 and need % (M * N * 4) == 0
@@ -129,7 +129,7 @@ def test_two_streams_take_the_split_plan_without_sharing_a_workspace():
     stream has its own workspace, so both int8 results stay bit-exact."""
     from flydsl_amd import _lib
 
-    M, N, K = 64, 2048, 8192
+    M, N, K = 80, 2048, 8192
     assert _lib.lib().psg_workspace_bytes(M, N, K, 0) > 0
     dev = torch.device("cuda")
     bias = torch.empty(0, dtype=torch.bfloat16, device=dev)

@@ -36,7 +36,7 @@ def test_static_scratch_entry_matches_workspace_entry(kind):
     torch.cuda.set_device(dev)
     assert handle.psg_init() == 0, handle.psg_last_error()
     stream = _lib.stream_handle(None)
-    for (M, N, K) in [(64, 2048, 8192), (72, 512, 6144)]:  # both take the split-K plan; the second is smaller
+    for (M, N, K) in [(80, 2048, 8192), (72, 512, 6144)]:  # both take the split-K plan; the second is smaller
         need = handle.psg_workspace_bytes(M, N, K, _lib.IN_DTYPE[kind])
         assert 0 < need <= handle.psg_static_scratch_bytes()
         d = make_a8w8(M, N, K, kind, seed=M)
