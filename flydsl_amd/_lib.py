@@ -34,6 +34,7 @@ EXPORTS = (
     "psg_debug_tile_order",
     "psg_moe_gemm",
     "psg_moe_reduce",
+    "psg_moe_reduce_masked",
     "psg_moe_sorting",
     "psg_moe_sorting_workspace_bytes",
 )
@@ -180,6 +181,8 @@ def lib() -> ctypes.CDLL:
     handle.psg_tile_coords.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
     handle.psg_debug_tile_order.restype = ctypes.c_int
     handle.psg_debug_tile_order.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p, ctypes.c_void_p]
+    handle.psg_moe_reduce_masked.restype = ctypes.c_int
+    handle.psg_moe_reduce_masked.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int32] * 5 + [ctypes.c_void_p]
     handle.psg_moe_sorting_workspace_bytes.restype = ctypes.c_uint64
     handle.psg_moe_sorting_workspace_bytes.argtypes = [ctypes.c_int32] * 3
     handle.psg_moe_reduce.restype = ctypes.c_int

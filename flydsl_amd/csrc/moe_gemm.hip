@@ -264,13 +264,20 @@ hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int bloc
 
 // sum over the topk slots: y[t, :] = sum_s x[t, s, :] (16-bit in and out, fp32 sum in slot order)
 namespace {
-__global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t* y, int tokens, int topk, int dim, int out_dtype) {
+// mask != nullptr: slot k of token t only counts when mask[ids[t*topk + k]] != 0 (expert parallelism: the rows of experts
+// that live elsewhere were never written by stage 2)
+__global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t* y, int tokens, int topk, int dim, int out_dtype,
+                                                    const int32_t* mask, const int32_t* ids, int experts) {
     const size_t q = (size_t)blockIdx.x * 256 + threadIdx.x;   // one thread per 4 columns
     const size_t quads = (size_t)tokens * (size_t)(dim >> 2);
     if (q >= quads) return;
     const size_t t = q / (size_t)(dim >> 2), c = (q % (size_t)(dim >> 2)) << 2;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     for (int k = 0; k < topk; k++) {
+        if (mask) {
+            const int e = ids[t * topk + k];
+            if ((unsigned)e >= (unsigned)experts || mask[e] == 0) continue;
+        }
         const v2i v = *reinterpret_cast<const v2i*>(x + (t * topk + k) * (size_t)dim + c);
         const uint16_t h0 = (uint16_t)(v[0] & 0xFFFF), h1 = (uint16_t)((uint32_t)v[0] >> 16), h2 = (uint16_t)(v[1] & 0xFFFF), h3 = (uint16_t)((uint32_t)v[1] >> 16);
         if (out_dtype == OUT_BF16) {
@@ -284,9 +291,10 @@ __global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t*
 }
 }  // namespace
 
-hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, hipStream_t stream) {
+hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, const int32_t* mask,
+                                 const int32_t* ids, int experts, hipStream_t stream) {
     const size_t quads = (size_t)tokens * (size_t)(dim >> 2);
     hipLaunchKernelGGL(k_moe_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, static_cast<const uint16_t*>(x),
-                       static_cast<uint16_t*>(y), tokens, topk, dim, out_dtype);
+                       static_cast<uint16_t*>(y), tokens, topk, dim, out_dtype, mask, ids, experts);
     return hipGetLastError();
 }

@@ -16,7 +16,8 @@ hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int bloc
 hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream);
 uint64_t psg_moe_sort_workspace(int64_t pairs, int experts);
 int psg_moe_sort_max_experts();
-hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, hipStream_t stream);
+hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, const int32_t* mask,
+                                 const int32_t* ids, int experts, hipStream_t stream);
 hipError_t psg_launch_mx_generic(const MxGenParams& p, int af, int bf, int store, int batch, hipStream_t stream);
 hipError_t psg_launch_mxfp4_smallm(const MxParams& p, int store, int nw, hipStream_t stream);
 hipError_t psg_launch_splitk_finalize(const A8W8Params& p, const void* partial, int is_int, int scaled, hipStream_t stream);
@@ -587,15 +588,29 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     return 0;
 }
 
-int psg_moe_reduce(const void* x, void* y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void* stream) {
+namespace {
+int moe_reduce_common(const void* x, void* y, const int32_t* mask, const int32_t* ids, int32_t tokens, int32_t topk, int32_t model_dim,
+                      int32_t experts, int32_t dtype, void* stream) {
     if (!x || !y) return fail(PSG_E_NULL, "x and y must be non-NULL");
     if (dtype != PSG_OUT_BF16 && dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "dtype %d must be bf16 or fp16", dtype);
     if (tokens < 1 || topk < 1 || model_dim < 4 || model_dim % 4) return fail(PSG_E_SHAPE, "need tokens, topk >= 1 and model_dim a positive multiple of 4");
     if (!aligned(x, 8) || !aligned(y, 8)) return fail(PSG_E_ALIGN, "x and y must be 8-byte aligned");
-    const hipError_t e = psg_launch_moe_reduce(x, y, tokens, topk, model_dim, dtype, static_cast<hipStream_t>(stream));
+    if (mask && (!ids || experts < 1)) return fail(PSG_E_NULL, "an expert mask needs topk_ids and experts >= 1");
+    const hipError_t e = psg_launch_moe_reduce(x, y, tokens, topk, model_dim, dtype, mask, ids, experts, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_reduce launch");
     g_err[0] = 0;
     return 0;
+}
+}  // namespace
+
+int psg_moe_reduce(const void* x, void* y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void* stream) {
+    return moe_reduce_common(x, y, nullptr, nullptr, tokens, topk, model_dim, 0, dtype, stream);
+}
+
+int psg_moe_reduce_masked(const void* x, void* y, const int32_t* expert_mask, const int32_t* topk_ids, int32_t tokens, int32_t topk,
+                          int32_t model_dim, int32_t experts, int32_t dtype, void* stream) {
+    if (!expert_mask || !topk_ids) return fail(PSG_E_NULL, "expert_mask and topk_ids must be non-NULL");
+    return moe_reduce_common(x, y, expert_mask, topk_ids, tokens, topk, model_dim, experts, dtype, stream);
 }
 
 uint64_t psg_moe_sorting_workspace_bytes(int32_t tokens, int32_t topk, int32_t experts) {

@@ -113,23 +113,34 @@ def compile_moe_gemm2(*, model_dim: int, inter_dim: int, experts: int, topk: int
 class MoeReduction:
     """Launcher returned by :func:`compile_moe_reduction`: ``(X, Y, expert_mask, topk_ids, m_tokens, stream)``."""
 
-    def __init__(self, topk, model_dim, dtype):
+    def __init__(self, topk, model_dim, dtype, use_mask=False, num_experts=0):
         self.topk, self.model_dim, self.dtype = int(topk), int(model_dim), dtype
+        self.use_mask, self.num_experts = bool(use_mask), int(num_experts)
         self._lib = _lib.lib()
 
     def __call__(self, X, Y, expert_mask, topk_ids, i32_m_tokens, stream=None):
         tokens = int(i32_m_tokens)
         dev = _lib.check_operand("Y", Y, min_elems=tokens * self.model_dim, elem_sizes=(2,))
         _lib.check_operand("X", X, min_elems=tokens * self.topk * self.model_dim, elem_sizes=(2,), device=dev)
-        rc = self._lib.psg_moe_reduce(X.data_ptr(), Y.data_ptr(), tokens, self.topk, self.model_dim, self.dtype, _lib.stream_handle(stream))
+        if self.use_mask:
+            # slots whose expert is masked out do not count (and their rows of X were never written)
+            _lib.check_operand("expert_mask", expert_mask, min_elems=self.num_experts, elem_sizes=(4,), device=dev)
+            _lib.check_operand("topk_ids", topk_ids, min_elems=tokens * self.topk, elem_sizes=(4,), device=dev)
+            rc = self._lib.psg_moe_reduce_masked(X.data_ptr(), Y.data_ptr(), expert_mask.data_ptr(), topk_ids.data_ptr(), tokens, self.topk,
+                                                 self.model_dim, self.num_experts, self.dtype, _lib.stream_handle(stream))
+        else:
+            rc = self._lib.psg_moe_reduce(X.data_ptr(), Y.data_ptr(), tokens, self.topk, self.model_dim, self.dtype, _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_moe_reduce")
 
 
 def compile_moe_reduction(*, topk: int, model_dim: int, dtype_str: str = "f16", use_mask: bool = False, num_experts: int = 0,
                           out_dtype_str: str | None = None):
-    """Sum over the topk slots (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203).  Built for f16 / bf16 with the same
-    input and output type and no expert mask; the rest raises ``NotImplementedError``."""
-    if dtype_str not in ("f16", "bf16") or (out_dtype_str not in (None, dtype_str)) or use_mask:
-        raise NotImplementedError("moe reduction is built for f16 / bf16, same type in and out, without an expert mask")
-    return MoeReduction(topk, model_dim, _OUT[dtype_str])
+    """Sum over the topk slots (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203), with ``use_mask`` only over the slots
+    whose expert has ``expert_mask != 0`` (``num_experts`` entries).  Built for f16 / bf16 with the same input and output
+    type; the rest (f32, the MXFP8 route-out rows) raises ``NotImplementedError``."""
+    if dtype_str not in ("f16", "bf16") or (out_dtype_str not in (None, dtype_str)):
+        raise NotImplementedError("moe reduction is built for f16 / bf16, same type in and out")
+    if use_mask and int(num_experts) < 1:
+        raise ValueError("use_mask needs num_experts >= 1")
+    return MoeReduction(topk, model_dim, _OUT[dtype_str], use_mask, num_experts)

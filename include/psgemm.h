@@ -276,9 +276,16 @@ typedef struct psg_moe_args {
 int psg_moe_gemm(const psg_moe_args *args, void *stream);
 
 /* y[t, :] = sum over the topk slots of x[t, slot, :] (fp32 sum in slot order), the pass after stage 2 with accumulate = 0
- * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203, without its expert mask).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16;
+ * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203 with use_mask = False).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16;
  * model_dim % 4 == 0. */
 int psg_moe_reduce(const void *x, void *y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void *stream);
+
+/* The same sum with the reference's expert mask (moe_reduce.py:100-103,147-148): slot k of token t only counts when
+ * expert_mask[topk_ids[t*topk + k]] != 0 (ids outside [0, experts) count as masked).  With expert parallelism the sorter
+ * drops the masked experts, stage 2 never writes their rows of x, and this pass must not read them.
+ * expert_mask [experts] int32, topk_ids [tokens, topk] int32. */
+int psg_moe_reduce_masked(const void *x, void *y, const int32_t *expert_mask, const int32_t *topk_ids, int32_t tokens, int32_t topk,
+                          int32_t model_dim, int32_t experts, int32_t dtype, void *stream);
 
 /*
  * Expert sorting of the routed (token, slot) pairs on the device: what the reference's moe_sorting_flydsl

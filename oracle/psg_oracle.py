@@ -512,6 +512,23 @@ def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int
     return sorted_ids, sorted_w, sorted_e, np.array([begin, tokens], dtype=np.int32)
 
 
+def moe_reduce(x, topk_ids=None, expert_mask=None):
+    """Slot reduction behind the non-accumulating stage 2 (kernels/moe/moe_gemm_2stage/moe_reduce.py:141-150): ``y[t] =
+    sum_k x[t, k]`` in fp32 in slot order; with a mask only the slots with ``expert_mask[topk_ids[t, k]] != 0`` count (the
+    others are replaced by zeros before the addition, so whatever they hold, NaN included, never reaches the sum).  ``x``
+    fp32 ``[tokens, topk, dim]``.  Pinned by a scalar loop on a hand-made case with poisoned masked rows."""
+    x = np.asarray(x, dtype=np.float32)
+    tokens, topk, dim = x.shape
+    y = np.zeros((tokens, dim), dtype=np.float32)
+    for k in range(topk):
+        if expert_mask is None:
+            y += x[:, k]
+        else:
+            on = np.asarray(expert_mask)[np.asarray(topk_ids)[:, k]] != 0
+            y[on] += x[on, k]
+    return y
+
+
 def moe_gemm1(x_q, w1_q, scale_x, scale_w1, topk_ids, topk_weights, inter_dim: int, doweight_stage1: bool, kind: str = "fp8"):
     """Stage 1 of the 2-stage MoE (tests/kernels/test_ref.py:91-161, per-row scales): for every routed (token, slot)
     with expert e, ``y = W1[e] @ x[token]`` over the dequantised operands, ``out[token, slot] = silu(y[:inter]) *

@@ -207,6 +207,89 @@ def test_two_stages_end_to_end_with_reduction():
     assert torch.equal(y, want)
 
 
+@pytest.mark.parametrize("dtype_str", ["bf16", "f16"])
+def test_masked_slot_reduction_skips_rows_stage2_never_wrote(dtype_str):
+    # expert parallelism: the sorter drops the masked experts, stage 2 never writes their rows, the reduction must not read
+    # them (kernels/moe/moe_gemm_2stage/moe_reduce.py:100-103,147-148)
+    from kernels.moe.moe_gemm_2stage import compile_moe_reduction
+
+    dev = torch.device("cuda")
+    tdt = torch.bfloat16 if dtype_str == "bf16" else torch.float16
+    tokens, topk, dim, experts = 77, 4, 520, 16
+    g = torch.Generator().manual_seed(3)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
+    mask = (torch.rand(experts, generator=g) < 0.5).to(torch.int32)
+    mask[0], mask[1] = 1, 0
+    x = torch.randn(tokens, topk, dim, generator=g).to(tdt)
+    xp = x.clone()
+    xp[mask[ids.long()] == 0] = float("nan")
+    y = torch.full((tokens + 2, dim), -8192.0, dtype=tdt, device=dev)
+    red = compile_moe_reduction(topk=topk, model_dim=dim, dtype_str=dtype_str, use_mask=True, num_experts=experts)
+    red(xp.to(dev), y, mask.to(dev), ids.to(dev), tokens, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    want = torch.from_numpy(O.moe_reduce(x.float().numpy(), ids.numpy(), mask.numpy())).to(tdt)
+    assert torch.equal(y[:tokens].cpu(), want)
+    assert (y[tokens:] == -8192.0).all()
+    # without the mask the launcher sums every slot, as before
+    y2 = torch.empty(tokens, dim, dtype=tdt, device=dev)
+    compile_moe_reduction(topk=topk, model_dim=dim, dtype_str=dtype_str)(x.to(dev), y2, None, None, tokens, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    assert torch.equal(y2.cpu(), torch.from_numpy(O.moe_reduce(x.float().numpy())).to(tdt))
+    with pytest.raises(ValueError):
+        compile_moe_reduction(topk=topk, model_dim=dim, dtype_str=dtype_str, use_mask=True)  # num_experts missing
+    with pytest.raises(ValueError):
+        red(xp.to(dev), y, mask.to(dev)[:4], ids.to(dev), tokens, None)  # mask shorter than num_experts
+
+
+def test_expert_parallel_chain_sorter_mask_stage2_masked_reduction():
+    # one rank of an expert-parallel layout: 8 experts, 5 of them local.  The device sorter drops the routed pairs of the other
+    # three and numbers the local experts densely, stage 2 runs on the local weights only and leaves the other slots' rows
+    # untouched (poisoned here), and the masked reduction sums exactly the local slots.
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm2, compile_moe_reduction
+    from kernels.moe.moe_sorting_kernel import moe_sorting_flydsl
+    from flydsl_amd.kernels.moe.moe_sorting import sorted_sizes
+
+    tokens, model_dim, inter_dim, experts, topk, tile_m = 150, 512, 256, 8, 3, 32
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(31)
+    vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
+    ids, wts = ids.to(torch.int32), torch.softmax(vals, dim=1).float()
+    mask = torch.tensor([1, 0, 1, 1, 0, 1, 0, 1], dtype=torch.int32)
+    local = int(mask.sum())
+    rows, blocks = sorted_sizes(tokens, topk, experts, tile_m)
+    sid = torch.empty(rows, dtype=torch.int32, device=dev)
+    swt = torch.empty(rows, dtype=torch.float32, device=dev)
+    se = torch.empty(blocks, dtype=torch.int32, device=dev)
+    nv = torch.empty(2, dtype=torch.int32, device=dev)
+    moe_sorting_flydsl(ids.to(dev), wts.to(dev), sid, swt, se, nv, None, experts, tile_m, mask.to(dev))
+    a2 = torch.randn(tokens * topk, inter_dim, generator=g)
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    a2q, sa2 = quant.pertoken_quant(a2, quant_dtype=torch.float8_e4m3fn)
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=torch.float8_e4m3fn)
+    keep = mask.bool()
+    w2_local = layout.shuffle_weight(w2q[keep].reshape(local * model_dim, inter_dim)).contiguous()
+    out2 = torch.full((tokens * topk, model_dim), float("nan"), dtype=torch.bfloat16, device=dev)
+    e2 = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=local, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128,
+                           doweight_stage2=True, out_dtype="bf16", accumulate=False, in_dtype="fp8")
+    e2(out2, a2q.to(dev).view(-1), w2_local.to(dev).view(-1), sa2.to(dev).view(-1).contiguous(), sw2[keep].to(dev).view(-1).contiguous(), sid, se, swt,
+       nv[:1].contiguous(), tokens, model_dim, inter_dim, blocks, torch.cuda.current_stream())
+    y = torch.empty(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+    compile_moe_reduction(topk=topk, model_dim=model_dim, dtype_str="bf16", use_mask=True, num_experts=experts)(
+        out2, y, mask.to(dev), ids.to(dev), tokens, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    per_slot = O.moe_gemm2(a2q.view(torch.uint8).numpy(), w2q.view(torch.uint8).numpy().reshape(-1, inter_dim), sa2.numpy().reshape(-1),
+                           sw2.numpy().reshape(-1), ids.numpy(), wts.numpy(), model_dim, True, "fp8", reduce_slots=False)
+    got2 = out2.float().cpu().numpy().reshape(tokens, topk, model_dim)
+    on = (mask[ids.long()] != 0).numpy()
+    assert np.isnan(got2[~on]).all(), "rows of masked experts were written"
+    ok, ratio = O.within_north_star_tolerance(got2[on], per_slot[on], 1e-2)
+    assert ok, f"stage 2 on the local experts outside tolerance ({ratio:.3f})"
+    want = torch.from_numpy(O.moe_reduce(np.nan_to_num(got2), ids.numpy(), mask.numpy())).to(torch.bfloat16)
+    assert torch.equal(y.cpu(), want)
+    ok, ratio = O.within_north_star_tolerance(y.float().cpu().numpy(), O.moe_reduce(per_slot, ids.numpy(), mask.numpy()), 2e-2)
+    assert ok, f"masked chain outside tolerance ({ratio:.3f})"
+
+
 def test_moe_argument_errors():
     from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2, compile_moe_reduction
 

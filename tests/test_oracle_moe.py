@@ -69,6 +69,27 @@ def test_moe_sorting_invariants_and_product_sorter():
             assert np.array_equal(a.numpy(), b)
 
 
+def test_moe_reduce_with_and_without_mask_against_a_scalar_loop():
+    rng = np.random.default_rng(5)
+    tokens, topk, dim, experts = 6, 3, 8, 5
+    x = rng.standard_normal((tokens, topk, dim)).astype(np.float32)
+    ids = rng.integers(0, experts, (tokens, topk)).astype(np.int32)
+    mask = np.array([1, 0, 1, 1, 0], dtype=np.int32)
+    xp = x.copy()
+    xp[mask[ids] == 0] = np.nan  # what stage 2 never wrote must not reach the sum
+    got = O.moe_reduce(xp, ids, mask)
+    for t in range(tokens):
+        for d in range(dim):
+            acc = np.float32(0)
+            for k in range(topk):
+                if mask[ids[t, k]]:
+                    acc = np.float32(acc + x[t, k, d])
+            assert got[t, d] == acc
+    assert np.array_equal(O.moe_reduce(x), x[:, 0] + x[:, 1] + x[:, 2])
+    assert np.array_equal(O.moe_reduce(x, ids, np.ones(experts, dtype=np.int32)), O.moe_reduce(x))
+    assert not np.isnan(got).any() and (O.moe_reduce(x, ids, np.zeros(experts, dtype=np.int32)) == 0).all()
+
+
 def test_moe_stage_references_against_scalar_loops():
     rng = np.random.default_rng(3)
     tokens, experts, topk, model_dim, inter = 5, 3, 2, 32, 16
