@@ -16,7 +16,7 @@ def _shapes(seed, n, k_unit, n_unit, k_max):
     rng = np.random.default_rng(seed)
     out = []
     for _ in range(n):
-        m = int(rng.choice([1, 2, 15, 16, 17, 31, 32, 33, 47, 64, 65, 100, 128, 129, 255, 256, 300, 513]))
+        m = int(rng.choice([1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 128, 129, 255, 256, 300, 513]))
         nn = int(rng.integers(1, 40)) * n_unit
         k = int(rng.integers(1, k_max // k_unit + 1)) * k_unit
         out.append((m, nn, k))
