@@ -126,7 +126,7 @@ class MoeArgs(ctypes.Structure):
         ("stage", ctypes.c_int32),
         ("doweight", ctypes.c_int32),
         ("accumulate", ctypes.c_int32),
-        ("pad0", ctypes.c_int32),
+        ("x_slot_major", ctypes.c_int32),
     ]
 
 

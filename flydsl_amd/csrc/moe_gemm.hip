@@ -59,11 +59,12 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         const uint32_t sid = (uint32_t)ids[r];
         const int t = (int)(sid & 0xFFFFFFu), s = (int)(sid >> 24);
         if (t >= p.tokens || s >= p.topk) return -1;
-        return STAGE == 1 ? t : t * p.topk + s;
+        if constexpr (STAGE == 1) return p.x_slot_major ? s * p.tokens + t : t;
+        return t * p.topk + s;
     };
 
     const int K = p.K, KT = K >> 7;
-    const int rows_x = STAGE == 1 ? p.tokens : p.tokens * p.topk;
+    const int rows_x = (STAGE == 1 && !p.x_slot_major) ? p.tokens : p.tokens * p.topk;
     const int rows_e = STAGE == 1 ? 2 * p.n_out : p.n_out;            // weight rows per expert
     __amdgpu_buffer_rsrc_t ra = make_rsrc(p.x, (uint64_t)rows_x * (uint64_t)K);
     const uint8_t* w_e = p.w + (uint64_t)e * (uint64_t)rows_e * (uint64_t)K;

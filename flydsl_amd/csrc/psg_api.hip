@@ -547,7 +547,8 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     if (a->out_dtype < PSG_OUT_BF16 || a->out_dtype > PSG_OUT_F32) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
     if (a->out_dtype == PSG_OUT_F32 && !(a->stage == 2 && a->accumulate))
         return fail(PSG_E_DTYPE, "fp32 output exists only for stage 2 with accumulate (kernels/moe/moe_gemm_2stage/gemm2.py:629)");
-    if (a->pad0 != 0) return fail(PSG_E_SHAPE, "pad0 must be 0");
+    if (a->x_slot_major != 0 && !(a->x_slot_major == 1 && a->stage == 1))
+        return fail(PSG_E_SHAPE, "x_slot_major=%d must be 0, or 1 for stage 1", a->x_slot_major);
     if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
     if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
     if (a->experts < 1) return fail(PSG_E_SHAPE, "experts=%d must be positive", a->experts);
@@ -557,7 +558,7 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     const int K = a->stage == 1 ? a->model_dim : a->inter_dim, n_out = a->stage == 1 ? a->inter_dim : a->model_dim;
     if (K < 128 || K % 128) return fail(PSG_E_SHAPE, "K=%d of stage %d must be a positive multiple of 128", K, a->stage);
     if (n_out < 16 || n_out % 16) return fail(PSG_E_SHAPE, "output width %d of stage %d must be a positive multiple of 16", n_out, a->stage);
-    const uint64_t rows_x = a->stage == 1 ? (uint64_t)a->tokens : (uint64_t)a->tokens * (uint64_t)a->topk;
+    const uint64_t rows_x = (a->stage == 1 && !a->x_slot_major) ? (uint64_t)a->tokens : (uint64_t)a->tokens * (uint64_t)a->topk;
     const uint64_t rows_e = a->stage == 1 ? 2ull * (uint64_t)n_out : (uint64_t)n_out;
     if (rows_x * (uint64_t)K > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "x exceeds the 4 GiB descriptor range");
     if (rows_e * (uint64_t)K > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "one expert's weights exceed the 4 GiB descriptor range");
@@ -573,6 +574,7 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     p.expert_ids = a->sorted_expert_ids;
     p.sorted_w = a->sorted_weights;
     p.num_valid = a->num_valid_ids;
+    p.x_slot_major = a->x_slot_major;
     p.tokens = a->tokens;
     p.topk = a->topk;
     p.experts = a->experts;

@@ -163,6 +163,7 @@ struct MoeParams {
     int out_dtype;              // OUT_BF16 / OUT_FP16 / OUT_F32 (stage 2 with accumulate only)
     int doweight;               // multiply by the routing weight in this stage
     int accumulate;             // stage 2: atomic add into out[token] (else one row per (token, slot))
+    int x_slot_major;           // stage 1: x / sx hold one row per (slot, token) at slot*tokens + token
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).

@@ -7,7 +7,8 @@
 
 (gemm1.py:541-580 / launch_moe_gemm1 :502-537; gemm2.py:595-643; moe_reduce.py:164-203.)  ``x`` / ``w`` are fp8
 (e4m3fn) or int8 with one fp32 scale per row; ``w`` is ``shuffle_weight`` of the experts' weights stacked along the
-rows.  Built: ``in_dtype`` "fp8" and "int8"; "int8smooth" and "int4" raise ``NotImplementedError``.  ``tile_m`` is the
+rows.  Built: ``in_dtype`` "fp8", "int8" and "int8smooth" (int8 whose stage-1 ``x`` / ``scale_x`` hold one row per (slot,
+token), gemm1.py:100-101,321-328; stage 2 is plain int8); "int4" raises ``NotImplementedError``.  ``tile_m`` is the
 block size of the expert sorting and must be 16, 32, 64 or 128; ``tile_n`` / ``tile_k`` are checked with the reference's
 rules and then treated as hints.
 """
@@ -43,7 +44,8 @@ class MoeStage:
         self.stage, self.model_dim, self.inter_dim = int(stage), int(model_dim), int(inter_dim)
         self.experts, self.topk, self.tile_m = int(experts), int(topk), int(tile_m)
         self.doweight, self.accumulate = bool(doweight), bool(accumulate)
-        self.out_dtype, self.in_dtype = _OUT[str(out_dtype).strip().lower()], _lib.IN_DTYPE[in_dtype]
+        self.slot_major = in_dtype == "int8smooth" and int(stage) == 1
+        self.out_dtype, self.in_dtype = _OUT[str(out_dtype).strip().lower()], _lib.IN_DTYPE["int8" if in_dtype == "int8smooth" else in_dtype]
         self._lib = _lib.lib()
 
     def __call__(self, out, x, w, scale_x, scale_w, sorted_token_ids, sorted_expert_ids, sorted_weights, num_valid_ids,
@@ -52,7 +54,7 @@ class MoeStage:
         n_out, K = (self.inter_dim, self.model_dim) if self.stage == 1 else (self.model_dim, self.inter_dim)
         if (int(dim0), int(dim1)) != (n_out, K):
             raise ValueError(f"stage {self.stage} was built for dims ({n_out}, {K}), called with ({dim0}, {dim1})")
-        rows_x = tokens if self.stage == 1 else tokens * self.topk
+        rows_x = tokens if (self.stage == 1 and not self.slot_major) else tokens * self.topk
         rows_w = self.experts * (2 * n_out if self.stage == 1 else n_out)
         rows_out = tokens * self.topk if (self.stage == 1 or not self.accumulate) else tokens
         osize = 4 if self.out_dtype == 2 else 2
@@ -75,6 +77,7 @@ class MoeStage:
         a.sorted_size, a.blocks, a.block_m = int(sorted_token_ids.numel()), blocks, self.tile_m
         a.in_dtype, a.out_dtype, a.stage = self.in_dtype, self.out_dtype, self.stage
         a.doweight, a.accumulate = int(self.doweight), int(self.accumulate)
+        a.x_slot_major = int(self.slot_major)
         rc = self._lib.psg_moe_gemm(ctypes.byref(a), _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_moe_gemm")
@@ -83,8 +86,8 @@ class MoeStage:
 def _check_in_dtype(in_dtype):
     if in_dtype not in ("fp8", "int8", "int8smooth", "int4"):
         raise ValueError(f"in_dtype must be 'fp8', 'int8', 'int8smooth', or 'int4', got {in_dtype!r}")
-    if in_dtype in ("int8smooth", "int4"):
-        raise NotImplementedError(f"in_dtype={in_dtype!r} is not built (fp8 and int8 are)")
+    if in_dtype == "int4":
+        raise NotImplementedError("in_dtype='int4' (W4A8) is not built (fp8, int8 and int8smooth are)")
 
 
 def compile_moe_gemm1(*, model_dim: int, inter_dim: int, experts: int, topk: int, tile_m: int, tile_n: int, tile_k: int,

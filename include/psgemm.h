@@ -270,7 +270,8 @@ typedef struct psg_moe_args {
     int32_t stage;       /* 1 or 2 */
     int32_t doweight;
     int32_t accumulate;  /* stage 2 only */
-    int32_t pad0;        /* 0 */
+    int32_t x_slot_major; /* stage 1 only: 1 = x and scale_x hold one row per (slot, token), row slot*tokens + token (the
+                             reference's int8smooth inputs, kernels/moe/moe_gemm_2stage/gemm1.py:100-101,321-328); 0 = one row per token */
 } psg_moe_args;
 
 int psg_moe_gemm(const psg_moe_args *args, void *stream);

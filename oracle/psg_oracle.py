@@ -529,12 +529,15 @@ def moe_reduce(x, topk_ids=None, expert_mask=None):
     return y
 
 
-def moe_gemm1(x_q, w1_q, scale_x, scale_w1, topk_ids, topk_weights, inter_dim: int, doweight_stage1: bool, kind: str = "fp8"):
+def moe_gemm1(x_q, w1_q, scale_x, scale_w1, topk_ids, topk_weights, inter_dim: int, doweight_stage1: bool, kind: str = "fp8",
+              x_slot_major: bool = False):
     """Stage 1 of the 2-stage MoE (tests/kernels/test_ref.py:91-161, per-row scales): for every routed (token, slot)
     with expert e, ``y = W1[e] @ x[token]`` over the dequantised operands, ``out[token, slot] = silu(y[:inter]) *
     y[inter:]`` (times the routing weight when ``doweight_stage1``).  ``x_q [tokens, model_dim]``, ``w1_q
-    [experts*2*inter, model_dim]`` bit patterns (``kind`` "fp8" / "int8"), scales fp32 per row.  Returns fp32
-    ``[tokens, topk, inter_dim]``.  Pinned by scalar float64 loops on tiny inputs."""
+    [experts*2*inter, model_dim]`` bit patterns (``kind`` "fp8" / "int8"), scales fp32 per row.  With ``x_slot_major`` (the
+    int8smooth inputs, tests/kernels/test_moe_gemm_2stage.py:482-519) ``x_q`` / ``scale_x`` hold one row per (slot, token)
+    at ``slot*tokens + token`` and the pair (token, slot) multiplies ITS row.  Returns fp32 ``[tokens, topk, inter_dim]``.
+    Pinned by scalar float64 loops on tiny inputs (both layouts)."""
     x = _as_f32_operand(np.asarray(x_q), kind) * np.asarray(scale_x, dtype=np.float32).reshape(-1, 1)
     w = _as_f32_operand(np.asarray(w1_q), kind) * np.asarray(scale_w1, dtype=np.float32).reshape(-1, 1)
     ids = np.asarray(topk_ids)
@@ -545,7 +548,7 @@ def moe_gemm1(x_q, w1_q, scale_x, scale_w1, topk_ids, topk_weights, inter_dim: i
         t, s = np.nonzero(ids == e)
         if t.size == 0:
             continue
-        y2 = (x[t] @ w[e].T).astype(np.float32)
+        y2 = (x[s * tokens + t if x_slot_major else t] @ w[e].T).astype(np.float32)
         g, u = y2[:, :inter_dim], y2[:, inter_dim:]
         with np.errstate(over="ignore"):
             y = (g / (np.float32(1.0) + np.exp(-g))).astype(np.float32) * u

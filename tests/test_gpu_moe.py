@@ -241,6 +241,45 @@ def test_masked_slot_reduction_skips_rows_stage2_never_wrote(dtype_str):
         red(xp.to(dev), y, mask.to(dev)[:4], ids.to(dev), tokens, None)  # mask shorter than num_experts
 
 
+@pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile_m,tokens", [(16, 33), (32, 129), (64, 64), (128, 300)])
+def test_stage1_int8smooth_slot_major_rows(out_dtype, tile_m, tokens):
+    # the reference's int8smooth stage 1 (tests/kernels/test_moe_gemm_2stage.py:482-519,586-604): x is expanded per route, scaled
+    # by a per-expert smooth vector, quantised per (token, slot) and stored slot-major; the kernel gathers row slot*tokens + token
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1
+
+    model_dim, inter_dim, experts, topk = 256, 128, 8, 2
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(tokens)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, tokens)
+    x = torch.randn(tokens, model_dim, generator=g)
+    w1 = torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim)
+    smooth = 0.75 + 0.5 * torch.rand(experts, model_dim, generator=g)
+    x_route = x[:, None, :].expand(tokens, topk, model_dim) * smooth[ids.long()]
+    amax = x_route.abs().amax(dim=-1, keepdim=True)
+    sx = amax / 127.0
+    sx[sx == 0] = 1.0
+    xq = (x_route / sx).to(torch.int8)
+    xq_sm = xq.permute(1, 0, 2).contiguous().view(topk * tokens, model_dim)
+    sx_sm = sx.permute(1, 0, 2).contiguous().view(-1)
+    w1q, sw1 = quant.pertoken_quant(w1, quant_dtype=torch.int8)
+    out = torch.full((tokens, topk, inter_dim), float("nan"), dtype=TDT[out_dtype], device=dev)
+    exe = compile_moe_gemm1(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128,
+                            doweight_stage1=False, out_dtype=out_dtype, in_dtype="int8smooth")
+    _launch(exe, out, xq_sm, layout.shuffle_weight(w1q).view(-1, model_dim).contiguous(), sx_sm, sw1.view(-1, 1), routing, inter_dim, model_dim, tokens)
+    ref = O.moe_gemm1(xq_sm.view(torch.uint8).numpy(), w1q.view(torch.uint8).numpy().reshape(-1, model_dim), sx_sm.numpy(), sw1.numpy().reshape(-1),
+                      ids.numpy(), wts.numpy(), inter_dim, False, "int8", x_slot_major=True)
+    got = out.float().cpu().numpy()
+    assert _cos(got, ref) > 0.99  # the reference's own bar
+    ok, ratio = O.within_north_star_tolerance(got, ref, 1e-2)
+    assert ok, f"outside tolerance ({ratio:.3f})"
+    # stage 2 of int8smooth is the int8 stage 2: the launcher takes the name
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm2
+    e2 = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128,
+                           doweight_stage2=True, out_dtype=out_dtype, accumulate=True, in_dtype="int8smooth")
+    assert e2.slot_major is False
+
+
 def test_expert_parallel_chain_sorter_mask_stage2_masked_reduction():
     # one rank of an expert-parallel layout: 8 experts, 5 of them local.  The device sorter drops the routed pairs of the other
     # three and numbers the local experts densely, stage 2 runs on the local weights only and leaves the other slots' rows
@@ -303,6 +342,8 @@ def test_moe_argument_errors():
         compile_moe_gemm1(model_dim=384, inter_dim=128, experts=4, topk=2, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False)
     with pytest.raises(NotImplementedError):
         compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, in_dtype="int4")
+    with pytest.raises(ValueError):
+        compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, in_dtype="int2")
     with pytest.raises(ValueError):
         compile_moe_gemm1(**SHAPE, tile_m=48, tile_n=64, tile_k=128, doweight_stage1=False)
     with pytest.raises(NotImplementedError):

@@ -69,6 +69,33 @@ def test_moe_sorting_invariants_and_product_sorter():
             assert np.array_equal(a.numpy(), b)
 
 
+def test_moe_gemm1_slot_major_rows_against_a_scalar_loop():
+    # the int8smooth layout: one row of x and one scale per (slot, token) at slot*tokens + token
+    rng = np.random.default_rng(9)
+    tokens, experts, topk, model_dim, inter = 4, 3, 2, 16, 8
+    ids, w = _routing(tokens, experts, topk, 4)
+    xq = rng.integers(-127, 128, (topk * tokens, model_dim)).astype(np.int8)
+    w1q = rng.integers(-127, 128, (experts * 2 * inter, model_dim)).astype(np.int8)
+    sx = rng.uniform(0.01, 0.02, topk * tokens).astype(np.float32)
+    sw1 = rng.uniform(0.001, 0.002, experts * 2 * inter).astype(np.float32)
+    want = np.zeros((tokens, topk, inter))
+    for t in range(tokens):
+        for s in range(topk):
+            e, r = int(ids[t, s]), s * tokens + t
+            for n in range(inter):
+                g = sum(float(xq[r, k]) * sx[r] * float(w1q[e * 2 * inter + n, k]) * sw1[e * 2 * inter + n] for k in range(model_dim))
+                u = sum(float(xq[r, k]) * sx[r] * float(w1q[e * 2 * inter + inter + n, k]) * sw1[e * 2 * inter + inter + n] for k in range(model_dim))
+                want[t, s, n] = g / (1 + math.exp(-g)) * u
+    got = O.moe_gemm1(xq.view(np.uint8), w1q.view(np.uint8), sx, sw1, ids, w, inter, False, "int8", x_slot_major=True)
+    assert np.allclose(got, want, rtol=2e-5, atol=1e-6 * np.abs(want).max())
+    # rows that repeat the token's row in every slot give the token-major result
+    rep_x = np.tile(xq[:tokens], (topk, 1))
+    rep_s = np.tile(sx[:tokens], topk)
+    a = O.moe_gemm1(rep_x.view(np.uint8), w1q.view(np.uint8), rep_s, sw1, ids, w, inter, False, "int8", x_slot_major=True)
+    b = O.moe_gemm1(xq[:tokens].view(np.uint8), w1q.view(np.uint8), sx[:tokens], sw1, ids, w, inter, False, "int8")
+    assert np.array_equal(a, b)
+
+
 def test_moe_reduce_with_and_without_mask_against_a_scalar_loop():
     rng = np.random.default_rng(5)
     tokens, topk, dim, experts = 6, 3, 8, 5
