@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -37,6 +37,9 @@ EXPORTS = (
     "psg_moe_reduce_masked",
     "psg_moe_sorting",
     "psg_moe_sorting_workspace_bytes",
+    "psg_moe_topk_gating",
+    "psg_moe_softmax_sorting",
+    "psg_moe_softmax_sorting_fused",
 )
 
 
@@ -152,6 +155,21 @@ class MoeSortArgs(ctypes.Structure):
     ]
 
 
+class MoeGatingArgs(ctypes.Structure):
+    _fields_ = [
+        ("gating", ctypes.c_void_p),
+        ("weights", ctypes.c_void_p),
+        ("indices", ctypes.c_void_p),
+        ("token_expert_indices", ctypes.c_void_p),
+        ("tokens", ctypes.c_int32),
+        ("experts", ctypes.c_int32),
+        ("topk", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("renormalize", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
+    ]
+
+
 _lib = None
 
 
@@ -187,7 +205,11 @@ def lib() -> ctypes.CDLL:
     handle.psg_moe_sorting_workspace_bytes.argtypes = [ctypes.c_int32] * 3
     handle.psg_moe_reduce.restype = ctypes.c_int
     handle.psg_moe_reduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int32] * 4 + [ctypes.c_void_p]
-    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm", "psg_moe_sorting"):
+    handle.psg_moe_softmax_sorting.restype = ctypes.c_int
+    handle.psg_moe_softmax_sorting.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    handle.psg_moe_softmax_sorting_fused.restype = ctypes.c_int
+    handle.psg_moe_softmax_sorting_fused.argtypes = [ctypes.c_int32] * 3
+    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm", "psg_moe_sorting", "psg_moe_topk_gating"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]

@@ -18,7 +18,7 @@
 //      expert, the total, the block ids;
 //   3. one workgroup per (expert, slice) compacts that slice's pairs of that expert straight to their final rows.
 // Either way extra workgroups of the first launch clear the caller's accumulate buffer at full memory bandwidth.
-#include "psg_common.h"
+#include "moe_gating.h"
 
 namespace {
 
@@ -28,6 +28,8 @@ constexpr int SORT_MAX_EXPERTS = 4096;
 constexpr int SORT_ONESHOT_PAIRS = 4096;   // routings up to this many pairs always take the single launch
 constexpr int SORT_SLICE = 2048;           // pairs per slice of the three-launch path (more when there are > 64 slices)
 constexpr int SORT_MAX_SLICES = 64;
+constexpr int FUSE_MAX_TOKENS = 32;        // the gating + sorting launch: every sorting workgroup repeats the gating of all tokens
+constexpr int FUSE_MAX_PAIRS = 1024;
 
 __device__ __forceinline__ int pack_id(int slot, int token) { return (int)(((unsigned)slot << 24) | (unsigned)token); }
 
@@ -53,7 +55,7 @@ __device__ __forceinline__ void fill_tails(const MoeSortParams& p, int total, in
 
 // Stable compaction of the pairs [q_begin, q_end) whose expert is e into rows dst, dst + 1, ...: every wavefront takes a
 // contiguous quarter, counts its matches, and after one barrier writes them behind the wavefronts before it.
-__device__ __forceinline__ void compact_range(const MoeSortParams& p, int e, int q_begin, int q_end, int dst, int (&wcount)[SORT_WAVES]) {
+__device__ __forceinline__ void compact_range(const MoeSortParams& p, const int* ids, const float* wts, int e, int q_begin, int q_end, int dst, int (&wcount)[SORT_WAVES]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int len = q_end - q_begin, per = ((len + SORT_WAVES - 1) / SORT_WAVES + 63) & ~63;
     const int lo = q_begin + wave * per, hi = lo + per < q_end ? lo + per : q_end;
@@ -61,7 +63,7 @@ __device__ __forceinline__ void compact_range(const MoeSortParams& p, int e, int
 #pragma unroll 4
     for (int q0 = lo; q0 < hi; q0 += 64) {
         const int q = q0 + lane;
-        mine += __popcll(__ballot(q < hi && p.topk_ids[q] == e));
+        mine += __popcll(__ballot(q < hi && ids[q] == e));
     }
     if (lane == 0) wcount[wave] = mine;
     __syncthreads();
@@ -69,13 +71,13 @@ __device__ __forceinline__ void compact_range(const MoeSortParams& p, int e, int
     for (int w = 0; w < wave; w++) row += wcount[w];
     for (int q0 = lo; q0 < hi; q0 += 64) {
         const int q = q0 + lane;
-        const bool hit = q < hi && p.topk_ids[q] == e;
+        const bool hit = q < hi && ids[q] == e;
         const unsigned long long ballot = __ballot(hit);
         if (hit) {
             const int r = row + __popcll(ballot & ((1ull << lane) - 1ull));
             const int token = q / p.topk, slot = q - token * p.topk;
             p.sorted_ids[r] = pack_id(slot, token);
-            p.sorted_weights[r] = p.topk_weights[q];
+            p.sorted_weights[r] = wts[q];
         }
         row += __popcll(ballot);
     }
@@ -91,21 +93,17 @@ __device__ __forceinline__ void fill_padding(const MoeSortParams& p, int start, 
 }
 
 // ---- single launch: grid = experts sorting workgroups + clearing workgroups ----
-__global__ void __launch_bounds__(SORT_THREADS) k_moe_sort(MoeSortParams p) {
+// the work of sorting workgroup e on the routing (ids, wts), which lies in global memory or in LDS
+__device__ __forceinline__ void sort_one_expert(const MoeSortParams& p, const int* ids, const float* wts, int e) {
     __shared__ int hist[SORT_MAX_EXPERTS];
     __shared__ int wcount[SORT_WAVES];
     __shared__ int red[3][SORT_WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int e = (int)blockIdx.x;
-    if (e >= p.experts) {
-        clear_share(p, e - p.experts, (int)gridDim.x - p.experts);
-        return;
-    }
     const int P = p.tokens * p.topk, B = p.block_m;
     for (int i = tid; i < p.experts; i += SORT_THREADS) hist[i] = 0;
     __syncthreads();
     for (int q = tid; q < P; q += SORT_THREADS) {
-        const int id = p.topk_ids[q];
+        const int id = ids[q];
         if ((unsigned)id < (unsigned)p.experts) atomicAdd(&hist[id], 1);  // ids outside [0, experts) are dropped
     }
     __syncthreads();
@@ -141,13 +139,62 @@ __global__ void __launch_bounds__(SORT_THREADS) k_moe_sort(MoeSortParams p) {
     }
     const bool enabled = !p.expert_mask || p.expert_mask[e] != 0;
     const int cnt = enabled ? hist[e] : 0;
-    if (cnt > 0) compact_range(p, e, 0, P, below, wcount);  // cnt is uniform over the workgroup
+    if (cnt > 0) compact_range(p, ids, wts, e, 0, P, below, wcount);  // cnt is uniform over the workgroup
     fill_padding(p, below, cnt, local);
     fill_tails(p, total, e, p.experts);
     if (e == 0 && tid == 0) {
         p.num_valid[0] = total;
         p.num_valid[1] = p.tokens;
     }
+}
+
+__global__ void __launch_bounds__(SORT_THREADS) k_moe_sort(MoeSortParams p) {
+    const int e = (int)blockIdx.x;
+    if (e >= p.experts) {
+        clear_share(p, e - p.experts, (int)gridDim.x - p.experts);
+        return;
+    }
+    sort_one_expert(p, p.topk_ids, p.topk_weights, e);
+}
+
+// ---- gating + sorting in one launch (decode): every sorting workgroup first computes the routing of all tokens from the
+// router logits into LDS (a few KB of logits from L2 per workgroup, cheaper than a launch), then sorts from there.
+// Workgroup 0 also writes the routing to g.weights / g.indices / g.tei where those are given.
+template <typename T, int VPT>
+__global__ void __launch_bounds__(SORT_THREADS) k_moe_gate_sort(MoeSortParams p, MoeGatingParams g) {
+    __shared__ int s_ids[FUSE_MAX_PAIRS];
+    __shared__ float s_w[FUSE_MAX_PAIRS];
+    const int e = (int)blockIdx.x;
+    if (e >= p.experts) {
+        clear_share(p, e - p.experts, (int)gridDim.x - p.experts);
+        return;
+    }
+    const int L = g.lanes, sh = __builtin_ctz(L), tpb = SORT_THREADS >> sh;
+    const int gl = threadIdx.x & (L - 1);
+    for (int t0 = 0; t0 < p.tokens; t0 += tpb) {
+        const int t = t0 + (int)(threadIdx.x >> sh);
+        const bool live = t < p.tokens;
+        const T* row = static_cast<const T*>(g.gating) + (size_t)(live ? t : 0) * p.experts;
+        float sel_w[GATE_MAX_TOPK];
+        int sel_i[GATE_MAX_TOPK];
+        const float f = gate_row<T, VPT>(row, p.experts, p.topk, g.renorm != 0, L, gl, g.vec != 0, sel_w, sel_i);
+        if (live && gl == 0) {
+#pragma unroll
+            for (int k = 0; k < GATE_MAX_TOPK; k++)
+                if (k < p.topk) {
+                    const int q = t * p.topk + k;
+                    s_ids[q] = sel_i[k];
+                    s_w[q] = sel_w[k] * f;
+                    if (e == 0) {
+                        if (g.weights) g.weights[q] = sel_w[k] * f;
+                        if (g.indices) g.indices[q] = sel_i[k];
+                        if (g.tei) g.tei[q] = k * p.tokens + t;
+                    }
+                }
+        }
+    }
+    __syncthreads();
+    sort_one_expert(p, s_ids, s_w, e);
 }
 
 // ---- three launches.  Workspace (ints): off[(slices + 1) * experts] | start[experts] | local[experts] | total ----
@@ -242,7 +289,7 @@ __global__ void __launch_bounds__(SORT_THREADS) k_moe_sort_scatter(MoeSortParams
     if (next == first) return;  // uniform over the workgroup
     const int P = p.tokens * p.topk;
     const int lo = g * plan.slice_len, hi = lo + plan.slice_len < P ? lo + plan.slice_len : P;
-    compact_range(p, e, lo, hi, start[e] + first, wcount);
+    compact_range(p, p.topk_ids, p.topk_weights, e, lo, hi, start[e] + first, wcount);
 }
 
 int clear_wgs(const MoeSortParams& p) {
@@ -263,6 +310,43 @@ SortPlan make_plan(int64_t pairs) {
 }  // namespace
 
 int psg_moe_sort_max_experts() { return SORT_MAX_EXPERTS; }
+
+// whether gating + sorting of this routing runs as one launch
+bool psg_moe_gate_sort_fuses(int tokens, int topk, int experts) {
+    return tokens <= FUSE_MAX_TOKENS && (int64_t)tokens * topk <= FUSE_MAX_PAIRS && experts <= GATE_MAX_EXPERTS && topk <= GATE_MAX_TOPK;
+}
+
+namespace {
+template <typename T>
+hipError_t launch_gate_sort_t(const MoeSortParams& p, const MoeGatingParams& g, int vpt, int grid, hipStream_t stream) {
+    switch (vpt) {
+        case 1: hipLaunchKernelGGL((k_moe_gate_sort<T, 1>), dim3(grid), dim3(SORT_THREADS), 0, stream, p, g); break;
+        case 2: hipLaunchKernelGGL((k_moe_gate_sort<T, 2>), dim3(grid), dim3(SORT_THREADS), 0, stream, p, g); break;
+        case 4: hipLaunchKernelGGL((k_moe_gate_sort<T, 4>), dim3(grid), dim3(SORT_THREADS), 0, stream, p, g); break;
+        case 8: hipLaunchKernelGGL((k_moe_gate_sort<T, 8>), dim3(grid), dim3(SORT_THREADS), 0, stream, p, g); break;
+        default: hipLaunchKernelGGL((k_moe_gate_sort<T, 16>), dim3(grid), dim3(SORT_THREADS), 0, stream, p, g); break;
+    }
+    return hipGetLastError();
+}
+}  // namespace
+
+// One launch: gating of g (dtype 0 fp32, 1 bf16, 2 fp16) feeding the sort of p; p.topk_ids / p.topk_weights are not read.
+// Requires psg_moe_gate_sort_fuses(tokens, topk, experts).
+hipError_t psg_launch_moe_gate_sort(const MoeSortParams& p, MoeGatingParams g, int dtype, hipStream_t stream) {
+    int vpt, lanes;
+    gate_layout(p.experts, &vpt, &lanes);
+    const int esz = dtype == 0 ? 4 : 2;
+    const int chunk = vpt * esz, need = chunk < 16 ? chunk : 16;
+    g.lanes = lanes;
+    g.vec = p.experts % vpt == 0 && reinterpret_cast<uintptr_t>(g.gating) % need == 0 && ((size_t)p.experts * esz) % need == 0;
+    const int grid = p.experts + clear_wgs(p);
+    switch (dtype) {
+        case 0: return launch_gate_sort_t<float>(p, g, vpt, grid, stream);
+        case 1: return launch_gate_sort_t<uint16_t>(p, g, vpt, grid, stream);
+        case 2: return launch_gate_sort_t<_Float16>(p, g, vpt, grid, stream);
+    }
+    return hipErrorInvalidValue;
+}
 
 // bytes of workspace the three-launch path wants for this routing (0: the single launch is used anyway)
 uint64_t psg_moe_sort_workspace(int64_t pairs, int experts) {

@@ -8,6 +8,7 @@
 #include <mutex>
 
 #include "psg_common.h"
+#include "moe_gating.h"
 #include "tile_order.h"
 
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
@@ -16,6 +17,9 @@ hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int bloc
 hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream);
 uint64_t psg_moe_sort_workspace(int64_t pairs, int experts);
 int psg_moe_sort_max_experts();
+hipError_t psg_launch_moe_gating(MoeGatingParams p, int dtype, hipStream_t stream);
+hipError_t psg_launch_moe_gate_sort(const MoeSortParams& p, MoeGatingParams g, int dtype, hipStream_t stream);
+bool psg_moe_gate_sort_fuses(int tokens, int topk, int experts);
 hipError_t psg_launch_moe_reduce(const void* x, void* y, int tokens, int topk, int dim, int out_dtype, const int32_t* mask,
                                  const int32_t* ids, int experts, hipStream_t stream);
 hipError_t psg_launch_mx_generic(const MxGenParams& p, int af, int bf, int store, int batch, hipStream_t stream);
@@ -229,6 +233,73 @@ int static_scratch(void** out) {
         g_scratch_ptr[dev] = ptr;
     }
     *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+// Argument checks of the expert sorter; `need_routing`: topk_ids / topk_weights are read (not with the fused gating).
+int check_moe_sort(const psg_moe_sort_args* a, bool need_routing, MoeSortParams* out) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if ((need_routing && (!a->topk_ids || !a->topk_weights)) || !a->sorted_ids || !a->sorted_weights || !a->sorted_expert_ids || !a->num_valid_ids)
+        return fail(PSG_E_NULL, "topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids must be non-NULL");
+    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
+    if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
+    if (a->experts < 1 || a->experts > psg_moe_sort_max_experts()) return fail(PSG_E_SHAPE, "experts=%d outside [1, %d]", a->experts, psg_moe_sort_max_experts());
+    if (a->block_m < 1 || a->block_m > 4096) return fail(PSG_E_SHAPE, "block_m=%d outside [1, 4096]", a->block_m);
+    const int64_t pairs = (int64_t)a->tokens * a->topk;
+    const int64_t need = pairs + (int64_t)a->experts * a->block_m - a->topk;
+    if (need > 0x7FFFFFFF) return fail(PSG_E_SHAPE, "tokens*topk + experts*block_m must stay below 2^31");
+    if (a->sorted_size < need) return fail(PSG_E_SHAPE, "sorted_size=%d is below tokens*topk + experts*block_m - topk = %lld", a->sorted_size, (long long)need);
+    if ((int64_t)a->blocks * a->block_m < a->sorted_size)
+        return fail(PSG_E_SHAPE, "blocks=%d must cover sorted_size=%d rows in blocks of %d", a->blocks, a->sorted_size, a->block_m);
+    if (a->zero_buf && (a->zero_bytes < 0 || a->zero_bytes % 16 || !aligned(a->zero_buf, 16)))
+        return fail(PSG_E_ALIGN, "zero_buf must be 16-byte aligned and zero_bytes a multiple of 16");
+    if (a->workspace && !aligned(a->workspace, 4)) return fail(PSG_E_ALIGN, "workspace must be 4-byte aligned");
+    MoeSortParams p;
+    p.topk_ids = a->topk_ids;
+    p.topk_weights = a->topk_weights;
+    p.expert_mask = a->expert_mask;
+    p.sorted_ids = a->sorted_ids;
+    p.sorted_weights = a->sorted_weights;
+    p.sorted_expert_ids = a->sorted_expert_ids;
+    p.num_valid = a->num_valid_ids;
+    p.zero_buf = a->zero_bytes > 0 ? static_cast<v4i*>(a->zero_buf) : nullptr;
+    p.zero_vec = a->zero_buf ? a->zero_bytes / 16 : 0;
+    p.tokens = a->tokens;
+    p.topk = a->topk;
+    p.experts = a->experts;
+    p.block_m = a->block_m;
+    p.sorted_size = a->sorted_size;
+    p.blocks = a->blocks;
+    *out = p;
+    return 0;
+}
+
+// Argument checks of the router gating; `need_outputs`: weights / indices must be given (optional with the fused sorting).
+int check_moe_gating(const psg_moe_gating_args* a, bool need_outputs, MoeGatingParams* out) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!a->gating) return fail(PSG_E_NULL, "gating must be non-NULL");
+    if (need_outputs && (!a->weights || !a->indices)) return fail(PSG_E_NULL, "weights and indices must be non-NULL");
+    if (a->dtype < 0 || a->dtype > 2) return fail(PSG_E_DTYPE, "dtype %d unknown (0 fp32, 1 bf16, 2 fp16)", a->dtype);
+    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
+    if (a->experts < 1 || a->experts > GATE_MAX_EXPERTS) return fail(PSG_E_SHAPE, "experts=%d outside [1, %d]", a->experts, GATE_MAX_EXPERTS);
+    if (a->topk < 1 || a->topk > GATE_MAX_TOPK || a->topk > a->experts)
+        return fail(PSG_E_SHAPE, "topk=%d outside [1, min(%d, experts=%d)]", a->topk, GATE_MAX_TOPK, a->experts);
+    if (a->renormalize != 0 && a->renormalize != 1) return fail(PSG_E_SHAPE, "renormalize=%d must be 0 or 1", a->renormalize);
+    if (!aligned(a->gating, a->dtype == 0 ? 4 : 2) || (a->weights && !aligned(a->weights, 4)) || (a->indices && !aligned(a->indices, 4)) ||
+        (a->token_expert_indices && !aligned(a->token_expert_indices, 4)))
+        return fail(PSG_E_ALIGN, "gating must be aligned to its element size, the outputs to 4 bytes");
+    MoeGatingParams g;
+    g.gating = a->gating;
+    g.weights = a->weights;
+    g.indices = a->indices;
+    g.tei = a->token_expert_indices;
+    g.tokens = a->tokens;
+    g.experts = a->experts;
+    g.topk = a->topk;
+    g.renorm = a->renormalize;
+    g.lanes = 1;
+    g.vec = 0;
+    *out = g;
     return 0;
 }
 
@@ -621,40 +692,48 @@ uint64_t psg_moe_sorting_workspace_bytes(int32_t tokens, int32_t topk, int32_t e
 }
 
 int psg_moe_sorting(const psg_moe_sort_args* a, void* stream) {
-    if (!a) return fail(PSG_E_NULL, "args is NULL");
-    if (!a->topk_ids || !a->topk_weights || !a->sorted_ids || !a->sorted_weights || !a->sorted_expert_ids || !a->num_valid_ids)
-        return fail(PSG_E_NULL, "topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids must be non-NULL");
-    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
-    if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
-    if (a->experts < 1 || a->experts > psg_moe_sort_max_experts()) return fail(PSG_E_SHAPE, "experts=%d outside [1, %d]", a->experts, psg_moe_sort_max_experts());
-    if (a->block_m < 1 || a->block_m > 4096) return fail(PSG_E_SHAPE, "block_m=%d outside [1, 4096]", a->block_m);
-    const int64_t pairs = (int64_t)a->tokens * a->topk;
-    const int64_t need = pairs + (int64_t)a->experts * a->block_m - a->topk;
-    if (need > 0x7FFFFFFF) return fail(PSG_E_SHAPE, "tokens*topk + experts*block_m must stay below 2^31");
-    if (a->sorted_size < need) return fail(PSG_E_SHAPE, "sorted_size=%d is below tokens*topk + experts*block_m - topk = %lld", a->sorted_size, (long long)need);
-    if ((int64_t)a->blocks * a->block_m < a->sorted_size)
-        return fail(PSG_E_SHAPE, "blocks=%d must cover sorted_size=%d rows in blocks of %d", a->blocks, a->sorted_size, a->block_m);
-    if (a->zero_buf && (a->zero_bytes < 0 || a->zero_bytes % 16 || !aligned(a->zero_buf, 16)))
-        return fail(PSG_E_ALIGN, "zero_buf must be 16-byte aligned and zero_bytes a multiple of 16");
     MoeSortParams p;
-    p.topk_ids = a->topk_ids;
-    p.topk_weights = a->topk_weights;
-    p.expert_mask = a->expert_mask;
-    p.sorted_ids = a->sorted_ids;
-    p.sorted_weights = a->sorted_weights;
-    p.sorted_expert_ids = a->sorted_expert_ids;
-    p.num_valid = a->num_valid_ids;
-    p.zero_buf = a->zero_bytes > 0 ? static_cast<v4i*>(a->zero_buf) : nullptr;
-    p.zero_vec = a->zero_buf ? a->zero_bytes / 16 : 0;
-    p.tokens = a->tokens;
-    p.topk = a->topk;
-    p.experts = a->experts;
-    p.block_m = a->block_m;
-    p.sorted_size = a->sorted_size;
-    p.blocks = a->blocks;
-    if (a->workspace && !aligned(a->workspace, 4)) return fail(PSG_E_ALIGN, "workspace must be 4-byte aligned");
+    if (int rc = check_moe_sort(a, true, &p)) return rc;
     const hipError_t e = psg_launch_moe_sort(p, a->workspace, a->workspace ? a->workspace_bytes : 0, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_sorting launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+int psg_moe_topk_gating(const psg_moe_gating_args* a, void* stream) {
+    MoeGatingParams g;
+    if (int rc = check_moe_gating(a, true, &g)) return rc;
+    const hipError_t e = psg_launch_moe_gating(g, a->dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_topk_gating launch");
+    g_err[0] = 0;
+    return 0;
+}
+
+int psg_moe_softmax_sorting_fused(int32_t tokens, int32_t topk, int32_t experts) {
+    return tokens >= 1 && topk >= 1 && experts >= 1 && psg_moe_gate_sort_fuses(tokens, topk, experts) ? 1 : 0;
+}
+
+int psg_moe_softmax_sorting(const psg_moe_gating_args* ga, const psg_moe_sort_args* sa, void* stream) {
+    if (!ga || !sa) return fail(PSG_E_NULL, "args is NULL");
+    if (ga->tokens != sa->tokens || ga->topk != sa->topk || ga->experts != sa->experts)
+        return fail(PSG_E_SHAPE, "gating (tokens=%d topk=%d experts=%d) and sorting (tokens=%d topk=%d experts=%d) disagree", ga->tokens,
+                    ga->topk, ga->experts, sa->tokens, sa->topk, sa->experts);
+    const bool fused = ga->tokens >= 1 && ga->topk >= 1 && ga->experts >= 1 && psg_moe_gate_sort_fuses(ga->tokens, ga->topk, ga->experts);
+    MoeGatingParams g;
+    MoeSortParams p;
+    if (int rc = check_moe_gating(ga, !fused, &g)) return rc;
+    if (int rc = check_moe_sort(sa, false, &p)) return rc;
+    hipError_t e;
+    if (fused) {
+        e = psg_launch_moe_gate_sort(p, g, ga->dtype, static_cast<hipStream_t>(stream));
+    } else {
+        // two steps: the sorter reads what the gating kernel wrote
+        if ((const void*)sa->topk_ids != (const void*)ga->indices || (const void*)sa->topk_weights != (const void*)ga->weights)
+            return fail(PSG_E_NULL, "beyond the fused range the sorter's topk_ids / topk_weights must be the gating's indices / weights");
+        e = psg_launch_moe_gating(g, ga->dtype, static_cast<hipStream_t>(stream));
+        if (e == hipSuccess) e = psg_launch_moe_sort(p, sa->workspace, sa->workspace ? sa->workspace_bytes : 0, static_cast<hipStream_t>(stream));
+    }
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_softmax_sorting launch");
     g_err[0] = 0;
     return 0;
 }

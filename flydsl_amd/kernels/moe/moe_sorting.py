@@ -29,6 +29,47 @@ def moe_sorting_get_workspace_size(M, num_experts, topk, unit_size=UNIT_SIZE):
     return int(_lib.lib().psg_moe_sorting_workspace_bytes(int(M), int(topk), int(num_experts)))
 
 
+def _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size, expert_mask,
+               workspace, device, routing=()):
+    """Checks the sorter's tensors and fills a ``psg_moe_sort_args`` (``routing`` = (topk_ids, topk_weights) when they are read)."""
+    E, B = int(num_experts), int(unit_size)
+    need_rows, _ = sorted_sizes(tokens, topk, E, B)
+    checks = [("sorted_ids", sorted_ids, torch.int32, need_rows), ("sorted_weights", sorted_weights, torch.float32, need_rows),
+              ("sorted_expert_ids", sorted_expert_ids, torch.int32, (need_rows + B - 1) // B), ("num_valid_ids", num_valid_ids, torch.int32, 2)]
+    if routing:
+        checks += [("topk_ids", routing[0], torch.int32, tokens * topk), ("topk_weights", routing[1], torch.float32, tokens * topk)]
+    if expert_mask is not None:
+        checks.append(("expert_mask", expert_mask, torch.int32, E))
+    for name, t, dt, n in checks:
+        if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
+            raise ValueError(f"{name} must be a contiguous {dt} device tensor")
+        if t.numel() < n:
+            raise ValueError(f"{name} holds {t.numel()} elements, this call needs at least {n}")
+    if sorted_weights.numel() < sorted_ids.numel():
+        raise ValueError("sorted_weights must be as long as sorted_ids")
+    args = _lib.MoeSortArgs()
+    if routing:
+        args.topk_ids, args.topk_weights = routing[0].data_ptr(), routing[1].data_ptr()
+    args.expert_mask = expert_mask.data_ptr() if expert_mask is not None else None
+    args.sorted_ids, args.sorted_weights = sorted_ids.data_ptr(), sorted_weights.data_ptr()
+    args.sorted_expert_ids, args.num_valid_ids = sorted_expert_ids.data_ptr(), num_valid_ids.data_ptr()
+    if moe_buf is not None and moe_buf.numel():
+        if not moe_buf.is_cuda or not moe_buf.is_contiguous():
+            raise ValueError("moe_buf must be a contiguous device tensor")
+        args.zero_buf, args.zero_bytes = moe_buf.data_ptr(), moe_buf.numel() * moe_buf.element_size()
+    want = int(_lib.lib().psg_moe_sorting_workspace_bytes(tokens, topk, E))
+    if workspace is None and want:
+        workspace = torch.empty(want, dtype=torch.uint8, device=device)
+    if workspace is not None and workspace is not False:
+        if not workspace.is_cuda or not workspace.is_contiguous():
+            raise ValueError("workspace must be a contiguous device tensor")
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    args.tokens, args.topk, args.experts, args.block_m = tokens, topk, E, B
+    args.sorted_size = sorted_ids.numel()
+    args.blocks = min(sorted_expert_ids.numel(), (sorted_ids.numel() + B - 1) // B)
+    return args, workspace
+
+
 def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf,
                        num_experts, unit_size=UNIT_SIZE, expert_mask=None, num_local_tokens=None, workspace=None, *,
                        stream=None):
@@ -43,41 +84,41 @@ def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorte
     if topk_ids.dim() != 2 or topk_ids.shape != topk_weights.shape:
         raise ValueError("topk_ids and topk_weights must both be [tokens, topk]")
     tokens, topk = topk_ids.shape
-    E, B = int(num_experts), int(unit_size)
-    need_rows, _ = sorted_sizes(tokens, topk, E, B)
-    checks = [("topk_ids", topk_ids, torch.int32, tokens * topk), ("topk_weights", topk_weights, torch.float32, tokens * topk),
-              ("sorted_ids", sorted_ids, torch.int32, need_rows), ("sorted_weights", sorted_weights, torch.float32, need_rows),
-              ("sorted_expert_ids", sorted_expert_ids, torch.int32, (need_rows + B - 1) // B), ("num_valid_ids", num_valid_ids, torch.int32, 2)]
-    if expert_mask is not None:
-        checks.append(("expert_mask", expert_mask, torch.int32, E))
-    for name, t, dt, n in checks:
-        if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
-            raise ValueError(f"{name} must be a contiguous {dt} device tensor")
-        if t.numel() < n:
-            raise ValueError(f"{name} holds {t.numel()} elements, this call needs at least {n}")
-    if sorted_weights.numel() < sorted_ids.numel():
-        raise ValueError("sorted_weights must be as long as sorted_ids")
-    args = _lib.MoeSortArgs()
-    args.topk_ids, args.topk_weights = topk_ids.data_ptr(), topk_weights.data_ptr()
-    args.expert_mask = expert_mask.data_ptr() if expert_mask is not None else None
-    args.sorted_ids, args.sorted_weights = sorted_ids.data_ptr(), sorted_weights.data_ptr()
-    args.sorted_expert_ids, args.num_valid_ids = sorted_expert_ids.data_ptr(), num_valid_ids.data_ptr()
-    if moe_buf is not None and moe_buf.numel():
-        if not moe_buf.is_cuda or not moe_buf.is_contiguous():
-            raise ValueError("moe_buf must be a contiguous device tensor")
-        args.zero_buf, args.zero_bytes = moe_buf.data_ptr(), moe_buf.numel() * moe_buf.element_size()
-    want = int(_lib.lib().psg_moe_sorting_workspace_bytes(tokens, topk, E))
-    if workspace is None and want:
-        workspace = torch.empty(want, dtype=torch.uint8, device=topk_ids.device)
-    if workspace is not None and workspace is not False:
-        if not workspace.is_cuda or not workspace.is_contiguous():
-            raise ValueError("workspace must be a contiguous device tensor")
-        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
-    args.tokens, args.topk, args.experts, args.block_m = tokens, topk, E, B
-    args.sorted_size = sorted_ids.numel()
-    args.blocks = min(sorted_expert_ids.numel(), (sorted_ids.numel() + B - 1) // B)
+    args, _ws = _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size,
+                           expert_mask, workspace, topk_ids.device, routing=(topk_ids, topk_weights))
     handle = _lib.lib()
     rc = handle.psg_moe_sorting(ctypes.byref(args), _lib.stream_handle(stream))
+    if rc != 0:
+        raise (ValueError if rc < 0 else RuntimeError)(handle.psg_last_error().decode())
+    return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf
+
+
+def moe_softmax_sort_flydsl(gating_logits, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, topk,
+                            dtype_str, unit_size=UNIT_SIZE, expert_mask=None, renormalize=True, num_local_tokens=None, *,
+                            topk_ids=None, topk_weights=None, workspace=None, stream=None):
+    """Router logits -> softmax -> top-k -> expert sort: the reference's fused entry point (moe_sorting_kernel.py:2250-2400),
+    same positional arguments and the same outputs as ``moe_sorting_flydsl``.  Up to 32 tokens this is ONE launch (every
+    sorting workgroup repeats the gating of all tokens in LDS; ``topk_ids`` / ``topk_weights`` are then optional extra
+    outputs); beyond that the gating kernel and the sorter run back to back, through ``topk_ids`` / ``topk_weights`` when the
+    caller gives them (``[tokens, topk]`` int32 / fp32; needed under graph capture) and through fresh tensors otherwise."""
+    from .topk_gating_softmax import gating_args
+
+    if num_local_tokens is not None:
+        raise NotImplementedError("num_local_tokens (expert-parallel token count) is not implemented")
+    if gating_logits.dim() != 2 or gating_logits.shape[1] != int(num_experts):
+        raise ValueError("gating_logits must be [tokens, num_experts]")
+    tokens, topk = int(gating_logits.shape[0]), int(topk)
+    handle = _lib.lib()
+    fused = bool(handle.psg_moe_softmax_sorting_fused(tokens, topk, int(num_experts)))
+    if not fused:
+        if topk_ids is None:
+            topk_ids = torch.empty((tokens, topk), dtype=torch.int32, device=gating_logits.device)
+        if topk_weights is None:
+            topk_weights = torch.empty((tokens, topk), dtype=torch.float32, device=gating_logits.device)
+    gargs = gating_args(gating_logits, topk_weights, topk_ids, None, tokens, int(num_experts), topk, dtype_str, renormalize)
+    sargs, _ws = _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size,
+                            expert_mask, workspace, gating_logits.device, routing=() if fused else (topk_ids, topk_weights))
+    rc = handle.psg_moe_softmax_sorting(ctypes.byref(gargs), ctypes.byref(sargs), _lib.stream_handle(stream))
     if rc != 0:
         raise (ValueError if rc < 0 else RuntimeError)(handle.psg_last_error().decode())
     return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf

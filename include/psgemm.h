@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 5
+#define PSG_ABI_VERSION 6
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
@@ -326,6 +326,38 @@ typedef struct psg_moe_sort_args {
 
 uint64_t psg_moe_sorting_workspace_bytes(int32_t tokens, int32_t topk, int32_t experts);
 int psg_moe_sorting(const psg_moe_sort_args *args, void *stream);
+
+/* Router gating in front of the sorter: softmax over the experts, top-k, optional renormalisation.  Replaces the
+ * launcher returned by build_topk_gating_softmax_module (kernels/moe/topk_gating_softmax_kernel.py:392-686; call shape
+ * (gating, weights, indices, tei, num_tokens, stream) :656-663; tests/kernels/test_topk_gating_softmax.py).
+ *   gating [tokens, experts] row-major, dtype 0 = fp32, 1 = bf16, 2 = fp16 (the x_dtype numbering of the quantisers);
+ *   p = exp2((x - max) * log2 e) / sum in fp32; top-k = k rounds of arg-max over p, the LOWER expert index winning ties,
+ *   the winner masked (:585-618); renormalize = 1 multiplies the k weights by 1 / max(their sum, 1e-20) (:623-625);
+ *   weights [tokens, topk] fp32, indices [tokens, topk] int32 in the order found (descending weight),
+ *   token_expert_indices NULL or [tokens, topk] int32 = k * tokens + token (:648-650).
+ * experts <= 1024 (any value, not only the reference's power-of-two splits), topk <= min(32, experts). */
+typedef struct psg_moe_gating_args {
+    const void *gating;
+    float *weights;
+    int32_t *indices;
+    int32_t *token_expert_indices;
+    int32_t tokens, experts, topk;
+    int32_t dtype;
+    int32_t renormalize; /* 0 or 1 */
+    int32_t pad0;        /* 0 */
+} psg_moe_gating_args;
+
+int psg_moe_topk_gating(const psg_moe_gating_args *args, void *stream);
+
+/* Gating followed by sorting: the reference's moe_softmax_sort_flydsl (kernels/moe/moe_sorting_kernel.py:2250-2400).
+ * tokens / topk / experts of both structs must agree.  psg_moe_softmax_sorting_fused(tokens, topk, experts) = 1 says that
+ * this routing runs as ONE launch (tokens <= 32 and tokens*topk <= 1024: every sorting workgroup repeats the gating of
+ * all tokens into LDS; the reference fuses up to 16 tokens, :2313-2320): then sort->topk_ids / topk_weights are not
+ * read, and gating->weights / indices / token_expert_indices are optional outputs (written when non-NULL).  Otherwise
+ * the gating kernel runs first and the sorter reads its outputs: sort->topk_ids must be gating->indices and
+ * sort->topk_weights gating->weights (both non-NULL). */
+int psg_moe_softmax_sorting_fused(int32_t tokens, int32_t topk, int32_t experts);
+int psg_moe_softmax_sorting(const psg_moe_gating_args *gating, const psg_moe_sort_args *sort, void *stream);
 
 #ifdef __cplusplus
 }

@@ -512,6 +512,33 @@ def moe_sorting(topk_ids: np.ndarray, topk_weights: np.ndarray, num_experts: int
     return sorted_ids, sorted_w, sorted_e, np.array([begin, tokens], dtype=np.int32)
 
 
+def topk_gating_softmax(gating, topk: int, renormalize: bool = True):
+    """Router gating (kernels/moe/topk_gating_softmax_kernel.py:545-650): fp32 ``p = exp2((x - max) * log2 e) * (1 / sum)``;
+    ``topk`` rounds of arg-max over ``p`` in which the LOWER expert index wins ties and the winner is masked with -inf
+    (:585-618); ``renormalize`` multiplies the winners by ``1 / max(their sum, 1e-20)`` (:623-625).  ``gating`` ``[tokens,
+    experts]`` (any float dtype; converted to fp32 as the kernel does).  Returns ``(weights fp32 [tokens, topk], indices int32
+    [tokens, topk], token_expert_indices int32 [tokens, topk] = k * tokens + token)`` (:648-650).
+    Pinned by ``scipy.special.softmax`` + a stable descending sort in float64, closed forms (uniform logits, one dominant
+    logit, topk = experts) and shift invariance."""
+    x = np.asarray(gating, dtype=np.float32)
+    tokens, experts = x.shape
+    mx = x.max(axis=1, keepdims=True)
+    e = np.exp2((x - mx) * np.float32(1.4426950408889634)).astype(np.float32)
+    p = e * (np.float32(1.0) / e.sum(axis=1, keepdims=True, dtype=np.float32))
+    w = np.zeros((tokens, topk), dtype=np.float32)
+    idx = np.zeros((tokens, topk), dtype=np.int32)
+    rows = np.arange(tokens)
+    for k in range(topk):
+        j = p.argmax(axis=1)  # the first maximum: the lowest index among equals
+        w[:, k] = p[rows, j]
+        idx[:, k] = j
+        p[rows, j] = -np.inf
+    if renormalize:
+        w = w * (np.float32(1.0) / np.maximum(w.sum(axis=1, keepdims=True, dtype=np.float32), np.float32(1e-20)))
+    tei = (np.arange(topk, dtype=np.int32)[None, :] * np.int32(tokens) + np.arange(tokens, dtype=np.int32)[:, None]).astype(np.int32)
+    return w.astype(np.float32), idx, tei
+
+
 def moe_reduce(x, topk_ids=None, expert_mask=None):
     """Slot reduction behind the non-accumulating stage 2 (kernels/moe/moe_gemm_2stage/moe_reduce.py:141-150): ``y[t] =
     sum_k x[t, k]`` in fp32 in slot order; with a mask only the slots with ``expert_mask[topk_ids[t, k]] != 0`` count (the

@@ -359,6 +359,8 @@ def test_struct_layouts_match_header():
                offsetof(psg_moe_args, accumulate));
         printf("%zu %zu %zu %zu\n", sizeof(psg_moe_sort_args), offsetof(psg_moe_sort_args, workspace_bytes), offsetof(psg_moe_sort_args, tokens),
                offsetof(psg_moe_sort_args, blocks));
+        printf("%zu %zu %zu %zu\n", sizeof(psg_moe_gating_args), offsetof(psg_moe_gating_args, token_expert_indices),
+               offsetof(psg_moe_gating_args, tokens), offsetof(psg_moe_gating_args, renormalize));
         return 0;
     }'''
     with tempfile.TemporaryDirectory() as d:
@@ -375,7 +377,46 @@ def test_struct_layouts_match_header():
     want += [ctypes.sizeof(e), e.num_valid_ids.offset, e.tokens.offset, e.accumulate.offset]
     so = _lib.MoeSortArgs
     want += [ctypes.sizeof(so), so.workspace_bytes.offset, so.tokens.offset, so.blocks.offset]
+    ga = _lib.MoeGatingArgs
+    want += [ctypes.sizeof(ga), ga.token_expert_indices.offset, ga.tokens.offset, ga.renormalize.offset]
     assert [int(v) for v in out] == want
+
+
+def test_gating_validation_errors_without_a_gpu():
+    handle = _lib.lib()
+    assert handle.psg_moe_topk_gating(None, None) == -1
+    g = _lib.MoeGatingArgs()
+    assert handle.psg_moe_topk_gating(ctypes.byref(g), None) == -1 and b"gating" in handle.psg_last_error()
+    g.gating = g.weights = g.indices = 0x1000
+    g.tokens, g.experts, g.topk, g.dtype, g.renormalize = 4, 128, 6, 1, 1
+    for field, val, code, word in (("dtype", 3, -3, b"dtype"), ("tokens", 0, -2, b"tokens"), ("experts", 1025, -2, b"experts"),
+                                   ("topk", 33, -2, b"topk"), ("topk", 0, -2, b"topk"), ("renormalize", 2, -2, b"renormalize"),
+                                   ("weights", 0x1002, -6, b"aligned"), ("gating", 0x1001, -6, b"aligned"), ("indices", 0, -1, b"indices")):
+        old = getattr(g, field)
+        setattr(g, field, val)
+        assert handle.psg_moe_topk_gating(ctypes.byref(g), None) == code, field
+        assert word in handle.psg_last_error(), (field, handle.psg_last_error())
+        setattr(g, field, old)
+    g.experts, g.topk = 4, 5  # more winners than experts
+    assert handle.psg_moe_topk_gating(ctypes.byref(g), None) == -2
+    g.experts, g.topk = 128, 6
+    # the pair: shapes must agree; beyond the fused range the sorter must read the gating's outputs
+    assert handle.psg_moe_softmax_sorting_fused(16, 8, 256) == 1 and handle.psg_moe_softmax_sorting_fused(32, 32, 64) == 1
+    assert handle.psg_moe_softmax_sorting_fused(33, 8, 256) == 0 and handle.psg_moe_softmax_sorting_fused(16, 8, 2048) == 0
+    assert handle.psg_moe_softmax_sorting_fused(0, 8, 256) == 0
+    s = _lib.MoeSortArgs()
+    for f in ("sorted_ids", "sorted_weights", "sorted_expert_ids", "num_valid_ids"):
+        setattr(s, f, 0x2000)
+    s.tokens, s.topk, s.experts, s.block_m = 4, 6, 64, 32
+    s.sorted_size, s.blocks = 4 * 6 + 128 * 32, (4 * 6 + 128 * 32 + 31) // 32
+    assert handle.psg_moe_softmax_sorting(ctypes.byref(g), None, None) == -1
+    assert handle.psg_moe_softmax_sorting(ctypes.byref(g), ctypes.byref(s), None) == -2 and b"disagree" in handle.psg_last_error()
+    s.experts = 128
+    g.tokens = s.tokens = 100  # two steps: topk_ids / topk_weights missing
+    s.sorted_size, s.blocks = 100 * 6 + 128 * 32, (100 * 6 + 128 * 32 + 31) // 32
+    assert handle.psg_moe_softmax_sorting(ctypes.byref(g), ctypes.byref(s), None) == -1
+    s.topk_ids, s.topk_weights = 0x3000, 0x1000  # ids are not the gating's indices
+    assert handle.psg_moe_softmax_sorting(ctypes.byref(g), ctypes.byref(s), None) == -1 and b"indices" in handle.psg_last_error()
 
 
 def test_validation_errors_come_back_as_codes_without_a_gpu():

@@ -156,3 +156,40 @@ def test_moe_stage_references_against_scalar_loops():
             assert np.allclose(got2, want2, rtol=2e-5, atol=1e-6 * np.abs(want2).max())
             per_slot = O.moe_gemm2(a2q, w2q, sa2, sw2, ids, w, model_dim, dow, kind, reduce_slots=False)
             assert np.allclose(per_slot.sum(1), got2, rtol=1e-6, atol=1e-7)
+
+
+def test_topk_gating_softmax_against_scipy_and_closed_forms():
+    import scipy.special
+
+    rng = np.random.default_rng(3)
+    for tokens, experts, topk in ((37, 128, 6), (5, 8, 2), (16, 96, 9), (3, 7, 7)):
+        x = rng.uniform(-2, 2, (tokens, experts)).astype(np.float32)
+        p = scipy.special.softmax(x.astype(np.float64), axis=1)
+        order = np.argsort(-p, axis=1, kind="stable")[:, :topk]  # an independent top-k: stable sort = lower index first
+        want_w = np.take_along_axis(p, order, axis=1)
+        for renorm in (False, True):
+            w, idx, tei = O.topk_gating_softmax(x, topk, renorm)
+            assert np.array_equal(idx, order.astype(np.int32))
+            ref = want_w / want_w.sum(1, keepdims=True) if renorm else want_w
+            assert np.allclose(w, ref, rtol=2e-6, atol=0)
+            assert w.dtype == np.float32 and idx.dtype == np.int32 and tei.dtype == np.int32
+            assert all(tei[t, k] == k * tokens + t for t in range(tokens) for k in range(topk))
+            if renorm:
+                assert np.allclose(w.sum(1), 1.0, atol=1e-6)
+        # a shift of the logits changes nothing (max subtraction)
+        w1, i1, _ = O.topk_gating_softmax(x + np.float32(8.0), topk, True)
+        w0, i0, _ = O.topk_gating_softmax(x, topk, True)
+        assert np.array_equal(i0, i1) and np.allclose(w0, w1, rtol=1e-5)
+    # uniform logits: every probability 1/E, ties go to the lowest indices in order; renormalised 1/k
+    w, idx, _ = O.topk_gating_softmax(np.full((2, 16), 0.25, np.float32), 4, False)
+    assert np.array_equal(idx, np.tile(np.arange(4, dtype=np.int32), (2, 1))) and np.allclose(w, 1 / 16)
+    w, _, _ = O.topk_gating_softmax(np.full((2, 16), 0.25, np.float32), 4, True)
+    assert np.allclose(w, 0.25)
+    # one dominant logit: weight ~1 first; equal runners-up in index order
+    x = np.zeros((1, 8), np.float32)
+    x[0, 5] = 40.0
+    w, idx, _ = O.topk_gating_softmax(x, 3, False)
+    assert idx.tolist() == [[5, 0, 1]] and abs(w[0, 0] - 1.0) < 1e-6 and w[0, 1] == w[0, 2] < 1e-15
+    # ties between distinct positions inside a row
+    x = np.array([[1.0, 3.0, 3.0, 0.0, 3.0, 2.0]], np.float32)
+    assert O.topk_gating_softmax(x, 4, True)[1].tolist() == [[1, 2, 4, 5]]
