@@ -335,6 +335,54 @@ def run_next_row_workloads():
         sec = timed(lambda: moe_sorting_flydsl(d_ids, d_w, *bufs, acc, experts, tile_m, None, None, ws), iters=50)
         out.append({"workload": f"moe_sorting_tokens{tokens}_e{experts}_top{topk}_block{tile_m}_clear{tokens}x{model_dim}bf16",
                     "us_per_launch_events": sec * 1e6, "tflops": 0.0, "weight_gb_per_s": 0.0})
+    # the router gating in front of the sorter, alone and as one call with the sorter; 20 launches recorded into a HIP graph
+    # (these kernels are shorter than the gap between two eager launches)
+    from kernels.moe.moe_sorting_kernel import moe_softmax_sort_flydsl
+    from kernels.moe.topk_gating_softmax_kernel import build_topk_gating_softmax_module
+
+    def graph_timed(f, steps=20):
+        for _ in range(3):
+            f()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(steps):
+                f()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / 1e3 / steps / 10)
+        return best
+
+    for tokens, experts, topk in ((16, 256, 8), (16, 128, 6), (1024, 128, 6), (16384, 256, 8)):
+        g = torch.Generator().manual_seed(0)
+        x = (torch.rand(tokens, experts, generator=g) * 4 - 2).to(torch.bfloat16).to(dev)
+        w = torch.empty(tokens, topk, dtype=torch.float32, device=dev)
+        idx = torch.empty(tokens, topk, dtype=torch.int32, device=dev)
+        tei = torch.empty_like(idx)
+        launch = build_topk_gating_softmax_module(num_experts=experts, topk=topk, dtype_str="bf16")
+        sec = graph_timed(lambda: launch(x, w, idx, tei, tokens, stream=torch.cuda.current_stream()))
+        out.append({"workload": f"moe_topk_gating_bf16_tokens{tokens}_e{experts}_top{topk}", "us_per_launch_events": sec * 1e6, "tflops": 0.0,
+                    "weight_gb_per_s": (tokens * experts * 2 + tokens * topk * 12) / sec / 1e9})
+        rows, blocks = sorted_sizes(tokens, topk, experts, 32)
+        bufs = (torch.empty(rows, dtype=torch.int32, device=dev), torch.empty(rows, dtype=torch.float32, device=dev),
+                torch.empty(blocks, dtype=torch.int32, device=dev), torch.empty(2, dtype=torch.int32, device=dev))
+        acc = torch.empty(tokens, 4096, dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(max(4, moe_sorting_get_workspace_size(tokens, experts, topk)), dtype=torch.uint8, device=dev)
+        sec = graph_timed(lambda: moe_softmax_sort_flydsl(x, *bufs, acc, experts, topk, "bf16", 32, None, True, None, topk_ids=idx, topk_weights=w,
+                                                          workspace=ws, stream=torch.cuda.current_stream()))
+        out.append({"workload": f"moe_softmax_sort_bf16_tokens{tokens}_e{experts}_top{topk}_block32_clear{tokens}x4096bf16", "us_per_launch_events": sec * 1e6,
+                    "tflops": 0.0, "weight_gb_per_s": 0.0})
     return out
 
 

@@ -19,16 +19,34 @@ __device__ __forceinline__ float gate_to_f32<_Float16>(_Float16 v) { return (flo
 template <>
 __device__ __forceinline__ float gate_to_f32<uint16_t>(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }  // bf16 bits
 
+// Exchange step S of a butterfly over a group of 2, 4, 8, 16, 32 or 64 lanes: every lane gets the value of lane ^ mask with
+// masks 1, 2, 7, 15 (DPP: quad permutes, half-row mirror, row mirror; any masks that span the group make a butterfly), then
+// 16 and 32 through the LDS crossbar.  Steps 0 .. log2(L)-1 cover a group of L lanes.
+template <int S>
+__device__ __forceinline__ int gate_xchg(int v) {
+    if constexpr (S == 0) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+    else if constexpr (S == 1) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    else if constexpr (S == 2) return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false); // row_half_mirror
+    else if constexpr (S == 3) return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false); // row_mirror
+    else if constexpr (S == 4) return __shfl_xor(v, 16);
+    else return __shfl_xor(v, 32);
+}
+template <int S>
+__device__ __forceinline__ float gate_xchg(float v) { return __builtin_bit_cast(float, gate_xchg<S>(__builtin_bit_cast(int, v))); }
+
+constexpr int GATE_KEEP = 16;  // winners a lane may have to keep: topk <= experts <= 16 * lanes
+
 // Lane gl of the group owns the columns [gl * VPT, gl * VPT + VPT) of `row`; columns >= E count as -inf.  `vec`: every
 // lane's columns can be fetched as one aligned vector (E % VPT == 0, base and row pitch aligned).  All L lanes of the
-// group must call this together; all of them return the same winners in sel_w / sel_i (entries 0 .. K-1) and the
-// factor to apply to the weights (1 without renormalisation).
-template <typename T, int VPT>
-__device__ __forceinline__ float gate_row(const T* row, int E, int K, bool renorm, int L, int gl, bool vec,
-                                          float (&sel_w)[GATE_MAX_TOPK], int (&sel_i)[GATE_MAX_TOPK]) {
+// group must call this together.  Winner k (k = 0 .. K-1, descending weight) is reported through found(k, index) on every
+// lane, and its weight stays with lane k % L in keep[k / L]; the return value is the factor to apply to the weights
+// (1 without renormalisation), the same on every lane.
+template <typename T, int VPT, class F>
+__device__ __forceinline__ float gate_row(const T* row, int E, int K, bool renorm, int L, int gl, bool vec, float (&keep)[GATE_KEEP], F&& found) {
     struct alignas(sizeof(T) * VPT) Vec {
         T v[VPT];
     };
+    const int sh = __builtin_ctz(L);
     const int c0 = gl * VPT;
     float x[VPT];
     if (vec) {
@@ -47,39 +65,57 @@ __device__ __forceinline__ float gate_row(const T* row, int E, int K, bool renor
     float mx = -INFINITY;
 #pragma unroll
     for (int v = 0; v < VPT; v++) mx = fmaxf(mx, x[v]);
-    for (int o = L >> 1; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    static_for<6>([&](auto S) {
+        if (decltype(S)::value < sh) mx = fmaxf(mx, gate_xchg<decltype(S)::value>(mx));
+    });
     float sum = 0.f;
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
-        x[v] = exp2f((x[v] - mx) * 1.4426950408889634f);  // exp2(-inf) = 0 for the columns past E
+        x[v] = __builtin_amdgcn_exp2f((x[v] - mx) * 1.4426950408889634f);  // the hardware exp2 (the reference's is fast-math too); exp2(-inf) = 0
         sum += x[v];
     }
-    for (int o = L >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    const float inv = 1.0f / sum;
+    static_for<6>([&](auto S) {
+        if (decltype(S)::value < sh) sum += gate_xchg<decltype(S)::value>(sum);
+    });
+    const float inv = __builtin_amdgcn_rcpf(sum);  // sum >= 1 (the maximum contributes exp2(0))
 #pragma unroll
     for (int v = 0; v < VPT; v++) x[v] = c0 + v < E ? x[v] * inv : -INFINITY;
     float picked = 0.f;
     for (int k = 0; k < K; k++) {
-        float bv = -INFINITY;
-        int bi = -1;
+        // arg-max of the lane's values as a tree (short dependency chains: one wavefront per SIMD has nothing else to
+        // issue); the higher column of a pair wins only when strictly greater, so the lowest column of equal values stays
+        float tv[VPT];
+        int ti[VPT];
 #pragma unroll
         for (int v = 0; v < VPT; v++) {
-            const bool better = x[v] > bv;  // strict: the lowest column of equal values stays
-            bv = better ? x[v] : bv;
-            bi = better ? c0 + v : bi;
-        }
-        for (int o = L >> 1; o > 0; o >>= 1) {
-            const float pv = __shfl_xor(bv, o);
-            const int pi = __shfl_xor(bi, o);
-            const bool take = pv > bv || (pv == bv && pi < bi);
-            bv = take ? pv : bv;
-            bi = take ? pi : bi;
+            tv[v] = x[v];
+            ti[v] = c0 + v;
         }
 #pragma unroll
-        for (int j = 0; j < GATE_MAX_TOPK; j++) {
-            sel_w[j] = j == k ? bv : sel_w[j];
-            sel_i[j] = j == k ? bi : sel_i[j];
-        }
+        for (int w = 1; w < VPT; w <<= 1)
+#pragma unroll
+            for (int v = 0; v + w < VPT; v += 2 * w) {
+                const bool hi = tv[v + w] > tv[v];
+                tv[v] = hi ? tv[v + w] : tv[v];
+                ti[v] = hi ? ti[v + w] : ti[v];
+            }
+        float bv = tv[0];
+        int bi = tv[0] == -INFINITY ? -1 : ti[0];
+        static_for<6>([&](auto S) {
+            if (decltype(S)::value < sh) {
+                const float pv = gate_xchg<decltype(S)::value>(bv);
+                const int pi = gate_xchg<decltype(S)::value>(bi);
+                const bool take = pv > bv || (pv == bv && pi < bi);
+                bv = take ? pv : bv;
+                bi = take ? pi : bi;
+            }
+        });
+        found(k, bi);
+        const int slot = k >> sh;
+        const bool mine = gl == (k & (L - 1));
+#pragma unroll
+        for (int j = 0; j < GATE_KEEP; j++)
+            if (j == slot) keep[j] = mine ? bv : keep[j];  // (slot is uniform: one predicated move per round)
         picked += bv;
 #pragma unroll
         for (int v = 0; v < VPT; v++) x[v] = c0 + v == bi ? -INFINITY : x[v];

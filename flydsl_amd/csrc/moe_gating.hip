@@ -13,17 +13,20 @@ __global__ void __launch_bounds__(256) k_topk_gating(MoeGatingParams p) {
     const int t = (int)blockIdx.x * (256 >> sh) + (int)(threadIdx.x >> sh);
     const bool live = t < p.tokens;
     const T* row = static_cast<const T*>(p.gating) + (size_t)(live ? t : 0) * p.experts;
-    float sel_w[GATE_MAX_TOPK];
-    int sel_i[GATE_MAX_TOPK];
-    const float f = gate_row<T, VPT>(row, p.experts, p.topk, p.renorm != 0, L, gl, p.vec != 0, sel_w, sel_i);
-    if (live && gl == 0) {
+    float keep[GATE_KEEP];
+    const float f = gate_row<T, VPT>(row, p.experts, p.topk, p.renorm != 0, L, gl, p.vec != 0, keep, [&](int k, int index) {
+        if (live && gl == 0) {
+            p.indices[(size_t)t * p.topk + k] = index;
+            if (p.tei) p.tei[(size_t)t * p.topk + k] = k * p.tokens + t;
+        }
+    });
+    // lane k % L holds the weight of winner k
+    if (live) {
 #pragma unroll
-        for (int k = 0; k < GATE_MAX_TOPK; k++)
-            if (k < p.topk) {
-                p.weights[(size_t)t * p.topk + k] = sel_w[k] * f;
-                p.indices[(size_t)t * p.topk + k] = sel_i[k];
-                if (p.tei) p.tei[(size_t)t * p.topk + k] = k * p.tokens + t;
-            }
+        for (int j = 0; j < GATE_KEEP; j++) {
+            const int k = (j << sh) + gl;
+            if (k < p.topk) p.weights[(size_t)t * p.topk + k] = keep[j] * f;
+        }
     }
 }
 

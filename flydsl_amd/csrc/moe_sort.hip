@@ -175,22 +175,27 @@ __global__ void __launch_bounds__(SORT_THREADS) k_moe_gate_sort(MoeSortParams p,
         const int t = t0 + (int)(threadIdx.x >> sh);
         const bool live = t < p.tokens;
         const T* row = static_cast<const T*>(g.gating) + (size_t)(live ? t : 0) * p.experts;
-        float sel_w[GATE_MAX_TOPK];
-        int sel_i[GATE_MAX_TOPK];
-        const float f = gate_row<T, VPT>(row, p.experts, p.topk, g.renorm != 0, L, gl, g.vec != 0, sel_w, sel_i);
-        if (live && gl == 0) {
+        float keep[GATE_KEEP];
+        const float f = gate_row<T, VPT>(row, p.experts, p.topk, g.renorm != 0, L, gl, g.vec != 0, keep, [&](int k, int index) {
+            if (live && gl == 0) {
+                const int q = t * p.topk + k;
+                s_ids[q] = index;
+                if (e == 0) {
+                    if (g.indices) g.indices[q] = index;
+                    if (g.tei) g.tei[q] = k * p.tokens + t;
+                }
+            }
+        });
+        if (live) {
 #pragma unroll
-            for (int k = 0; k < GATE_MAX_TOPK; k++)
+            for (int j = 0; j < GATE_KEEP; j++) {
+                const int k = (j << sh) + gl;
                 if (k < p.topk) {
                     const int q = t * p.topk + k;
-                    s_ids[q] = sel_i[k];
-                    s_w[q] = sel_w[k] * f;
-                    if (e == 0) {
-                        if (g.weights) g.weights[q] = sel_w[k] * f;
-                        if (g.indices) g.indices[q] = sel_i[k];
-                        if (g.tei) g.tei[q] = k * p.tokens + t;
-                    }
+                    s_w[q] = keep[j] * f;
+                    if (e == 0 && g.weights) g.weights[q] = keep[j] * f;
                 }
+            }
         }
     }
     __syncthreads();
@@ -313,7 +318,11 @@ int psg_moe_sort_max_experts() { return SORT_MAX_EXPERTS; }
 
 // whether gating + sorting of this routing runs as one launch
 bool psg_moe_gate_sort_fuses(int tokens, int topk, int experts) {
-    return tokens <= FUSE_MAX_TOKENS && (int64_t)tokens * topk <= FUSE_MAX_PAIRS && experts <= GATE_MAX_EXPERTS && topk <= GATE_MAX_TOPK;
+    if (experts > GATE_MAX_EXPERTS || topk > GATE_MAX_TOPK || (int64_t)tokens * topk > FUSE_MAX_PAIRS) return false;
+    int vpt, lanes;
+    gate_layout(experts, &vpt, &lanes);
+    // one pass of the workgroup's 256 lanes over the tokens: a second pass costs more than the launch it saves
+    return tokens <= FUSE_MAX_TOKENS && tokens <= SORT_THREADS / lanes;
 }
 
 namespace {

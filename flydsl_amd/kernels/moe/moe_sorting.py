@@ -97,8 +97,8 @@ def moe_softmax_sort_flydsl(gating_logits, sorted_ids, sorted_weights, sorted_ex
                             dtype_str, unit_size=UNIT_SIZE, expert_mask=None, renormalize=True, num_local_tokens=None, *,
                             topk_ids=None, topk_weights=None, workspace=None, stream=None):
     """Router logits -> softmax -> top-k -> expert sort: the reference's fused entry point (moe_sorting_kernel.py:2250-2400),
-    same positional arguments and the same outputs as ``moe_sorting_flydsl``.  Up to 32 tokens this is ONE launch (every
-    sorting workgroup repeats the gating of all tokens in LDS; ``topk_ids`` / ``topk_weights`` are then optional extra
+    same positional arguments and the same outputs as ``moe_sorting_flydsl``.  For decode-sized batches (16 tokens with 256
+    experts, 32 with up to 128) this is ONE launch (every sorting workgroup repeats the gating of all tokens in LDS; ``topk_ids`` / ``topk_weights`` are then optional extra
     outputs); beyond that the gating kernel and the sorter run back to back, through ``topk_ids`` / ``topk_weights`` when the
     caller gives them (``[tokens, topk]`` int32 / fp32; needed under graph capture) and through fresh tensors otherwise."""
     from .topk_gating_softmax import gating_args

@@ -351,8 +351,9 @@ int psg_moe_topk_gating(const psg_moe_gating_args *args, void *stream);
 
 /* Gating followed by sorting: the reference's moe_softmax_sort_flydsl (kernels/moe/moe_sorting_kernel.py:2250-2400).
  * tokens / topk / experts of both structs must agree.  psg_moe_softmax_sorting_fused(tokens, topk, experts) = 1 says that
- * this routing runs as ONE launch (tokens <= 32 and tokens*topk <= 1024: every sorting workgroup repeats the gating of
- * all tokens into LDS; the reference fuses up to 16 tokens, :2313-2320): then sort->topk_ids / topk_weights are not
+ * this routing runs as ONE launch (tokens <= 32, tokens*topk <= 1024 and all tokens in one pass of a workgroup's 256
+ * lanes, i.e. tokens <= 256 / lanes-per-token: 16 tokens for 256 experts, 32 for up to 128; every sorting workgroup repeats
+ * the gating of all tokens into LDS; the reference fuses up to 16 tokens, :2313-2320): then sort->topk_ids / topk_weights are not
  * read, and gating->weights / indices / token_expert_indices are optional outputs (written when non-NULL).  Otherwise
  * the gating kernel runs first and the sorter reads its outputs: sort->topk_ids must be gating->indices and
  * sort->topk_weights gating->weights (both non-NULL). */

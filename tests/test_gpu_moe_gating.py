@@ -134,8 +134,8 @@ def test_graph_replays_equal_eager():
 
 
 @pytest.mark.parametrize("tokens,experts,topk,unit,dtype_str", [
-    (1, 256, 8, 32, "bf16"), (4, 8, 2, 16, "f32"), (16, 128, 6, 32, "bf16"), (32, 256, 8, 32, "f16"), (32, 64, 32, 16, "bf16"),  # one launch
-    (33, 256, 8, 32, "bf16"), (200, 128, 6, 64, "f16"), (1500, 32, 4, 32, "f32"),                                                 # two steps
+    (1, 256, 8, 32, "bf16"), (4, 8, 2, 16, "f32"), (16, 128, 6, 32, "bf16"), (16, 256, 8, 32, "f16"), (32, 64, 32, 16, "bf16"),  # one launch
+    (17, 256, 8, 32, "bf16"), (33, 128, 8, 32, "bf16"), (200, 128, 6, 64, "f16"), (1500, 32, 4, 32, "f32"),                                                 # two steps
 ])
 @pytest.mark.parametrize("masked", [False, True])
 def test_gating_plus_sorting_equals_the_two_steps(tokens, experts, topk, unit, dtype_str, masked):
