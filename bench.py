@@ -322,6 +322,23 @@ def run_next_row_workloads():
                     "weight_gb_per_s": experts * 2 * inter_dim * model_dim / s1 / 1e9})
         out.append({"workload": f"moe_fp8_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
                     "weight_gb_per_s": experts * model_dim * inter_dim / s2 / 1e9})
+        if tokens == 333:
+            continue
+        # the same two stages with int8 activations and packed int4 weights (W4A8): half the weight bytes
+        x8, sx8 = quant.pertoken_quant(torch.randn(tokens, model_dim, generator=g), quant_dtype=torch.int8)
+        a8, sa8 = quant.pertoken_quant(torch.randn(tokens * topk, inter_dim, generator=g), quant_dtype=torch.int8)
+        w1p = layout.pack_shuffled_int8_to_int4(layout.shuffle_weight(torch.randint(-8, 8, (experts * 2 * inter_dim, model_dim), generator=g, dtype=torch.int8)))
+        w2p = layout.pack_shuffled_int8_to_int4(layout.shuffle_weight(torch.randint(-8, 8, (experts * model_dim, inter_dim), generator=g, dtype=torch.int8)))
+        x8, a8, sx8, sa8, w1p, w2p = [t.to(dev).contiguous().view(-1) for t in (x8, a8, sx8, sa8, w1p, w2p)]
+        kw["in_dtype"] = "int4"
+        f1 = compile_moe_gemm1(doweight_stage1=False, out_dtype="bf16", **kw)
+        f2 = compile_moe_gemm2(doweight_stage2=True, out_dtype="bf16", accumulate=True, **kw)
+        s1 = timed(lambda: f1(out1, x8, w1p, sx8, sw1, sid, se, swt, nv, tokens, inter_dim, model_dim, blocks, None))
+        s2 = timed(lambda: f2(out2, a8, w2p, sa8, sw2, sid, se, swt, nv, tokens, model_dim, inter_dim, blocks, None))
+        out.append({"workload": f"moe_w4a8_stage1_{tag}", "us_per_launch_events": s1 * 1e6, "tflops": 2.0 * tokens * topk * 2 * inter_dim * model_dim / s1 / 1e12,
+                    "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s1 / 1e9})
+        out.append({"workload": f"moe_w4a8_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
+                    "weight_gb_per_s": experts * model_dim * inter_dim / 2 / s2 / 1e9})
     # the device-side expert sorter in front of the stages (outputs pre-allocated, accumulate buffer cleared by the same launch)
     for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)):
         g = torch.Generator().manual_seed(0)

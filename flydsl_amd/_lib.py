@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
 ABI_VERSION = 6
 
-IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3}
+IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3, "int4": 6}  # "int4": the MoE stages' int8 x packed-int4 weights
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
 EPILOGUE = {"none": 0, "bias": 1, "bias_relu": 2, "bias_silu": 3, "bias_gelu": 4}
 

@@ -1,4 +1,5 @@
-// MoE grouped GEMMs for gfx950 over expert-sorted token blocks, int8 or OCP fp8 operands with per-row fp32 scales.
+// MoE grouped GEMMs for gfx950 over expert-sorted token blocks, int8 or OCP fp8 operands with per-row fp32 scales, or int8
+// activations against packed int4 weights (W4A8).
 //
 // The sorted row list (one entry per routed (token, slot), padded per expert to whole blocks of BM rows) says which
 // row of x each tile row reads; one expert id per block says which slab of the preshuffled weights it multiplies.
@@ -10,6 +11,10 @@
 // XOR-swizzled LDS tile; W fragments go straight from the expert's slab into MFMA operand registers (lane l reads
 // bytes [16l, 16l+16) of a 1 KB block, the same wire format as the plain GEMM).  Stage 1 keeps two accumulators per
 // fragment (gate and up) so silu(g)*u happens in registers.
+// W4A8: the weights are the preshuffled int8 bytes with every 8 consecutive values v0..v7 packed into 4 bytes, byte j =
+// (v_j & 15) | (v_{j+4} << 4) (tests/kernels/test_moe_gemm_2stage.py:64-80 of the reference), so a lane's 16-byte piece
+// of a fragment is 8 bytes at half the offset; it is unpacked with the reference's sign-extending mask-and-multiply
+// (kernels/common/mma/mfma_preshuffle_pipeline.py:225-238) into the same int8 fragment and multiplied by the int8 MFMA.
 #include "psg_common.h"
 
 namespace {
@@ -25,6 +30,23 @@ template <>
 struct MoeAcc<KIND_INT8> {
     using type = v4i;
 };
+template <>
+struct MoeAcc<KIND_INT8W4> {
+    using type = v4i;
+};
+
+// 8 packed int4 (one dword) -> two dwords of int8: the low nibbles of the four bytes, then the high nibbles
+__device__ __forceinline__ void unpack_int4(int packed, int& even, int& odd) {
+    even = (packed & 0x0F0F0F0F) | ((packed & 0x08080808) * 0x1E);
+    const int t = (int)((unsigned)packed >> 4);
+    odd = (t & 0x0F0F0F0F) | ((t & 0x08080808) * 0x1E);
+}
+__device__ __forceinline__ v4i unpack_int4x16(v2i packed) {
+    int e0, o0, e1, o1;
+    unpack_int4(packed[0], e0, o0);
+    unpack_int4(packed[1], e1, o1);
+    return (v4i){e0, o0, e1, o1};
+}
 
 __device__ __forceinline__ int moe_lds_off(int row, int kc) { return row * 128 + ((kc ^ ((row >> 1) & 7)) << 4); }
 
@@ -36,6 +58,8 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     constexpr int BM = 16 * MR, TN = 64 * NR;
     constexpr int NSET = STAGE == 1 ? 2 : 1;           // gate and up
     constexpr int A_LOADS = (BM * 8 + 255) / 256;      // 16-byte chunks of the A tile per thread
+    constexpr bool W4 = KIND == KIND_INT8W4;           // packed int4 weights
+    constexpr int WSH = W4 ? 1 : 0;                    // weight byte offsets are halved
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * 128];
     __shared__ int ids[BM];
 
@@ -67,8 +91,8 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     const int rows_x = (STAGE == 1 && !p.x_slot_major) ? p.tokens : p.tokens * p.topk;
     const int rows_e = STAGE == 1 ? 2 * p.n_out : p.n_out;            // weight rows per expert
     __amdgpu_buffer_rsrc_t ra = make_rsrc(p.x, (uint64_t)rows_x * (uint64_t)K);
-    const uint8_t* w_e = p.w + (uint64_t)e * (uint64_t)rows_e * (uint64_t)K;
-    __amdgpu_buffer_rsrc_t rb = make_rsrc(w_e, (uint64_t)rows_e * (uint64_t)K);
+    const uint8_t* w_e = p.w + (((uint64_t)e * (uint64_t)rows_e * (uint64_t)K) >> WSH);
+    __amdgpu_buffer_rsrc_t rb = make_rsrc(w_e, ((uint64_t)rows_e * (uint64_t)K) >> WSH);
 
     uint32_t a_voff[A_LOADS];
     int a_ldsoff[A_LOADS];
@@ -88,7 +112,7 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
             const int n = n0 + (ni * 4 + wave) * 16;                  // first column of the block: the four wavefronts of pass ni
                                                                       // cover 64 consecutive columns
             const int nb = (n + s * p.n_out) >> 4;
-            b_voff[s][ni] = n < p.n_out ? (uint32_t)nb * 16u * (uint32_t)K + (uint32_t)lane * 16u : 0xFFFFFFF0u;
+            b_voff[s][ni] = n < p.n_out ? ((uint32_t)nb * 16u * (uint32_t)K + (uint32_t)lane * 16u) >> WSH : 0xFFFFFFF0u;
         }
 
     v4i areg[A_LOADS];
@@ -104,15 +128,21 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         for (int j = 0; j < A_LOADS; j++)
             if (a_ldsoff[j] >= 0) *reinterpret_cast<v4i*>(&lds[stage][a_ldsoff[j]]) = areg[j];
     };
-    v4i blo[2][NSET][NR], bhi[2][NSET][NR];
+    using wreg_t = typename std::conditional<W4, v2i, v4i>::type;  // a lane's piece of a W fragment as it is loaded
+    wreg_t blo[2][NSET][NR], bhi[2][NSET][NR];
     auto load_b = [&](int kt, int set) {
 #pragma unroll
         for (int s = 0; s < NSET; s++)
 #pragma unroll
             for (int ni = 0; ni < NR; ni++) {
                 const bool ok = kt < KT;
-                blo[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
-                bhi[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] + 1024u : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
+                if constexpr (W4) {
+                    blo[set][s][ni] = buf_load8(rb, ok ? b_voff[s][ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 1024u : 0u);
+                    bhi[set][s][ni] = buf_load8(rb, ok ? b_voff[s][ni] + 512u : 0xFFFFFFF0u, ok ? (uint32_t)kt * 1024u : 0u);
+                } else {
+                    blo[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
+                    bhi[set][s][ni] = buf_load16(rb, ok ? b_voff[s][ni] + 1024u : 0xFFFFFFF0u, ok ? (uint32_t)kt * 2048u : 0u);
+                }
             }
     };
 
@@ -128,6 +158,17 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         constexpr int S = decltype(SP)::value;
         load_a(kt + 1);
         load_b(kt + 1, S ^ 1);
+        // packed int4: this step's fragments unpacked once, in front of the row blocks that share them
+        v4i ulo[W4 ? NSET : 1][W4 ? NR : 1], uhi[W4 ? NSET : 1][W4 ? NR : 1];
+        if constexpr (W4) {
+#pragma unroll
+            for (int s = 0; s < NSET; s++)
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    ulo[s][ni] = unpack_int4x16(blo[S][s][ni]);
+                    uhi[s][ni] = unpack_int4x16(bhi[S][s][ni]);
+                }
+        }
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
             const int row = mi * 16 + li;
@@ -137,7 +178,10 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
                 constexpr int s = decltype(SI)::value;
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
-                    if constexpr (KIND == KIND_INT8) {
+                    if constexpr (W4) {
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ulo[s][ni], alo, acc[mi][s][ni], 0, 0, 0);
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(uhi[s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
+                    } else if constexpr (KIND == KIND_INT8) {
                         acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[S][s][ni], alo, acc[mi][s][ni], 0, 0, 0);
                         acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[S][s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
                     } else {
@@ -257,9 +301,10 @@ hipError_t launch_kind(const MoeParams& p, int block_m, int blocks, hipStream_t 
 
 }  // namespace
 
-// kind: KIND_INT8 / KIND_FP8; stage 1 or 2; block_m in {16, 32, 64, 128}; blocks = entries of expert_ids
+// kind: KIND_INT8 / KIND_FP8 / KIND_INT8W4; stage 1 or 2; block_m in {16, 32, 64, 128}; blocks = entries of expert_ids
 hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream) {
     if (kind == KIND_INT8) return stage == 1 ? launch_kind<KIND_INT8, 1>(p, block_m, blocks, stream) : launch_kind<KIND_INT8, 2>(p, block_m, blocks, stream);
+    if (kind == KIND_INT8W4) return stage == 1 ? launch_kind<KIND_INT8W4, 1>(p, block_m, blocks, stream) : launch_kind<KIND_INT8W4, 2>(p, block_m, blocks, stream);
     return stage == 1 ? launch_kind<KIND_FP8, 1>(p, block_m, blocks, stream) : launch_kind<KIND_FP8, 2>(p, block_m, blocks, stream);
 }
 

@@ -614,7 +614,8 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
         return fail(PSG_E_NULL, "out, x, w, scale_x, scale_w, sorted_token_ids, sorted_expert_ids, num_valid_ids must be non-NULL");
     if (a->doweight && !a->sorted_weights) return fail(PSG_E_NULL, "sorted_weights must be non-NULL when doweight is set");
     if (a->stage != 1 && a->stage != 2) return fail(PSG_E_SHAPE, "stage=%d must be 1 or 2", a->stage);
-    if (a->in_dtype != PSG_IN_INT8 && a->in_dtype != PSG_IN_FP8_E4M3FN) return fail(PSG_E_DTYPE, "in_dtype %d must be int8 or fp8", a->in_dtype);
+    if (a->in_dtype != PSG_IN_INT8 && a->in_dtype != PSG_IN_FP8_E4M3FN && a->in_dtype != PSG_IN_INT8_W4)
+        return fail(PSG_E_DTYPE, "in_dtype %d must be int8, fp8 or int8 with int4 weights", a->in_dtype);
     if (a->out_dtype < PSG_OUT_BF16 || a->out_dtype > PSG_OUT_F32) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
     if (a->out_dtype == PSG_OUT_F32 && !(a->stage == 2 && a->accumulate))
         return fail(PSG_E_DTYPE, "fp32 output exists only for stage 2 with accumulate (kernels/moe/moe_gemm_2stage/gemm2.py:629)");
@@ -655,7 +656,7 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     p.out_dtype = a->out_dtype;
     p.doweight = a->doweight ? 1 : 0;
     p.accumulate = a->stage == 2 && a->accumulate ? 1 : 0;
-    const hipError_t e = psg_launch_moe_gemm(p, a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : KIND_FP8, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
+    const hipError_t e = psg_launch_moe_gemm(p, a->in_dtype == PSG_IN_INT8 ? KIND_INT8 : a->in_dtype == PSG_IN_INT8_W4 ? KIND_INT8W4 : KIND_FP8, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_gemm launch");
     g_err[0] = 0;
     return 0;

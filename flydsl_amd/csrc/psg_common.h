@@ -12,7 +12,7 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3, KIND_MXFP4 = 4, KIND_MXFP8 = 5 };
+enum { KIND_INT8 = 0, KIND_FP8 = 1, KIND_FP16 = 2, KIND_BF16 = 3, KIND_MXFP4 = 4, KIND_MXFP8 = 5, KIND_INT8W4 = 6 };
 enum { OUT_BF16 = 0, OUT_FP16 = 1 };
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_RELU = 2, EPI_BIAS_SILU = 3, EPI_BIAS_GELU = 4 };
 // what a kernel writes: the scaled/activated C, or the raw accumulators
@@ -31,6 +31,10 @@ __device__ __forceinline__ v4i buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t vof
 // non-temporal variant for data that is streamed exactly once
 __device__ __forceinline__ v4i buf_load16_nt(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
     return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 2);
+}
+
+__device__ __forceinline__ v2i buf_load8(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return (v2i)__builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0);
 }
 
 __device__ __forceinline__ int buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
@@ -149,7 +153,8 @@ constexpr int OUT_F32 = 2;
 struct MoeParams {
     void* out;
     const uint8_t* x;           // stage 1: [tokens, K]; stage 2: [tokens*topk, K]
-    const uint8_t* w;           // preshuffled [experts * rows_per_expert, K] (rows_per_expert = 2*inter or model_dim)
+    const uint8_t* w;           // preshuffled [experts * rows_per_expert, K] (rows_per_expert = 2*inter or model_dim); K/2 bytes
+                                // per row for packed int4
     const float* sx;            // one scale per row of x
     const float* sw;            // [experts * rows_per_expert]
     const int32_t* sorted_ids;  // (slot << 24) | token per sorted row; padding rows hold token >= tokens

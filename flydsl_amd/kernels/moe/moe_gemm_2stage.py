@@ -8,7 +8,8 @@
 (gemm1.py:541-580 / launch_moe_gemm1 :502-537; gemm2.py:595-643; moe_reduce.py:164-203.)  ``x`` / ``w`` are fp8
 (e4m3fn) or int8 with one fp32 scale per row; ``w`` is ``shuffle_weight`` of the experts' weights stacked along the
 rows.  Built: ``in_dtype`` "fp8", "int8" and "int8smooth" (int8 whose stage-1 ``x`` / ``scale_x`` hold one row per (slot,
-token), gemm1.py:100-101,321-328; stage 2 is plain int8); "int4" raises ``NotImplementedError``.  ``tile_m`` is the
+token), gemm1.py:100-101,321-328; stage 2 is plain int8) and "int4" (W4A8: int8 ``x``, ``w`` =
+``flydsl_amd.layout.pack_shuffled_int8_to_int4(shuffle_weight(w_q))``, half the bytes; gemm1.py:41,170-189).  ``tile_m`` is the
 block size of the expert sorting and must be 16, 32, 64 or 128; ``tile_n`` / ``tile_k`` are checked with the reference's
 rules and then treated as hints.
 """
@@ -45,6 +46,7 @@ class MoeStage:
         self.experts, self.topk, self.tile_m = int(experts), int(topk), int(tile_m)
         self.doweight, self.accumulate = bool(doweight), bool(accumulate)
         self.slot_major = in_dtype == "int8smooth" and int(stage) == 1
+        self.w4 = in_dtype == "int4"
         self.out_dtype, self.in_dtype = _OUT[str(out_dtype).strip().lower()], _lib.IN_DTYPE["int8" if in_dtype == "int8smooth" else in_dtype]
         self._lib = _lib.lib()
 
@@ -60,7 +62,7 @@ class MoeStage:
         osize = 4 if self.out_dtype == 2 else 2
         dev = _lib.check_operand("out", out, min_elems=rows_out * n_out, elem_sizes=(osize,))
         _lib.check_operand("x", x, min_elems=rows_x * K, elem_sizes=(1,), device=dev)
-        _lib.check_operand("w", w, min_elems=rows_w * K, elem_sizes=(1,), device=dev)
+        _lib.check_operand("w", w, min_elems=rows_w * K // (2 if self.w4 else 1), elem_sizes=(1,), device=dev)
         _lib.check_operand("scale_x", scale_x, min_elems=rows_x, elem_sizes=(4,), device=dev)
         _lib.check_operand("scale_w", scale_w, min_elems=rows_w, elem_sizes=(4,), device=dev)
         _lib.check_operand("sorted_token_ids", sorted_token_ids, min_elems=1, elem_sizes=(4,), device=dev)
@@ -86,8 +88,6 @@ class MoeStage:
 def _check_in_dtype(in_dtype):
     if in_dtype not in ("fp8", "int8", "int8smooth", "int4"):
         raise ValueError(f"in_dtype must be 'fp8', 'int8', 'int8smooth', or 'int4', got {in_dtype!r}")
-    if in_dtype == "int4":
-        raise NotImplementedError("in_dtype='int4' (W4A8) is not built (fp8, int8 and int8smooth are)")
 
 
 def compile_moe_gemm1(*, model_dim: int, inter_dim: int, experts: int, topk: int, tile_m: int, tile_n: int, tile_k: int,

@@ -74,6 +74,21 @@ def shuffle_scale_w4(src: torch.Tensor, experts_cnt: int = 1, gate_up: bool = Fa
     return v.permute(0, 3, 5, 2, 4, 1).contiguous().reshape(r, kb)
 
 
+def pack_shuffled_int8_to_int4(x_shuf: torch.Tensor) -> torch.Tensor:
+    """Packed int4 weights of the W4A8 MoE stages from PRESHUFFLED int8 values in [-8, 7]: every 8 consecutive values
+    ``v0..v7`` become 4 bytes, ``byte j = (v_j & 15) | (v_{j+4} << 4)`` (low nibbles v0..v3, high nibbles v4..v7; the
+    reference's ``_pack_shuffled_int8_to_packed_int4``, tests/kernels/test_moe_gemm_2stage.py:64-80).  Returns int8 of half
+    the size, flat."""
+    if x_shuf.dtype != torch.int8 or x_shuf.numel() % 8:
+        raise ValueError("expected an int8 tensor whose size is a multiple of 8")
+    v = x_shuf.contiguous().view(-1, 2, 4)
+    if int(v.min()) < -8 or int(v.max()) > 7:
+        raise ValueError("int4 weights must lie in [-8, 7]")
+    lo = v[:, 0, :].to(torch.uint8) & 0xF
+    hi = (v[:, 1, :].to(torch.uint8) & 0xF) << 4
+    return (lo | hi).contiguous().view(-1).view(torch.int8)
+
+
 def preshuffle_b(b_t: torch.Tensor) -> torch.Tensor:
     """Permute row-major 1-byte ``B_T [N, K]`` into the preshuffled fragment layout, as the reference's helper of the
     row-scale fp8 GEMMs does (kernels/gemm/fp8_gemm_utils.py:24-28): blocks ``[N/16][K/64][4][16][16 B]``, i.e. the

@@ -45,7 +45,8 @@ extern "C" {
 #define PSG_ABI_VERSION 6
 
 /* input element types of A and B */
-enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3 };
+enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3,
+                    PSG_IN_INT8_W4 = 6 /* psg_moe_gemm only: int8 activations, packed int4 weights */ };
 /* output element types of C */
 enum psg_out_dtype { PSG_OUT_BF16 = 0, PSG_OUT_FP16 = 1, PSG_OUT_F32 = 2 /* psg_moe_gemm stage 2 with accumulate only */ };
 /* fused epilogue, as the reference's `epilogue` keyword (kernels/gemm/preshuffle_gemm.py:118) */
@@ -265,7 +266,9 @@ typedef struct psg_moe_args {
     int32_t sorted_size; /* entries of sorted_token_ids / sorted_weights */
     int32_t blocks;      /* entries of sorted_expert_ids = grid size along the sorted rows */
     int32_t block_m;
-    int32_t in_dtype;    /* PSG_IN_INT8 or PSG_IN_FP8_E4M3FN */
+    int32_t in_dtype;    /* PSG_IN_INT8, PSG_IN_FP8_E4M3FN, or PSG_IN_INT8_W4: x int8 and w the preshuffled int8 bytes (values in
+                            [-8, 7]) with every 8 consecutive values v0..v7 packed into 4 bytes, byte j = (v_j & 15) | (v_{j+4} << 4)
+                            (W4A8; tests/kernels/test_moe_gemm_2stage.py:64-80, kernels/moe/moe_gemm_2stage/layout_helpers.py:146-189) */
     int32_t out_dtype;   /* enum psg_out_dtype */
     int32_t stage;       /* 1 or 2 */
     int32_t doweight;

@@ -280,6 +280,75 @@ def test_stage1_int8smooth_slot_major_rows(out_dtype, tile_m, tokens):
     assert e2.slot_major is False
 
 
+def _w4a8(stage, tokens, tile_m, out_dtype, swap_nibbles=False, accumulate=True, seed=0):
+    """One W4A8 stage (int8 activations x packed int4 weights) and its oracle result; the weights are drawn from randn so that
+    all of [-8, 7] occurs, as in the reference's tests (tests/kernels/test_moe_gemm_2stage.py:292-303)."""
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+
+    model_dim, inter_dim, experts, topk = 256, 128, 4, 2
+    g = torch.Generator().manual_seed(seed + 300)
+    ids, wts, routing = _routing(tokens, experts, topk, tile_m, seed)
+    if stage == 1:
+        x = torch.randn(tokens, model_dim, generator=g)
+        w = torch.randn(experts, 2 * inter_dim, model_dim, generator=g)
+        K, rows_e = model_dim, 2 * inter_dim
+    else:
+        x = torch.randn(tokens, topk, inter_dim, generator=g)
+        w = torch.randn(experts, model_dim, inter_dim, generator=g)
+        K, rows_e = inter_dim, model_dim
+    xq, sx = quant.pertoken_quant(x, quant_dtype=torch.int8)
+    wq, sw = quant.pertoken_quant(w, quant_dtype=torch.int8, dtypeMax=7)
+    assert int(wq.min()) >= -8 and int(wq.max()) <= 7 and int(wq.min()) <= -7
+    packed = layout.pack_shuffled_int8_to_int4(layout.shuffle_weight(wq).view(experts * rows_e, K).contiguous())
+    assert packed.numel() == experts * rows_e * K // 2
+    if swap_nibbles:
+        b = packed.view(torch.uint8)
+        packed = (((b & 0xF) << 4) | (b >> 4)).view(torch.int8)
+    if stage == 1:
+        out = torch.full((tokens, topk, inter_dim), float("nan"), dtype=TDT[out_dtype], device="cuda")
+        exe = compile_moe_gemm1(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128,
+                                doweight_stage1=False, out_dtype=out_dtype, in_dtype="int4")
+        _launch(exe, out, xq, packed, sx, sw.view(-1, 1), routing, inter_dim, model_dim, tokens)
+        ref = O.moe_gemm1(xq.view(torch.uint8).numpy(), wq.view(torch.uint8).numpy().reshape(-1, K), sx.numpy(), sw.numpy().reshape(-1),
+                          ids.numpy(), wts.numpy(), inter_dim, False, "int8")
+    else:
+        rows = tokens if accumulate else tokens * topk
+        out = torch.zeros(rows, model_dim, dtype=TDT[out_dtype], device="cuda")
+        exe = compile_moe_gemm2(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128,
+                                doweight_stage2=True, out_dtype=out_dtype, accumulate=accumulate, in_dtype="int4")
+        _launch(exe, out, xq, packed, sx, sw.view(-1, 1), routing, model_dim, inter_dim, tokens)
+        ref = O.moe_gemm2(xq.view(torch.uint8).numpy(), wq.view(torch.uint8).numpy().reshape(-1, K), sx.numpy().reshape(-1), sw.numpy().reshape(-1),
+                          ids.numpy(), wts.numpy(), model_dim, True, "int8", reduce_slots=accumulate).reshape(rows, model_dim)
+    return out.float().cpu().numpy(), ref
+
+
+@pytest.mark.parametrize("stage", [1, 2])
+@pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile_m,tokens", [(16, 8), (32, 100), (64, 128), (128, 333)])
+def test_w4a8_stages_match_the_int8_oracle_on_the_unpacked_weights(stage, out_dtype, tile_m, tokens):
+    # the reference's numeric cases with in_dtype="int4" (tests/kernels/test_moe_gemm_2stage.py:382-408,608-642)
+    got, ref = _w4a8(stage, tokens, tile_m, out_dtype, seed=tokens)
+    assert _cos(got, ref) > 0.99
+    tol = 1e-2 if stage == 1 else 2e-2  # stage 2 adds topk rounded 16-bit contributions per output
+    ok, ratio = O.within_north_star_tolerance(got, ref, tol)
+    assert ok, f"outside tolerance ({ratio:.3f})"
+
+
+def test_w4a8_per_slot_stage2():
+    got, ref = _w4a8(2, 70, 32, "bf16", accumulate=False)
+    ok, ratio = O.within_north_star_tolerance(got, ref, 1e-2)
+    assert ok and _cos(got, ref) > 0.999, ratio
+
+
+@pytest.mark.parametrize("stage", [1, 2])
+def test_w4a8_nibble_order_matters(stage):
+    # swapping the two nibbles of every packed byte must wreck the result: guards the v_j | v_{j+4} << 4 packing the kernel's
+    # unpack assumes (the reference's test_moe_gemm1_int4_perturb / test_moe_gemm2_int4_perturb, :411-478,:645-700)
+    good, ref = _w4a8(stage, 64, 32, "bf16")
+    bad, _ = _w4a8(stage, 64, 32, "bf16", swap_nibbles=True)
+    assert _cos(good, ref) > 0.99 and _cos(bad, ref) < 0.9
+
+
 def test_expert_parallel_chain_sorter_mask_stage2_masked_reduction():
     # one rank of an expert-parallel layout: 8 experts, 5 of them local.  The device sorter drops the routed pairs of the other
     # three and numbers the local experts densely, stage 2 runs on the local weights only and leaves the other slots' rows
@@ -340,8 +409,6 @@ def test_moe_argument_errors():
         compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=64, doweight_stage1=False)
     with pytest.raises(AssertionError):  # model_dim must be an EVEN multiple of tile_k in stage 1
         compile_moe_gemm1(model_dim=384, inter_dim=128, experts=4, topk=2, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False)
-    with pytest.raises(NotImplementedError):
-        compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, in_dtype="int4")
     with pytest.raises(ValueError):
         compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False, in_dtype="int2")
     with pytest.raises(ValueError):

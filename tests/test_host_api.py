@@ -148,7 +148,7 @@ def test_moe_c_abi_validation_codes():
         setattr(m, f, 0x1000)
     m.tokens, m.topk, m.experts, m.model_dim, m.inter_dim = 8, 2, 4, 256, 128
     m.sorted_size, m.blocks, m.block_m, m.in_dtype, m.out_dtype, m.stage = 76, 5, 16, 1, 0, 1
-    for field, val, code, word in (("stage", 3, -2, b"stage"), ("in_dtype", 2, -3, b"in_dtype"), ("out_dtype", 2, -3, b"fp32 output"),
+    for field, val, code, word in (("stage", 3, -2, b"stage"), ("in_dtype", 2, -3, b"in_dtype"), ("in_dtype", 5, -3, b"in_dtype"), ("out_dtype", 2, -3, b"fp32 output"),
                                    ("block_m", 48, -2, b"block_m"), ("model_dim", 192, -2, b"K=192"), ("inter_dim", 24, -2, b"output width"),
                                    ("tokens", 1 << 24, -2, b"tokens"), ("blocks", 0, -2, b"blocks"), ("x", 0x1004, -6, b"aligned"), ("x_slot_major", 2, -2, b"x_slot_major")):
         old = getattr(m, field)
@@ -341,6 +341,31 @@ def test_rowscale_fp8_entry_points_keep_the_reference_assertions():
     # preshuffle_b is the byte map of shuffle_weight for 1-byte elements
     w = torch.arange(64 * 256, dtype=torch.int32).remainder(251).to(torch.uint8).reshape(64, 256)
     assert torch.equal(preshuffle_b(w).reshape(64, 256), layout.shuffle_weight(w).reshape(64, 256))
+
+
+def test_int4_packing_against_a_scalar_loop():
+    # byte j of every group of 8 values v0..v7 is (v_j & 15) | (v_{j+4} << 4)
+    g = torch.Generator().manual_seed(4)
+    v = torch.randint(-8, 8, (6, 16), generator=g, dtype=torch.int8)
+    got = layout.pack_shuffled_int8_to_int4(v).view(torch.uint8).tolist()
+    flat = v.view(-1).tolist()
+    want = []
+    for base in range(0, len(flat), 8):
+        for j in range(4):
+            want.append((flat[base + j] & 15) | ((flat[base + j + 4] & 15) << 4))
+    assert got == want
+    # and back: low nibbles are v0..v3, high nibbles v4..v7, two's complement
+    back = []
+    for base in range(0, len(got), 4):
+        for shift in (0, 4):
+            for j in range(4):
+                n = (got[base + j] >> shift) & 15
+                back.append(n - 16 if n >= 8 else n)
+    assert back == flat
+    with pytest.raises(ValueError):
+        layout.pack_shuffled_int8_to_int4(torch.full((8,), 9, dtype=torch.int8))
+    with pytest.raises(ValueError):
+        layout.pack_shuffled_int8_to_int4(torch.zeros(12, dtype=torch.int8))
 
 
 def test_struct_layouts_match_header():
