@@ -130,6 +130,8 @@ class MoeArgs(ctypes.Structure):
         ("doweight", ctypes.c_int32),
         ("accumulate", ctypes.c_int32),
         ("x_slot_major", ctypes.c_int32),
+        ("no_pairing", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
     ]
 
 

@@ -52,10 +52,15 @@ __device__ __forceinline__ int moe_lds_off(int row, int kc) { return row * 128 +
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
-template <int KIND, int MR, int NR, int STAGE>
+// CO = 2: the workgroup's BM rows are TWO consecutive blocks of the sorted list when both belong to the same expert (blocks
+// of 16 or 32 rows: an expert with 17 to 32 routed rows would otherwise stream its weights once per block).  Blocks pair up
+// from the start of each run of equal expert ids: the workgroup of the second block of a pair ends at once, and the
+// first one treats the second half of its tile as padding when the run ends there.
+template <int KIND, int MR, int NR, int STAGE, int CO = 1>
 __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     using acc_t = typename MoeAcc<KIND>::type;
     constexpr int BM = 16 * MR, TN = 64 * NR;
+    constexpr int BLK = BM / CO;                        // rows of one block of the sorted list
     constexpr int NSET = STAGE == 1 ? 2 : 1;           // gate and up
     constexpr int A_LOADS = (BM * 8 + 255) / 256;      // 16-byte chunks of the A tile per thread
     constexpr bool W4 = KIND == KIND_INT8W4;           // packed int4 weights
@@ -68,13 +73,29 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     const int lane = tid & 63, li = lane & 15, lg = lane >> 4;
     const int blk = (int)blockIdx.y;
     const int n0 = (int)blockIdx.x * TN;
-    if (blk * BM >= p.num_valid[0]) return;            // uniform: blocks past the sorted rows in use
+    const int used = p.num_valid[0];
+    if (blk * BLK >= used) return;                     // uniform: blocks past the sorted rows in use
     const int e = p.expert_ids[blk];
     if (e < 0 || e >= p.experts) return;               // uniform: a block without an expert
+    int rows_live = BLK;                               // rows of the tile that belong to this workgroup's expert
+    if constexpr (CO == 2) {
+        // position of this block in its run of equal expert ids: 64 earlier ids at a time, one per lane
+        int before = 0;
+        for (int base = blk - 1; base >= 0; base -= 64) {
+            const int j = base - lane;
+            const unsigned long long same = __ballot(j >= 0 && p.expert_ids[j] == e);
+            const int run = same == ~0ull ? 64 : __builtin_ctzll(~same);
+            before += run;
+            if (run < 64) break;
+        }
+        before = __builtin_amdgcn_readfirstlane(before);
+        if (before & 1) return;                        // uniform: the second block of a pair
+        if ((blk + 1) * BLK < used && p.expert_ids[blk + 1] == e) rows_live = BM;
+    }
 
     if (tid < BM) {
-        const int q = blk * BM + tid;
-        ids[tid] = q < p.sorted_size ? p.sorted_ids[q] : p.tokens;  // past the list = a padding row
+        const int q = blk * BLK + tid;
+        ids[tid] = (tid < rows_live && q < p.sorted_size) ? p.sorted_ids[q] : p.tokens;  // past the list or the pair = a padding row
     }
     __syncthreads();
 
@@ -227,7 +248,7 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
             const int r = mi * 16 + li;
             const int xr = x_row(r);
             const float sx = xr >= 0 ? p.sx[xr] : 0.f;
-            const float rw = (p.doweight && xr >= 0) ? p.sorted_w[blk * BM + r] : 1.0f;
+            const float rw = (p.doweight && xr >= 0) ? p.sorted_w[blk * BLK + r] : 1.0f;
             v4f y;
             if constexpr (STAGE == 1) {
                 const acc_t ag = acc[mi][0][ni], au = acc[mi][NSET - 1][ni];
@@ -278,25 +299,35 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
 }
 
 template <int KIND, int STAGE, int NR>
-hipError_t launch_nr(const MoeParams& p, int block_m, int blocks, hipStream_t stream) {
+hipError_t launch_nr(const MoeParams& p, int block_m, int blocks, bool pair, hipStream_t stream) {
     const dim3 grid((p.n_out + 64 * NR - 1) / (64 * NR), blocks, 1);
-#define PSG_MOE(MR_)                                                                                \
-    if (block_m == 16 * MR_) {                                                                      \
-        hipLaunchKernelGGL((k_moe_gemm<KIND, MR_, NR, STAGE>), grid, dim3(256), 0, stream, p);     \
-        return hipGetLastError();                                                                   \
+#define PSG_MOE(MR_, CO_)                                                                                \
+    {                                                                                                    \
+        hipLaunchKernelGGL((k_moe_gemm<KIND, MR_, NR, STAGE, CO_>), grid, dim3(256), 0, stream, p);     \
+        return hipGetLastError();                                                                        \
     }
-    PSG_MOE(1) PSG_MOE(2) PSG_MOE(4) PSG_MOE(8)
+    if (pair && block_m == 16) PSG_MOE(2, 2)
+    if (pair && block_m == 32) PSG_MOE(4, 2)
+    if (block_m == 16) PSG_MOE(1, 1)
+    if (block_m == 32) PSG_MOE(2, 1)
+    if (block_m == 64) PSG_MOE(4, 1)
+    if (block_m == 128) PSG_MOE(8, 1)
 #undef PSG_MOE
     return hipErrorInvalidValue;
 }
 
 template <int KIND, int STAGE>
 hipError_t launch_kind(const MoeParams& p, int block_m, int blocks, hipStream_t stream) {
-    // 128 columns per workgroup when they divide the output; stage 1 (two accumulator sets) only for blocks of up to 32
+    // Stage 1 with one-byte weights multiplies blocks of 16 and 32 rows two at a time where they share an expert (64 tokens x
+    // top-8 on 32 experts, blocks of 16: 107 -> 92 us).  Measured and left alone: stage 2 (34 -> 37 us: its second pass over an
+    // expert's smaller slab already hits in L2, and pairing halves the workgroups in flight) and packed int4 weights (49 -> 50).
+    const bool pair = block_m <= 32 && p.pair_blocks != 0 && STAGE == 1 && KIND != KIND_INT8W4;
+    const int tile_m = pair ? 2 * block_m : block_m;
+    // 128 columns per workgroup when they divide the output; stage 1 (two accumulator sets) only for tiles of up to 32
     // rows: measured at 4096 tokens x top-8, blocks of 128: stage 1 488 us with 64 columns against 800 with 128, stage 2
     // 442 against 412
-    if (p.n_out % 128 == 0 && (STAGE == 2 || block_m <= 32)) return launch_nr<KIND, STAGE, 2>(p, block_m, blocks, stream);
-    return launch_nr<KIND, STAGE, 1>(p, block_m, blocks, stream);
+    if (p.n_out % 128 == 0 && (STAGE == 2 || tile_m <= 32)) return launch_nr<KIND, STAGE, 2>(p, block_m, blocks, pair, stream);
+    return launch_nr<KIND, STAGE, 1>(p, block_m, blocks, pair, stream);
 }
 
 }  // namespace

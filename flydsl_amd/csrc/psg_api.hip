@@ -621,6 +621,7 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
         return fail(PSG_E_DTYPE, "fp32 output exists only for stage 2 with accumulate (kernels/moe/moe_gemm_2stage/gemm2.py:629)");
     if (a->x_slot_major != 0 && !(a->x_slot_major == 1 && a->stage == 1))
         return fail(PSG_E_SHAPE, "x_slot_major=%d must be 0, or 1 for stage 1", a->x_slot_major);
+    if ((a->no_pairing != 0 && a->no_pairing != 1) || a->pad0 != 0) return fail(PSG_E_SHAPE, "no_pairing must be 0 or 1 and pad0 0");
     if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
     if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
     if (a->experts < 1) return fail(PSG_E_SHAPE, "experts=%d must be positive", a->experts);
@@ -647,6 +648,7 @@ int psg_moe_gemm(const psg_moe_args* a, void* stream) {
     p.sorted_w = a->sorted_weights;
     p.num_valid = a->num_valid_ids;
     p.x_slot_major = a->x_slot_major;
+    p.pair_blocks = a->no_pairing ? 0 : 1;
     p.tokens = a->tokens;
     p.topk = a->topk;
     p.experts = a->experts;

@@ -169,6 +169,7 @@ struct MoeParams {
     int doweight;               // multiply by the routing weight in this stage
     int accumulate;             // stage 2: atomic add into out[token] (else one row per (token, slot))
     int x_slot_major;           // stage 1: x / sx hold one row per (slot, token) at slot*tokens + token
+    int pair_blocks;            // blocks of 16 / 32 rows: multiply two consecutive blocks of one expert in one workgroup
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).

@@ -47,6 +47,7 @@ class MoeStage:
         self.doweight, self.accumulate = bool(doweight), bool(accumulate)
         self.slot_major = in_dtype == "int8smooth" and int(stage) == 1
         self.w4 = in_dtype == "int4"
+        self.no_pairing = False  # True: one workgroup per block of the sorted list even for blocks of 16 / 32 rows (tests)
         self.out_dtype, self.in_dtype = _OUT[str(out_dtype).strip().lower()], _lib.IN_DTYPE["int8" if in_dtype == "int8smooth" else in_dtype]
         self._lib = _lib.lib()
 
@@ -80,6 +81,7 @@ class MoeStage:
         a.in_dtype, a.out_dtype, a.stage = self.in_dtype, self.out_dtype, self.stage
         a.doweight, a.accumulate = int(self.doweight), int(self.accumulate)
         a.x_slot_major = int(self.slot_major)
+        a.no_pairing = int(self.no_pairing)
         rc = self._lib.psg_moe_gemm(ctypes.byref(a), _lib.stream_handle(stream))
         if rc:
             _lib.check(rc, "psg_moe_gemm")

@@ -275,6 +275,10 @@ typedef struct psg_moe_args {
     int32_t accumulate;  /* stage 2 only */
     int32_t x_slot_major; /* stage 1 only: 1 = x and scale_x hold one row per (slot, token), row slot*tokens + token (the
                              reference's int8smooth inputs, kernels/moe/moe_gemm_2stage/gemm1.py:100-101,321-328); 0 = one row per token */
+    int32_t no_pairing;  /* 0: in stage 1 with one-byte weights and block_m 16 or 32, two consecutive blocks of the same expert are multiplied by one workgroup,
+                            so that an expert with up to 2*block_m routed rows streams its weights once (same results: the
+                            rows of a block never mix); 1: every block gets its own workgroup (tests, tuning) */
+    int32_t pad0;        /* 0 */
 } psg_moe_args;
 
 int psg_moe_gemm(const psg_moe_args *args, void *stream);

@@ -280,6 +280,52 @@ def test_stage1_int8smooth_slot_major_rows(out_dtype, tile_m, tokens):
     assert e2.slot_major is False
 
 
+@pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
+@pytest.mark.parametrize("tile_m,tokens", [(16, 8), (16, 64), (16, 200), (32, 40), (32, 333)])
+def test_paired_blocks_give_the_same_bits_as_single_blocks(in_dtype, tile_m, tokens):
+    # with blocks of 16 / 32 rows a workgroup multiplies two consecutive blocks of one expert; rows never mix, so every output
+    # must be bit-identical to the launch with one workgroup per block.  Skewed routing: experts with 0, 1, 2, 3 and more blocks.
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+
+    model_dim, inter_dim, experts, topk = 256, 128, 8, 2
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(tokens)
+    score = torch.rand(tokens, experts, generator=g) + torch.tensor([1.5, 0.8, 0.4, 0.2, 0.1, 0.0, 0.0, -5.0])
+    vals, ids = torch.topk(score, k=topk, dim=1)
+    wts = torch.softmax(vals, dim=1).float()
+    sid, sw, se, npp = moe_sorting(ids.int(), wts, num_experts=experts, block_size=tile_m)
+    used = int(npp[0]) // tile_m
+    runs = np.bincount(se[:used].numpy(), minlength=experts)
+    assert tokens < 20 or (runs.max() >= 2 and (tokens < 64 or (runs % 2 == 1).any()))  # pairs and an odd run
+    routing = (sid, sw, se, npp[:1].contiguous(), int(se.numel()))
+    x = torch.randn(tokens, model_dim, generator=g)
+    w1 = torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim)
+    xq, sx = quant.pertoken_quant(x, quant_dtype=QDT[in_dtype])
+    w1q, sw1 = quant.pertoken_quant(w1, quant_dtype=QDT[in_dtype])
+    w1s = layout.shuffle_weight(w1q).view(-1, model_dim).contiguous()
+    a2 = torch.randn(tokens, topk, inter_dim, generator=g)
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    a2q, sa2 = quant.pertoken_quant(a2, quant_dtype=QDT[in_dtype])
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=QDT[in_dtype])
+    w2s = layout.shuffle_weight(w2q).view(-1, inter_dim).contiguous()
+    kw = dict(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128, out_dtype="bf16", in_dtype=in_dtype)
+    outs = {}
+    for single in (False, True):
+        e1 = compile_moe_gemm1(doweight_stage1=True, **kw)
+        e2 = compile_moe_gemm2(doweight_stage2=True, accumulate=False, **kw)
+        e1.no_pairing = e2.no_pairing = single
+        o1 = torch.full((tokens, topk, inter_dim), float("nan"), dtype=torch.bfloat16, device=dev)
+        o2 = torch.full((tokens * topk, model_dim), float("nan"), dtype=torch.bfloat16, device=dev)
+        _launch(e1, o1, xq, w1s, sx, sw1.view(-1, 1), routing, inter_dim, model_dim, tokens)
+        _launch(e2, o2, a2q, w2s, sa2, sw2.view(-1, 1), routing, model_dim, inter_dim, tokens)
+        outs[single] = (o1.view(torch.int16).cpu(), o2.view(torch.int16).cpu())
+    assert torch.equal(outs[False][0], outs[True][0]) and torch.equal(outs[False][1], outs[True][1])
+    ref = O.moe_gemm1(xq.view(torch.uint8).numpy(), w1q.view(torch.uint8).numpy().reshape(-1, model_dim), sx.numpy(), sw1.numpy().reshape(-1),
+                      ids.int().numpy(), wts.numpy(), inter_dim, True, in_dtype)
+    ok, ratio = O.within_north_star_tolerance(outs[False][0].view(torch.bfloat16).float().numpy(), ref, 1e-2)
+    assert ok, ratio
+
+
 def _w4a8(stage, tokens, tile_m, out_dtype, swap_nibbles=False, accumulate=True, seed=0):
     """One W4A8 stage (int8 activations x packed int4 weights) and its oracle result; the weights are drawn from randn so that
     all of [-8, 7] occurs, as in the reference's tests (tests/kernels/test_moe_gemm_2stage.py:292-303)."""

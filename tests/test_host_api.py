@@ -150,7 +150,8 @@ def test_moe_c_abi_validation_codes():
     m.sorted_size, m.blocks, m.block_m, m.in_dtype, m.out_dtype, m.stage = 76, 5, 16, 1, 0, 1
     for field, val, code, word in (("stage", 3, -2, b"stage"), ("in_dtype", 2, -3, b"in_dtype"), ("in_dtype", 5, -3, b"in_dtype"), ("out_dtype", 2, -3, b"fp32 output"),
                                    ("block_m", 48, -2, b"block_m"), ("model_dim", 192, -2, b"K=192"), ("inter_dim", 24, -2, b"output width"),
-                                   ("tokens", 1 << 24, -2, b"tokens"), ("blocks", 0, -2, b"blocks"), ("x", 0x1004, -6, b"aligned"), ("x_slot_major", 2, -2, b"x_slot_major")):
+                                   ("tokens", 1 << 24, -2, b"tokens"), ("blocks", 0, -2, b"blocks"), ("x", 0x1004, -6, b"aligned"), ("x_slot_major", 2, -2, b"x_slot_major"), ("no_pairing", 2, -2, b"no_pairing"),
+                                   ("pad0", 1, -2, b"pad0")):
         old = getattr(m, field)
         setattr(m, field, val)
         assert handle.psg_moe_gemm(ctypes.byref(m), None) == code, field
