@@ -150,7 +150,12 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
             if (a_ldsoff[j] >= 0) *reinterpret_cast<v4i*>(&lds[stage][a_ldsoff[j]]) = areg[j];
     };
     using wreg_t = typename std::conditional<W4, v2i, v4i>::type;  // a lane's piece of a W fragment as it is loaded
-    wreg_t blo[2][NSET][NR], bhi[2][NSET][NR];
+    // W register sets: the fragments of step kt live in set kt % NWS and are requested WPF steps ahead.  Stage-1 tiles of up
+    // to 32 rows (decode) are bound by the bytes of W a workgroup keeps in flight (64 tokens x top-8 on 32 experts: 86 -> 80 us
+    // with three steps ahead); stage 2 (34 -> 36 us) and packed int4 weights (36 -> 38) are not and stay one step ahead
+    constexpr int WPF = (MR <= 2 && STAGE == 1 && !W4) ? 3 : 1;
+    constexpr int NWS = WPF + 1;
+    wreg_t blo[NWS][NSET][NR], bhi[NWS][NSET][NR];
     auto load_b = [&](int kt, int set) {
 #pragma unroll
         for (int s = 0; s < NSET; s++)
@@ -175,10 +180,11 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
 #pragma unroll
             for (int ni = 0; ni < NR; ni++) acc[mi][s][ni] = (acc_t){0, 0, 0, 0};
 
-    auto step = [&](int kt, auto SP) __attribute__((always_inline)) {
-        constexpr int S = decltype(SP)::value;
+    auto step = [&](int kt, auto SP, auto WP) __attribute__((always_inline)) {
+        constexpr int S = decltype(SP)::value;    // LDS stage of this step's A tile
+        constexpr int WS = decltype(WP)::value;   // register set of this step's W fragments
         load_a(kt + 1);
-        load_b(kt + 1, S ^ 1);
+        load_b(kt + WPF, (WS + WPF) % NWS);
         // packed int4: this step's fragments unpacked once, in front of the row blocks that share them
         v4i ulo[W4 ? NSET : 1][W4 ? NR : 1], uhi[W4 ? NSET : 1][W4 ? NR : 1];
         if constexpr (W4) {
@@ -186,8 +192,8 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
             for (int s = 0; s < NSET; s++)
 #pragma unroll
                 for (int ni = 0; ni < NR; ni++) {
-                    ulo[s][ni] = unpack_int4x16(blo[S][s][ni]);
-                    uhi[s][ni] = unpack_int4x16(bhi[S][s][ni]);
+                    ulo[s][ni] = unpack_int4x16(blo[WS][s][ni]);
+                    uhi[s][ni] = unpack_int4x16(bhi[WS][s][ni]);
                 }
         }
         static_for<MR>([&](auto MI) {
@@ -203,10 +209,10 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
                         acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ulo[s][ni], alo, acc[mi][s][ni], 0, 0, 0);
                         acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(uhi[s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
                     } else if constexpr (KIND == KIND_INT8) {
-                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[S][s][ni], alo, acc[mi][s][ni], 0, 0, 0);
-                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[S][s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(blo[WS][s][ni], alo, acc[mi][s][ni], 0, 0, 0);
+                        acc[mi][s][ni] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bhi[WS][s][ni], ahi, acc[mi][s][ni], 0, 0, 0);
                     } else {
-                        const v8i w8 = __builtin_shufflevector(blo[S][s][ni], bhi[S][s][ni], 0, 1, 2, 3, 4, 5, 6, 7);
+                        const v8i w8 = __builtin_shufflevector(blo[WS][s][ni], bhi[WS][s][ni], 0, 1, 2, 3, 4, 5, 6, 7);
                         const v8i a8 = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
                         acc[mi][s][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w8, a8, acc[mi][s][ni], 0, 0, 0, 0, 0, 0);
                     }
@@ -218,12 +224,16 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     };
 
     load_a(0);
-    load_b(0, 0);
+    static_for<WPF>([&](auto I) { load_b(decltype(I)::value, decltype(I)::value); });
     store_a(0);
     __syncthreads();
-    for (int kt = 0; kt < KT; kt += 2) {
-        step(kt, std::integral_constant<int, 0>{});
-        if (kt + 1 < KT) step(kt + 1, std::integral_constant<int, 1>{});
+    // unrolled over lcm(2 LDS stages, NWS register sets) steps so that both indices are compile-time
+    constexpr int UN = NWS % 2 == 0 ? NWS : 2 * NWS;
+    for (int kt0 = 0; kt0 < KT; kt0 += UN) {
+        static_for<UN>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if (kt0 + i < KT) step(kt0 + i, std::integral_constant<int, i & 1>{}, std::integral_constant<int, i % NWS>{});
+        });
     }
 
     // Epilogue, one pass per ni (64 consecutive columns of the tile): every lane finishes its own fragments (rows
@@ -326,7 +336,11 @@ hipError_t launch_kind(const MoeParams& p, int block_m, int blocks, hipStream_t 
     // 128 columns per workgroup when they divide the output; stage 1 (two accumulator sets) only for tiles of up to 32
     // rows: measured at 4096 tokens x top-8, blocks of 128: stage 1 488 us with 64 columns against 800 with 128, stage 2
     // 442 against 412
-    if (p.n_out % 128 == 0 && (STAGE == 2 || tile_m <= 32)) return launch_nr<KIND, STAGE, 2>(p, block_m, blocks, pair, stream);
+    // ... and only when that still leaves several workgroups per CU: a workgroup streams its slab at the pace its loads in
+    // flight allow, so a decode-sized stage 1 (64 tokens x top-8 on 32 experts: at most 63 blocks x 12 column tiles) is faster
+    // with twice as many workgroups of half the width
+    const long wgs128 = (long)blocks / (pair ? 2 : 1) * (long)(p.n_out / 128);
+    if (p.n_out % 128 == 0 && (STAGE == 2 || (tile_m <= 32 && wgs128 >= 1024))) return launch_nr<KIND, STAGE, 2>(p, block_m, blocks, pair, stream);
     return launch_nr<KIND, STAGE, 1>(p, block_m, blocks, pair, stream);
 }
 
