@@ -238,11 +238,19 @@ __global__ void __launch_bounds__(1024) k_moe_sort_plan(MoeSortParams p, SortPla
     int* start = ws + (plan.slices + 1) * E;
     int* local = start + E;
     for (int j = tid; j < E; j += 1024) {
+        // the counts of the column in batches of independent loads (one memory latency per batch, not one per slice), then the running sums;
+        // neighbouring threads walk neighbouring columns: coalesced
         int acc = 0;
-        for (int g = 0; g < plan.slices; g++) {  // neighbouring threads walk neighbouring columns: coalesced
-            const int c = off[g * E + j];
-            off[g * E + j] = acc;
-            acc += c;
+        for (int g0 = 0; g0 < plan.slices; g0 += 16) {  // 16 at a time: the registers of 1024 threads allow no more
+            int c[16];
+#pragma unroll
+            for (int g = 0; g < 16; g++) c[g] = g0 + g < plan.slices ? off[(g0 + g) * E + j] : 0;
+#pragma unroll
+            for (int g = 0; g < 16; g++)
+                if (g0 + g < plan.slices) {
+                    off[(g0 + g) * E + j] = acc;
+                    acc += c[g];
+                }
         }
         const int enabled = !p.expert_mask || p.expert_mask[j] != 0;
         off[plan.slices * E + j] = enabled ? acc : 0;  // row `slices` = pairs of the expert that are kept
@@ -250,23 +258,44 @@ __global__ void __launch_bounds__(1024) k_moe_sort_plan(MoeSortParams p, SortPla
         padded[j] = enabled ? (acc + B - 1) / B * B : 0;
     }
     __syncthreads();
-    if (tid == 0) {  // E <= 4096 serial steps: a few microseconds, once per routing
-        int row = 0, loc = 0;
-        for (int j = 0; j < E; j++) {
-            s_start[j] = row;
-            s_local[j] = loc;
-            row += padded[j];
-            loc += on[j];
-        }
-        start[2 * E] = row;  // the total, behind start[] and local[]
-        p.num_valid[0] = row;
-        p.num_valid[1] = p.tokens;
+    // exclusive prefix sums of padded[] (start rows) and on[] (local expert numbers): a Hillis-Steele scan over the experts in LDS,
+    // up to four entries per thread, log2(E) rounds
+    for (int j = tid; j < E; j += 1024) {
+        s_start[j] = padded[j];
+        s_local[j] = on[j];
     }
     __syncthreads();
+    for (int d = 1; d < E; d <<= 1) {
+        int add_p[SORT_MAX_EXPERTS / 1024], add_o[SORT_MAX_EXPERTS / 1024];
+#pragma unroll
+        for (int q = 0; q < SORT_MAX_EXPERTS / 1024; q++) {
+            const int j = tid + q * 1024;
+            const bool take = j < E && j >= d;
+            add_p[q] = take ? s_start[j - d] : 0;
+            add_o[q] = take ? s_local[j - d] : 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < SORT_MAX_EXPERTS / 1024; q++) {
+            const int j = tid + q * 1024;
+            if (j < E) {
+                s_start[j] += add_p[q];
+                s_local[j] += add_o[q];
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        const int total = s_start[E - 1];
+        start[2 * E] = total;  // behind start[] and local[]
+        p.num_valid[0] = total;
+        p.num_valid[1] = p.tokens;
+    }
     for (int j = tid; j < E; j += 1024) {
-        start[j] = s_start[j];
-        local[j] = s_local[j];
-        for (int b = 0; b < padded[j] / B; b++) p.sorted_expert_ids[s_start[j] / B + b] = s_local[j];
+        const int st = s_start[j] - padded[j], lo = s_local[j] - on[j];
+        start[j] = st;
+        local[j] = lo;
+        for (int b = 0; b < padded[j] / B; b++) p.sorted_expert_ids[st / B + b] = lo;
     }
 }
 
