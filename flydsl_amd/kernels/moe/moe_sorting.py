@@ -70,6 +70,17 @@ def _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_
     return args, workspace
 
 
+def _local_tokens(num_local_tokens, rows):
+    """The reference's ``num_local_tokens`` (moe_sorting_kernel.py:2100-2104): only the first so many rows are routed; a tensor is
+    read with ``.item()`` (a host synchronisation, as in the reference), an int costs nothing."""
+    if num_local_tokens is None:
+        return int(rows)
+    m = int(num_local_tokens.item()) if isinstance(num_local_tokens, torch.Tensor) else int(num_local_tokens)
+    if not 1 <= m <= rows:
+        raise ValueError(f"num_local_tokens={m} must lie in [1, {rows}]")
+    return m
+
+
 def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf,
                        num_experts, unit_size=UNIT_SIZE, expert_mask=None, num_local_tokens=None, workspace=None, *,
                        stream=None):
@@ -78,12 +89,12 @@ def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorte
     int32 ``[tokens, topk]``, ``topk_weights`` fp32, ``expert_mask`` int32 ``[num_experts]`` or ``None``.  ``workspace``:
     a device tensor of ``moe_sorting_get_workspace_size(...)`` bytes lets routings of more than 4096 pairs sort in three
     short launches; ``None`` allocates one when it is needed (pass your own under graph capture or in serving loops),
-    ``False`` forces the single launch.  ``num_local_tokens`` (expert parallelism) is not implemented."""
-    if num_local_tokens is not None:
-        raise NotImplementedError("num_local_tokens (expert-parallel token count) is not implemented")
+    ``False`` forces the single launch.  ``num_local_tokens`` (int, or a tensor read with ``.item()``): sort only the first so
+    many tokens; the padding value and ``num_valid_ids[1]`` then carry that count."""
     if topk_ids.dim() != 2 or topk_ids.shape != topk_weights.shape:
         raise ValueError("topk_ids and topk_weights must both be [tokens, topk]")
     tokens, topk = topk_ids.shape
+    tokens = _local_tokens(num_local_tokens, tokens)
     args, _ws = _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size,
                            expert_mask, workspace, topk_ids.device, routing=(topk_ids, topk_weights))
     handle = _lib.lib()
@@ -103,11 +114,9 @@ def moe_softmax_sort_flydsl(gating_logits, sorted_ids, sorted_weights, sorted_ex
     caller gives them (``[tokens, topk]`` int32 / fp32; needed under graph capture) and through fresh tensors otherwise."""
     from .topk_gating_softmax import gating_args
 
-    if num_local_tokens is not None:
-        raise NotImplementedError("num_local_tokens (expert-parallel token count) is not implemented")
     if gating_logits.dim() != 2 or gating_logits.shape[1] != int(num_experts):
         raise ValueError("gating_logits must be [tokens, num_experts]")
-    tokens, topk = int(gating_logits.shape[0]), int(topk)
+    tokens, topk = _local_tokens(num_local_tokens, int(gating_logits.shape[0])), int(topk)
     handle = _lib.lib()
     fused = bool(handle.psg_moe_softmax_sorting_fused(tokens, topk, int(num_experts)))
     if not fused:

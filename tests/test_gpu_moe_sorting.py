@@ -163,7 +163,31 @@ def test_bad_arguments_are_refused_before_launch():
         moe_sorting_flydsl(ids.to(dev).long(), w.to(dev), *ok(), None, 8, 32)
     with pytest.raises(ValueError):
         moe_sorting_flydsl(ids, w, *ok(), None, 8, 32)  # host tensors
-    with pytest.raises(NotImplementedError):
-        moe_sorting_flydsl(ids.to(dev), w.to(dev), *ok(), None, 8, 32, None, 16)
+    with pytest.raises(ValueError):
+        moe_sorting_flydsl(ids.to(dev), w.to(dev), *ok(), None, 8, 32, None, 0)  # num_local_tokens outside [1, tokens]
     with pytest.raises(ValueError):
         moe_sorting_flydsl(ids.to(dev), w.to(dev), *ok(), None, 5000, 32)  # more experts than the kernel's histogram holds
+
+
+@pytest.mark.parametrize("local", [40, torch.tensor([7], dtype=torch.int32)])
+def test_num_local_tokens_sorts_only_the_first_rows(local):
+    # the reference's expert-parallel token count (moe_sorting_kernel.py:2100-2104): the routing behaves as if it had that many tokens
+    dev = torch.device("cuda")
+    tokens, experts, topk, unit = 64, 16, 4, 16
+    ids, w = _routing(tokens, experts, topk, 11)
+    m = int(local.item()) if isinstance(local, torch.Tensor) else local
+    rows, blocks = sorted_sizes(tokens, topk, experts, unit)
+    s_ids = torch.full((rows,), -7, dtype=torch.int32, device=dev)
+    s_w = torch.full((rows,), float("nan"), dtype=torch.float32, device=dev)
+    s_e = torch.full((blocks,), -7, dtype=torch.int32, device=dev)
+    nv = torch.full((2,), -7, dtype=torch.int32, device=dev)
+    moe_sorting_flydsl(ids.to(dev), w.to(dev), s_ids, s_w, s_e, nv, None, experts, unit, None, local.to(dev) if isinstance(local, torch.Tensor) else local)
+    torch.cuda.synchronize()
+    want = O.moe_sorting(ids[:m].numpy(), w[:m].numpy(), experts, unit)
+    n = want[0].size  # the oracle sizes its outputs for m tokens; the caller's are larger and padded the same way
+    assert np.array_equal(s_ids.cpu().numpy()[:n], want[0]) and np.all(s_ids.cpu().numpy()[n:] == ((topk << 24) | m))
+    assert np.array_equal(s_w.cpu().numpy()[:n], want[1]) and np.array_equal(nv.cpu().numpy(), want[3])
+    nb = want[2].size
+    assert np.array_equal(s_e.cpu().numpy()[:nb], want[2]) and np.all(s_e.cpu().numpy()[nb:] == -1)
+    with pytest.raises(ValueError):
+        moe_sorting_flydsl(ids.to(dev), w.to(dev), s_ids, s_w, s_e, nv, None, experts, unit, None, tokens + 1)
