@@ -353,7 +353,7 @@ hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int bloc
     return stage == 1 ? launch_kind<KIND_FP8, 1>(p, block_m, blocks, stream) : launch_kind<KIND_FP8, 2>(p, block_m, blocks, stream);
 }
 
-// sum over the topk slots: y[t, :] = sum_s x[t, s, :] (16-bit in and out, fp32 sum in slot order)
+// sum over the topk slots: y[t, :] = sum_s x[t, s, :] (bf16, fp16 or fp32, the same type in and out; fp32 sum in slot order)
 namespace {
 // mask != nullptr: slot k of token t only counts when mask[ids[t*topk + k]] != 0 (expert parallelism: the rows of experts
 // that live elsewhere were never written by stage 2)
@@ -369,6 +369,11 @@ __global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t*
             const int e = ids[t * topk + k];
             if ((unsigned)e >= (unsigned)experts || mask[e] == 0) continue;
         }
+        if (out_dtype == OUT_F32) {
+            const v4f v = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(x) + (t * topk + k) * (size_t)dim + c);
+            s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+            continue;
+        }
         const v2i v = *reinterpret_cast<const v2i*>(x + (t * topk + k) * (size_t)dim + c);
         const uint16_t h0 = (uint16_t)(v[0] & 0xFFFF), h1 = (uint16_t)((uint32_t)v[0] >> 16), h2 = (uint16_t)(v[1] & 0xFFFF), h3 = (uint16_t)((uint32_t)v[1] >> 16);
         if (out_dtype == OUT_BF16) {
@@ -376,6 +381,10 @@ __global__ void __launch_bounds__(256) k_moe_reduce(const uint16_t* x, uint16_t*
         } else {
             s0 += from_out16<OUT_FP16>(h0); s1 += from_out16<OUT_FP16>(h1); s2 += from_out16<OUT_FP16>(h2); s3 += from_out16<OUT_FP16>(h3);
         }
+    }
+    if (out_dtype == OUT_F32) {
+        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(y) + t * (size_t)dim + c) = (v4f){s0, s1, s2, s3};
+        return;
     }
     const v2i o = out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(s0, s1, s2, s3) : pack4_out16<OUT_FP16>(s0, s1, s2, s3);
     *reinterpret_cast<v2i*>(y + t * (size_t)dim + c) = o;

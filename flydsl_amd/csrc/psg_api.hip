@@ -668,9 +668,10 @@ namespace {
 int moe_reduce_common(const void* x, void* y, const int32_t* mask, const int32_t* ids, int32_t tokens, int32_t topk, int32_t model_dim,
                       int32_t experts, int32_t dtype, void* stream) {
     if (!x || !y) return fail(PSG_E_NULL, "x and y must be non-NULL");
-    if (dtype != PSG_OUT_BF16 && dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "dtype %d must be bf16 or fp16", dtype);
+    if (dtype != PSG_OUT_BF16 && dtype != PSG_OUT_FP16 && dtype != PSG_OUT_F32) return fail(PSG_E_DTYPE, "dtype %d must be bf16, fp16 or fp32", dtype);
     if (tokens < 1 || topk < 1 || model_dim < 4 || model_dim % 4) return fail(PSG_E_SHAPE, "need tokens, topk >= 1 and model_dim a positive multiple of 4");
-    if (!aligned(x, 8) || !aligned(y, 8)) return fail(PSG_E_ALIGN, "x and y must be 8-byte aligned");
+    const int al = dtype == PSG_OUT_F32 ? 16 : 8;
+    if (!aligned(x, al) || !aligned(y, al)) return fail(PSG_E_ALIGN, "x and y must be %d-byte aligned", al);
     if (mask && (!ids || experts < 1)) return fail(PSG_E_NULL, "an expert mask needs topk_ids and experts >= 1");
     const hipError_t e = psg_launch_moe_reduce(x, y, tokens, topk, model_dim, dtype, mask, ids, experts, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_reduce launch");

@@ -125,8 +125,9 @@ class MoeReduction:
 
     def __call__(self, X, Y, expert_mask, topk_ids, i32_m_tokens, stream=None):
         tokens = int(i32_m_tokens)
-        dev = _lib.check_operand("Y", Y, min_elems=tokens * self.model_dim, elem_sizes=(2,))
-        _lib.check_operand("X", X, min_elems=tokens * self.topk * self.model_dim, elem_sizes=(2,), device=dev)
+        esz = (4 if self.dtype == 2 else 2,)
+        dev = _lib.check_operand("Y", Y, min_elems=tokens * self.model_dim, elem_sizes=esz)
+        _lib.check_operand("X", X, min_elems=tokens * self.topk * self.model_dim, elem_sizes=esz, device=dev)
         if self.use_mask:
             # slots whose expert is masked out do not count (and their rows of X were never written)
             _lib.check_operand("expert_mask", expert_mask, min_elems=self.num_experts, elem_sizes=(4,), device=dev)
@@ -142,10 +143,10 @@ class MoeReduction:
 def compile_moe_reduction(*, topk: int, model_dim: int, dtype_str: str = "f16", use_mask: bool = False, num_experts: int = 0,
                           out_dtype_str: str | None = None):
     """Sum over the topk slots (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203), with ``use_mask`` only over the slots
-    whose expert has ``expert_mask != 0`` (``num_experts`` entries).  Built for f16 / bf16 with the same input and output
-    type; the rest (f32, the MXFP8 route-out rows) raises ``NotImplementedError``."""
-    if dtype_str not in ("f16", "bf16") or (out_dtype_str not in (None, dtype_str)):
-        raise NotImplementedError("moe reduction is built for f16 / bf16, same type in and out")
+    whose expert has ``expert_mask != 0`` (``num_experts`` entries).  Built for the dense variants f16 / bf16 / f32 (same
+    input and output type, :57-61); the MXFP8 route-out rows (``dtype_str="fp8"``) raise ``NotImplementedError``."""
+    if dtype_str not in ("f16", "bf16", "f32") or (out_dtype_str not in (None, dtype_str)):
+        raise NotImplementedError("moe reduction is built for f16 / bf16 / f32, same type in and out")
     if use_mask and int(num_experts) < 1:
         raise ValueError("use_mask needs num_experts >= 1")
     return MoeReduction(topk, model_dim, _OUT[dtype_str], use_mask, num_experts)

@@ -284,8 +284,8 @@ typedef struct psg_moe_args {
 int psg_moe_gemm(const psg_moe_args *args, void *stream);
 
 /* y[t, :] = sum over the topk slots of x[t, slot, :] (fp32 sum in slot order), the pass after stage 2 with accumulate = 0
- * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203 with use_mask = False).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16;
- * model_dim % 4 == 0. */
+ * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203 with use_mask = False).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16 / PSG_OUT_F32,
+ * the type of both x and y (the reference's dense variants, :57-61); model_dim % 4 == 0. */
 int psg_moe_reduce(const void *x, void *y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void *stream);
 
 /* The same sum with the reference's expert mask (moe_reduce.py:100-103,147-148): slot k of token t only counts when

@@ -207,14 +207,14 @@ def test_two_stages_end_to_end_with_reduction():
     assert torch.equal(y, want)
 
 
-@pytest.mark.parametrize("dtype_str", ["bf16", "f16"])
+@pytest.mark.parametrize("dtype_str", ["bf16", "f16", "f32"])
 def test_masked_slot_reduction_skips_rows_stage2_never_wrote(dtype_str):
     # expert parallelism: the sorter drops the masked experts, stage 2 never writes their rows, the reduction must not read
     # them (kernels/moe/moe_gemm_2stage/moe_reduce.py:100-103,147-148)
     from kernels.moe.moe_gemm_2stage import compile_moe_reduction
 
     dev = torch.device("cuda")
-    tdt = torch.bfloat16 if dtype_str == "bf16" else torch.float16
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype_str]
     tokens, topk, dim, experts = 77, 4, 520, 16
     g = torch.Generator().manual_seed(3)
     ids = torch.stack([torch.randperm(experts, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
@@ -460,7 +460,7 @@ def test_moe_argument_errors():
     with pytest.raises(ValueError):
         compile_moe_gemm1(**SHAPE, tile_m=48, tile_n=64, tile_k=128, doweight_stage1=False)
     with pytest.raises(NotImplementedError):
-        compile_moe_reduction(topk=2, model_dim=256, dtype_str="f32")
+        compile_moe_reduction(topk=2, model_dim=256, dtype_str="fp8")
     exe = compile_moe_gemm1(**SHAPE, tile_m=16, tile_n=64, tile_k=128, doweight_stage1=False)
     z = torch.zeros(16, device="cuda")
     with pytest.raises(ValueError, match="built for dims"):

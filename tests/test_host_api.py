@@ -159,7 +159,8 @@ def test_moe_c_abi_validation_codes():
         setattr(m, field, old)
     assert handle.psg_moe_reduce(None, None, 1, 1, 4, 0, None) == -1
     assert handle.psg_moe_reduce(0x1000, 0x1000, 4, 2, 6, 0, None) == -2
-    assert handle.psg_moe_reduce(0x1000, 0x1000, 4, 2, 8, 2, None) == -3
+    assert handle.psg_moe_reduce(0x1000, 0x1000, 4, 2, 8, 3, None) == -3
+    assert handle.psg_moe_reduce(0x1008, 0x1000, 4, 2, 8, 2, None) == -6  # fp32 rows are moved 16 bytes at a time
 
 
 def test_mx_quantisers_match_the_oracle_byte_for_byte():
