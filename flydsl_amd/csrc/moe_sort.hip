@@ -16,7 +16,8 @@
 //   1. the pairs are cut into slices; one workgroup per slice writes the slice's histogram to the workspace;
 //   2. one workgroup turns the histograms into per-(slice, expert) offsets, the start row and local number of every
 //      expert, the total, the block ids;
-//   3. one workgroup per (expert, slice) compacts that slice's pairs of that expert straight to their final rows.
+//   3. one workgroup per slice moves the slice's pairs straight to their final rows (lanes with the same expert find each
+//      other with ballots and share a running base in LDS).
 // Either way extra workgroups of the first launch clear the caller's accumulate buffer at full memory bandwidth.
 #include "moe_gating.h"
 
@@ -26,7 +27,7 @@ constexpr int SORT_THREADS = 256;
 constexpr int SORT_WAVES = SORT_THREADS / 64;
 constexpr int SORT_MAX_EXPERTS = 4096;
 constexpr int SORT_ONESHOT_PAIRS = 4096;   // routings up to this many pairs always take the single launch
-constexpr int SORT_SLICE = 2048;           // pairs per slice of the three-launch path (more when there are > 64 slices)
+constexpr int SORT_SLICE = 1024;           // pairs per slice of the three-launch path (more when there would be > 64 slices)
 constexpr int SORT_MAX_SLICES = 64;
 constexpr int FUSE_MAX_TOKENS = 32;        // the gating + sorting launch: every sorting workgroup repeats the gating of all tokens
 constexpr int FUSE_MAX_PAIRS = 1024;
@@ -299,31 +300,95 @@ __global__ void __launch_bounds__(1024) k_moe_sort_plan(MoeSortParams p, SortPla
     }
 }
 
-// launch 3: grid (slices, experts + 1): workgroup (g, e) moves slice g's pairs of expert e; row `experts` fills the tails
+// launch 3: one workgroup per slice moves the slice's pairs straight to their final rows (work proportional to the pairs,
+// whatever the expert count); one more workgroup fills the tails.  Every wavefront owns a contiguous quarter of the slice:
+//   pass 1  histogram of the quarter in a row of LDS counters of its own;
+//   then    the counters become running bases: rows of the expert taken by earlier slices (launch 2) + by earlier wavefronts;
+//   pass 2  64 pairs at a time, in order: the lanes with the same expert find each other with one ballot per bit of the
+//           expert id, rank themselves by lane, read the running base, and the first of them advances it.
+// Stable by construction (slices, wavefronts, chunks and lanes all in pair order) and free of global atomics.
 __global__ void __launch_bounds__(SORT_THREADS) k_moe_sort_scatter(MoeSortParams p, SortPlan plan, const int* ws) {
-    __shared__ int wcount[SORT_WAVES];
-    const int g = (int)blockIdx.x, e = (int)blockIdx.y, E = p.experts;
+    __shared__ int base[SORT_WAVES][SORT_MAX_EXPERTS];
+    const int g = (int)blockIdx.x, E = p.experts, B = p.block_m;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int* off = ws;
     const int* start = ws + (plan.slices + 1) * E;
-    if (e == E) {
-        fill_tails(p, start[2 * E], g, plan.slices);
+    if (g == plan.slices) {
+        fill_tails(p, start[2 * E], 0, 1);
         return;
     }
-    const int kept = off[plan.slices * E + e];  // 0 for a masked expert
-    if (g == 0) {  // padding rows of the expert
-        const int B = p.block_m, padded = (kept + B - 1) / B * B, sentinel = pack_id(p.topk, p.tokens);
-        for (int i = kept + (int)threadIdx.x; i < padded; i += SORT_THREADS) {
-            p.sorted_ids[start[e] + i] = sentinel;
-            p.sorted_weights[start[e] + i] = 0.f;
+    // padding rows: one thread per expert (independent loads; an expert has fewer than block_m padding rows)
+    const int sentinel = pack_id(p.topk, p.tokens);
+    for (int e = g * SORT_THREADS + tid; e < E; e += plan.slices * SORT_THREADS) {
+        const int kept = off[plan.slices * E + e], padded = (kept + B - 1) / B * B, st = start[e];
+        for (int i = kept; i < padded; i++) {
+            p.sorted_ids[st + i] = sentinel;
+            p.sorted_weights[st + i] = 0.f;
         }
     }
-    if (kept == 0) return;
-    const int first = off[g * E + e];
-    const int next = g + 1 < plan.slices ? off[(g + 1) * E + e] : kept;
-    if (next == first) return;  // uniform over the workgroup
     const int P = p.tokens * p.topk;
-    const int lo = g * plan.slice_len, hi = lo + plan.slice_len < P ? lo + plan.slice_len : P;
-    compact_range(p, p.topk_ids, p.topk_weights, e, lo, hi, start[e] + first, wcount);
+    const int lo_s = g * plan.slice_len, hi_s = lo_s + plan.slice_len < P ? lo_s + plan.slice_len : P;
+    const int per = ((hi_s - lo_s + SORT_WAVES - 1) / SORT_WAVES + 63) & ~63;
+    const int lo = lo_s + wave * per, hi = lo + per < hi_s ? lo + per : hi_s;
+    for (int i = lane; i < E; i += 64) base[wave][i] = 0;
+    __syncthreads();
+    constexpr int G = 8;  // chunks of 64 pairs whose loads are issued together (one memory latency per group, not per chunk)
+    for (int q0 = lo; q0 < hi; q0 += 64 * G) {
+        int id[G];
+#pragma unroll
+        for (int c = 0; c < G; c++) {
+            const int q = q0 + c * 64 + lane;
+            id[c] = q < hi ? p.topk_ids[q] : -1;
+        }
+#pragma unroll
+        for (int c = 0; c < G; c++)
+            if ((unsigned)id[c] < (unsigned)E) atomicAdd(&base[wave][id[c]], 1);
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += SORT_THREADS) {
+        int run = start[e] + off[g * E + e];
+#pragma unroll
+        for (int w = 0; w < SORT_WAVES; w++) {
+            const int c = base[w][e];
+            base[w][e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    int bits = 1;
+    while ((1 << bits) < E) bits++;
+    for (int q0 = lo; q0 < hi; q0 += 64 * G) {  // uniform per wavefront
+        int id[G];
+        float wt[G];
+        bool ok[G];
+#pragma unroll
+        for (int c = 0; c < G; c++) {
+            const int q = q0 + c * 64 + lane;
+            id[c] = q < hi ? p.topk_ids[q] : -1;
+            wt[c] = q < hi ? p.topk_weights[q] : 0.f;
+        }
+#pragma unroll
+        for (int c = 0; c < G; c++) ok[c] = (unsigned)id[c] < (unsigned)E && (!p.expert_mask || p.expert_mask[id[c]] != 0);
+#pragma unroll
+        for (int c = 0; c < G; c++) {
+            if (q0 + c * 64 >= hi) break;  // uniform
+            const int q = q0 + c * 64 + lane;
+            unsigned long long peers = __ballot(ok[c]);
+            for (int b = 0; b < bits; b++) {
+                const unsigned long long set = __ballot((id[c] >> b) & 1);
+                peers &= ((id[c] >> b) & 1) ? set : ~set;
+            }
+            const unsigned long long below = peers & ((1ull << lane) - 1ull);
+            if (ok[c]) {
+                const int row = base[wave][id[c]] + __popcll(below);
+                const int token = q / p.topk, slot = q - token * p.topk;
+                p.sorted_ids[row] = pack_id(slot, token);
+                p.sorted_weights[row] = wt[c];
+            }
+            // every lane has read its base: now the first lane of each expert advances it (LDS operations of a wavefront complete in order)
+            if (ok[c] && below == 0) base[wave][id[c]] += __popcll(peers);
+        }
+    }
 }
 
 int clear_wgs(const MoeSortParams& p) {
@@ -405,6 +470,6 @@ hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t
     int* ws = static_cast<int*>(workspace);
     hipLaunchKernelGGL(k_moe_sort_count, dim3(plan.slices + zwgs), dim3(SORT_THREADS), 0, stream, p, plan, ws);
     hipLaunchKernelGGL(k_moe_sort_plan, dim3(1), dim3(1024), 0, stream, p, plan, ws);
-    hipLaunchKernelGGL(k_moe_sort_scatter, dim3(plan.slices, p.experts + 1), dim3(SORT_THREADS), 0, stream, p, plan, (const int*)ws);
+    hipLaunchKernelGGL(k_moe_sort_scatter, dim3(plan.slices + 1), dim3(SORT_THREADS), 0, stream, p, plan, (const int*)ws);
     return hipGetLastError();
 }
