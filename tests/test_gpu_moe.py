@@ -280,6 +280,84 @@ def test_stage1_int8smooth_slot_major_rows(out_dtype, tile_m, tokens):
     assert e2.slot_major is False
 
 
+@pytest.mark.parametrize("tokens,experts,topk,tile_m", [(16, 64, 4, 16), (200, 32, 6, 32)])
+def test_layer_from_router_logits_on_the_device_and_in_a_graph(tokens, experts, topk, tile_m):
+    # logits -> gating + sorting (one launch for 16 tokens, two for 200) -> stage 1 -> device quantiser -> stage 2 with atomics,
+    # nothing on the host in between; then the same launches recorded into a HIP graph and replayed on new logits.  Checked
+    # against the oracle chain fed with the routing the device found (the gating itself is checked in test_gpu_moe_gating.py).
+    from flydsl_amd import quant_device
+    from flydsl_amd.kernels.moe.moe_sorting import sorted_sizes
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+    from kernels.moe.moe_sorting_kernel import moe_softmax_sort_flydsl
+
+    model_dim, inter_dim = 512, 256
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, model_dim, generator=g)
+    w1 = torch.randn(experts, 2 * inter_dim, model_dim, generator=g) / math.sqrt(model_dim)
+    w2 = torch.randn(experts, model_dim, inter_dim, generator=g) / math.sqrt(inter_dim)
+    xq, sx = quant.pertoken_quant(x, quant_dtype=torch.float8_e4m3fn)
+    w1q, sw1 = quant.pertoken_quant(w1, quant_dtype=torch.float8_e4m3fn)
+    w2q, sw2 = quant.pertoken_quant(w2, quant_dtype=torch.float8_e4m3fn)
+    d = lambda t: t.to(dev).contiguous()
+    xq_d, sx_d = d(xq).view(-1), d(sx).view(-1)
+    w1_d, sw1_d = d(layout.shuffle_weight(w1q).view(-1, model_dim)).view(-1), d(sw1).view(-1)
+    w2_d, sw2_d = d(layout.shuffle_weight(w2q).view(-1, inter_dim)).view(-1), d(sw2).view(-1)
+    rows, blocks = sorted_sizes(tokens, topk, experts, tile_m)
+    s_ids = torch.empty(rows, dtype=torch.int32, device=dev)
+    s_w = torch.empty(rows, dtype=torch.float32, device=dev)
+    s_e = torch.empty(blocks, dtype=torch.int32, device=dev)
+    nv = torch.empty(2, dtype=torch.int32, device=dev)
+    t_ids = torch.empty(tokens, topk, dtype=torch.int32, device=dev)
+    t_w = torch.empty(tokens, topk, dtype=torch.float32, device=dev)
+    ws = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+    a2 = torch.empty(tokens, topk, inter_dim, dtype=torch.bfloat16, device=dev)
+    a2q = torch.empty(tokens * topk, inter_dim, dtype=torch.float8_e4m3fn, device=dev)
+    sa2 = torch.empty(tokens * topk, dtype=torch.float32, device=dev)
+    out = torch.full((tokens, model_dim), 7.0, dtype=torch.bfloat16, device=dev)
+    logits = torch.empty(tokens, experts, dtype=torch.bfloat16, device=dev)
+    kw = dict(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=128, tile_k=128, in_dtype="fp8")
+    e1 = compile_moe_gemm1(doweight_stage1=False, out_dtype="bf16", **kw)
+    e2 = compile_moe_gemm2(doweight_stage2=True, out_dtype="bf16", accumulate=True, **kw)
+
+    def layer(stream):
+        moe_softmax_sort_flydsl(logits, s_ids, s_w, s_e, nv, out, experts, topk, "bf16", tile_m, None, True, None,
+                                topk_ids=t_ids, topk_weights=t_w, workspace=ws, stream=stream)
+        e1(a2, xq_d, w1_d, sx_d, sw1_d, s_ids, s_e, s_w, nv, tokens, inter_dim, model_dim, blocks, stream)
+        quant_device.pertoken_quant(a2.view(tokens * topk, inter_dim), torch.float8_e4m3fn, stream=stream, out=(a2q, sa2))
+        e2(out, a2q.view(-1), w2_d, sa2, sw2_d, s_ids, s_e, s_w, nv, tokens, model_dim, inter_dim, blocks, stream)
+
+    def check():
+        ids, wts = t_ids.cpu().numpy(), t_w.cpu().numpy()
+        assert ids.min() >= 0 and ids.max() < experts and np.allclose(wts.sum(1), 1.0, atol=1e-5)
+        ref1 = O.moe_gemm1(xq.view(torch.uint8).numpy(), w1q.view(torch.uint8).numpy().reshape(-1, model_dim), sx.numpy(), sw1.numpy().reshape(-1),
+                           ids, wts, inter_dim, False, "fp8")
+        ok, ratio = O.within_north_star_tolerance(a2.float().cpu().numpy(), ref1, 1e-2)
+        assert ok, f"stage 1 outside tolerance ({ratio:.3f})"
+        ref2 = O.moe_gemm2(a2q.view(torch.uint8).cpu().numpy(), w2q.view(torch.uint8).numpy().reshape(-1, inter_dim), sa2.cpu().numpy(),
+                           sw2.numpy().reshape(-1), ids, wts, model_dim, True, "fp8", reduce_slots=True)
+        ok, ratio = O.within_north_star_tolerance(out.float().cpu().numpy(), ref2.reshape(tokens, model_dim), 2e-2)
+        assert ok, f"stage 2 outside tolerance ({ratio:.3f})"
+
+    mk = lambda seed: (torch.rand(tokens, experts, generator=torch.Generator().manual_seed(seed)) * 4 - 2).to(torch.bfloat16).to(dev)
+    logits.copy_(mk(1))
+    layer(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    check()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        layer(torch.cuda.current_stream())
+    for seed in (2, 3):
+        logits.copy_(mk(seed))
+        out.fill_(7.0)  # the sorter's launch clears it again
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check()
+
+
 @pytest.mark.parametrize("in_dtype", ["fp8", "int8"])
 @pytest.mark.parametrize("tile_m,tokens", [(16, 8), (16, 64), (16, 200), (32, 40), (32, 333)])
 def test_paired_blocks_give_the_same_bits_as_single_blocks(in_dtype, tile_m, tokens):
