@@ -191,3 +191,28 @@ def test_num_local_tokens_sorts_only_the_first_rows(local):
     assert np.array_equal(s_e.cpu().numpy()[:nb], want[2]) and np.all(s_e.cpu().numpy()[nb:] == -1)
     with pytest.raises(ValueError):
         moe_sorting_flydsl(ids.to(dev), w.to(dev), s_ids, s_w, s_e, nv, None, experts, unit, None, tokens + 1)
+
+
+def test_random_routings_both_plans():
+    # 40 random shapes around the borders of the kernels: 4096 pairs (one launch / three), 1024-pair slices, 64-pair chunks,
+    # expert counts that are not powers of two, masks, ids outside the range
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        experts = int(rng.choice([3, 8, 17, 32, 96, 129, 256, 1000]))
+        topk = int(rng.integers(1, min(experts, 9) + 1))
+        pairs = int(rng.choice([1, 63, 64, 65, 1023, 1025, 4095, 4097, 6000, 9000, 20000]))
+        tokens = max(1, pairs // topk)
+        unit = int(rng.choice([1, 16, 32, 64, 128]))
+        ids = torch.from_numpy(rng.integers(0, experts, (tokens, topk)).astype(np.int32))
+        if case % 5 == 0:
+            ids[rng.integers(0, tokens), rng.integers(0, topk)] = experts + 3  # dropped by the kernel, as by the oracle
+        w = torch.from_numpy(rng.random((tokens, topk), dtype=np.float32))
+        mask = None
+        if case % 3 == 0:
+            mask = (rng.random(experts) < 0.7).astype(np.int32)
+        valid = ids.clone()
+        for workspace in (None, False):
+            got = _run(valid, w, experts, unit, mask, workspace=workspace)
+            want = O.moe_sorting(np.where(valid.numpy() < experts, valid.numpy(), -1), w.numpy(), experts, unit, expert_mask=mask)
+            for name, a, b in zip(("sorted_ids", "sorted_weights", "sorted_expert_ids", "num_valid_ids"), got, want):
+                assert np.array_equal(a, b), (case, name, tokens, experts, topk, unit, workspace)
