@@ -335,7 +335,7 @@ hipError_t launch_kind(const MoeParams& p, int block_m, int blocks, hipStream_t 
     const int tile_m = pair ? 2 * block_m : block_m;
     // 128 columns per workgroup when they divide the output; stage 1 (two accumulator sets) only for tiles of up to 32
     // rows: measured at 4096 tokens x top-8, blocks of 128: stage 1 488 us with 64 columns against 800 with 128, stage 2
-    // 442 against 412 (stage 2 with 256 columns and one workgroup per CU: 805)
+    // 442 against 412 (stage 2 with 256 columns: 805 with one workgroup per CU, 492 when held to two)
     // ... and only when that still leaves several workgroups per CU: a workgroup streams its slab at the pace its loads in
     // flight allow, so a decode-sized stage 1 (64 tokens x top-8 on 32 experts: at most 63 blocks x 12 column tiles) is faster
     // with twice as many workgroups of half the width
