@@ -67,6 +67,7 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     constexpr int WSH = W4 ? 1 : 0;                    // weight byte offsets are halved
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * 128];
     __shared__ int ids[BM];
+    __shared__ float s_sx[BM], s_rw[BM];  // per tile row: scale of its x row and routing weight, fetched before the K loop
 
     const int tid = threadIdx.x;
     const int wave = wave_id();
@@ -107,6 +108,13 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         if constexpr (STAGE == 1) return p.x_slot_major ? s * p.tokens + t : t;
         return t * p.topk + s;
     };
+    // the epilogue's per-row factors now, so that their memory latency runs under the K loop (whose barriers also make them
+    // visible to every wavefront)
+    if (tid < BM) {
+        const int xr = x_row(tid);
+        s_sx[tid] = xr >= 0 ? p.sx[xr] : 0.f;
+        s_rw[tid] = (p.doweight && xr >= 0) ? p.sorted_w[blk * BLK + tid] : 1.0f;
+    }
 
     const int K = p.K, KT = K >> 7;
     const int rows_x = (STAGE == 1 && !p.x_slot_major) ? p.tokens : p.tokens * p.topk;
@@ -171,6 +179,16 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
                 }
             }
     };
+
+    // the weight scales of the lane's columns (pass ni: columns ni*64 + wave*16 + lg*4 + 0..3), also ahead of the K loop
+    v4f swa_[NR], swb_[STAGE == 1 ? NR : 1];
+#pragma unroll
+    for (int ni = 0; ni < NR; ni++) {
+        const int ncol = n0 + ni * 64 + wave * 16 + lg * 4;
+        const bool in = ncol < p.n_out;
+        swa_[ni] = in ? *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + ncol) : (v4f){0.f, 0.f, 0.f, 0.f};
+        if constexpr (STAGE == 1) swb_[ni] = in ? *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + p.n_out + ncol) : (v4f){0.f, 0.f, 0.f, 0.f};
+    }
 
     acc_t acc[MR][NSET][NR];
 #pragma unroll
@@ -248,17 +266,12 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     static_for<NR>([&](auto NI) {
         constexpr int ni = decltype(NI)::value;
         const int ncol = n0 + ni * 64 + wave * 16 + lg * 4;   // first of the lane's four columns
-        v4f swa = {0.f, 0.f, 0.f, 0.f}, swb = {0.f, 0.f, 0.f, 0.f};
-        if (ncol < p.n_out) {
-            swa = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + ncol);
-            if constexpr (STAGE == 1) swb = *reinterpret_cast<const v4f*>(p.sw + (size_t)e * rows_e + p.n_out + ncol);
-        }
+        const v4f swa = swa_[ni], swb = swb_[STAGE == 1 ? ni : 0];
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
             const int r = mi * 16 + li;
-            const int xr = x_row(r);
-            const float sx = xr >= 0 ? p.sx[xr] : 0.f;
-            const float rw = (p.doweight && xr >= 0) ? p.sorted_w[blk * BLK + r] : 1.0f;
+            const float sx = s_sx[r];
+            const float rw = s_rw[r];
             v4f y;
             if constexpr (STAGE == 1) {
                 const acc_t ag = acc[mi][0][ni], au = acc[mi][NSET - 1][ni];
