@@ -94,28 +94,6 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         if ((blk + 1) * BLK < used && p.expert_ids[blk + 1] == e) rows_live = BM;
     }
 
-    if (tid < BM) {
-        const int q = blk * BLK + tid;
-        ids[tid] = (tid < rows_live && q < p.sorted_size) ? p.sorted_ids[q] : p.tokens;  // past the list or the pair = a padding row
-    }
-    __syncthreads();
-
-    // row of x (and of its scale) a tile row reads, or -1 for a padding row
-    auto x_row = [&](int r) {
-        const uint32_t sid = (uint32_t)ids[r];
-        const int t = (int)(sid & 0xFFFFFFu), s = (int)(sid >> 24);
-        if (t >= p.tokens || s >= p.topk) return -1;
-        if constexpr (STAGE == 1) return p.x_slot_major ? s * p.tokens + t : t;
-        return t * p.topk + s;
-    };
-    // the epilogue's per-row factors now, so that their memory latency runs under the K loop (whose barriers also make them
-    // visible to every wavefront)
-    if (tid < BM) {
-        const int xr = x_row(tid);
-        s_sx[tid] = xr >= 0 ? p.sx[xr] : 0.f;
-        s_rw[tid] = (p.doweight && xr >= 0) ? p.sorted_w[blk * BLK + tid] : 1.0f;
-    }
-
     const int K = p.K, KT = K >> 7;
     const int rows_x = (STAGE == 1 && !p.x_slot_major) ? p.tokens : p.tokens * p.topk;
     const int rows_e = STAGE == 1 ? 2 * p.n_out : p.n_out;            // weight rows per expert
@@ -123,15 +101,6 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
     const uint8_t* w_e = p.w + (((uint64_t)e * (uint64_t)rows_e * (uint64_t)K) >> WSH);
     __amdgpu_buffer_rsrc_t rb = make_rsrc(w_e, ((uint64_t)rows_e * (uint64_t)K) >> WSH);
 
-    uint32_t a_voff[A_LOADS];
-    int a_ldsoff[A_LOADS];
-#pragma unroll
-    for (int j = 0; j < A_LOADS; j++) {
-        const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
-        const int xr = row < BM ? x_row(row) : -1;
-        a_voff[j] = xr >= 0 ? (uint32_t)xr * (uint32_t)K + (uint32_t)kc * 16u : 0xFFFFFFF0u;
-        a_ldsoff[j] = row < BM ? moe_lds_off(row, kc) : -1;
-    }
     // n-blocks of this wavefront inside the expert's slab: set 0 = gate (or the only set), set 1 = up
     uint32_t b_voff[NSET][NR];
 #pragma unroll
@@ -144,6 +113,8 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
             b_voff[s][ni] = n < p.n_out ? ((uint32_t)nb * 16u * (uint32_t)K + (uint32_t)lane * 16u) >> WSH : 0xFFFFFFF0u;
         }
 
+    uint32_t a_voff[A_LOADS];
+    int a_ldsoff[A_LOADS];
     v4i areg[A_LOADS];
     auto load_a = [&](int kt) {
 #pragma unroll
@@ -241,8 +212,38 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         __syncthreads();
     };
 
-    load_a(0);
+    // W first: its addresses need only the expert, so these requests are in flight while the sorted row list is fetched
     static_for<WPF>([&](auto I) { load_b(decltype(I)::value, decltype(I)::value); });
+    if (tid < BM) {
+        const int q = blk * BLK + tid;
+        ids[tid] = (tid < rows_live && q < p.sorted_size) ? p.sorted_ids[q] : p.tokens;  // past the list or the pair = a padding row
+    }
+    __syncthreads();
+
+    // row of x (and of its scale) a tile row reads, or -1 for a padding row
+    auto x_row = [&](int r) {
+        const uint32_t sid = (uint32_t)ids[r];
+        const int t = (int)(sid & 0xFFFFFFu), s = (int)(sid >> 24);
+        if (t >= p.tokens || s >= p.topk) return -1;
+        if constexpr (STAGE == 1) return p.x_slot_major ? s * p.tokens + t : t;
+        return t * p.topk + s;
+    };
+    // the epilogue's per-row factors now, so that their memory latency runs under the K loop (whose barriers also make them
+    // visible to every wavefront)
+    if (tid < BM) {
+        const int xr = x_row(tid);
+        s_sx[tid] = xr >= 0 ? p.sx[xr] : 0.f;
+        s_rw[tid] = (p.doweight && xr >= 0) ? p.sorted_w[blk * BLK + tid] : 1.0f;
+    }
+
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) {
+        const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
+        const int xr = row < BM ? x_row(row) : -1;
+        a_voff[j] = xr >= 0 ? (uint32_t)xr * (uint32_t)K + (uint32_t)kc * 16u : 0xFFFFFFF0u;
+        a_ldsoff[j] = row < BM ? moe_lds_off(row, kc) : -1;
+    }
+    load_a(0);
     store_a(0);
     __syncthreads();
     // unrolled over lcm(2 LDS stages, NWS register sets) steps so that both indices are compile-time
