@@ -591,3 +591,63 @@ def test_moe_stages_replay_from_a_graph():
         assert torch.equal(out1, want1)
         # fp32 atomics: one addition per slot, order not fixed -> equal up to fp32 rounding
         assert torch.allclose(out2, want2, rtol=1e-5, atol=1e-5 * float(want2.abs().max()))
+
+
+def test_random_moe_stage_shapes_against_the_oracle():
+    # 24 random problems over every input format, block size and output mode, with skewed routings (experts without rows,
+    # experts with several blocks) and widths that are not multiples of the 128-column tile
+    from kernels.moe.moe_gemm_2stage import compile_moe_gemm1, compile_moe_gemm2
+
+    rng = np.random.default_rng(77)
+    dev = torch.device("cuda")
+    for case in range(24):
+        in_dtype = ["fp8", "int8", "int4", "int8smooth"][case % 4]
+        tile_m = int(rng.choice([16, 32, 64, 128]))
+        experts = int(rng.choice([3, 8, 17]))
+        topk = int(rng.integers(1, min(experts, 4) + 1))
+        tokens = int(rng.choice([1, 5, 33, 70, 200]))
+        model_dim = int(rng.choice([256, 512, 768]))
+        inter_dim = int(rng.choice([128, 256, 384]))
+        stage = 1 + case % 2
+        g = torch.Generator().manual_seed(1000 + case)
+        bias = torch.linspace(1.0, -1.0, experts)
+        vals, ids = torch.topk(torch.rand(tokens, experts, generator=g) + bias, k=topk, dim=1)
+        ids, wts = ids.int(), torch.softmax(vals, dim=1).float()
+        sid, swt, se, npp = moe_sorting(ids, wts, num_experts=experts, block_size=tile_m)
+        routing = (sid, swt, se, npp[:1].contiguous(), int(se.numel()))
+        qdt = torch.float8_e4m3fn if in_dtype == "fp8" else torch.int8
+        kind = "fp8" if in_dtype == "fp8" else "int8"
+        wmax = {"dtypeMax": 7} if in_dtype == "int4" else {}
+        K, n_out = (model_dim, inter_dim) if stage == 1 else (inter_dim, model_dim)
+        rows_e = 2 * n_out if stage == 1 else n_out
+        slot_major = stage == 1 and in_dtype == "int8smooth"
+        rows_x = tokens if (stage == 1 and not slot_major) else tokens * topk
+        x = torch.randn(rows_x, K, generator=g)
+        w = torch.randn(experts * rows_e, K, generator=g) / math.sqrt(K)
+        xq, sx = quant.pertoken_quant(x, quant_dtype=qdt)
+        wq, sw = quant.pertoken_quant(w * (8.0 if in_dtype == "int4" else 1.0), quant_dtype=qdt, **wmax)
+        wk = layout.shuffle_weight(wq).view(experts * rows_e, K).contiguous()
+        if in_dtype == "int4":
+            wk = layout.pack_shuffled_int8_to_int4(wk)
+        kw = dict(model_dim=model_dim, inter_dim=inter_dim, experts=experts, topk=topk, tile_m=tile_m, tile_n=64, tile_k=128, in_dtype=in_dtype)
+        tag = (case, in_dtype, stage, tile_m, experts, topk, tokens, model_dim, inter_dim)
+        if stage == 1:
+            doweight = bool(case & 4)
+            out = torch.full((tokens, topk, inter_dim), float("nan"), dtype=torch.bfloat16, device=dev)
+            exe = compile_moe_gemm1(doweight_stage1=doweight, out_dtype="bf16", **kw)
+            _launch(exe, out, xq, wk, sx, sw.view(-1, 1), routing, inter_dim, model_dim, tokens)
+            ref = O.moe_gemm1(xq.view(torch.uint8).numpy(), wq.view(torch.uint8).numpy(), sx.numpy(), sw.numpy().reshape(-1), ids.numpy(), wts.numpy(),
+                              inter_dim, doweight, kind, x_slot_major=slot_major)
+            got = out.float().cpu().numpy()
+        else:
+            accumulate = bool(case & 4)
+            rows = tokens if accumulate else tokens * topk
+            out = torch.zeros(rows, model_dim, dtype=torch.bfloat16, device=dev)
+            exe = compile_moe_gemm2(doweight_stage2=True, out_dtype="bf16", accumulate=accumulate, **kw)
+            _launch(exe, out, xq, wk, sx, sw.view(-1, 1), routing, model_dim, inter_dim, tokens)
+            ref = O.moe_gemm2(xq.view(torch.uint8).numpy(), wq.view(torch.uint8).numpy(), sx.numpy().reshape(-1), sw.numpy().reshape(-1), ids.numpy(),
+                              wts.numpy(), model_dim, True, kind, reduce_slots=accumulate).reshape(rows, model_dim)
+            got = out.float().cpu().numpy()
+        assert not np.isnan(got).any(), tag
+        ok, ratio = O.within_north_star_tolerance(got, ref, 2e-2 if (stage == 2) else 1e-2)
+        assert ok, (tag, ratio)
