@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(256) k_moe_gemm(MoeParams p) {
         }
         before = __builtin_amdgcn_readfirstlane(before);
         if (before & 1) return;                        // uniform: the second block of a pair
-        if ((blk + 1) * BLK < used && p.expert_ids[blk + 1] == e) rows_live = BM;
+        if (blk + 1 < (int)gridDim.y && (blk + 1) * BLK < used && p.expert_ids[blk + 1] == e) rows_live = BM;  // (gridDim.y = entries of expert_ids)
     }
 
     const int K = p.K, KT = K >> 7;
