@@ -145,12 +145,13 @@ int pick_splits(int M, int N, int kbytes, Tile t) {
     const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
     const int steps = (kbytes + 127) / 128;
     if (tiles >= 192 || steps < 32) return 1;
-    // measured optimum: about 16 K steps per workgroup, at most ~1024 workgroups, partial traffic bounded: a quarter of W
-    // once every CU has a workgroup; while CUs would stay idle the bound is five times looser, because an idle CU costs more
-    // than the partial sums (fp8 512x4096x14336, 128 tiles: 71 us unsplit, 49 us with two splits; 256x4096x14336: 45 -> 32 us)
+    // measured on operands that do not fit the last-level cache: at least 12 K steps per workgroup, at most one workgroup per
+    // CU (256) in total, partial traffic bounded: a quarter of W once half the CUs have a workgroup; while more than half would
+    // stay idle the bound is five times looser, because an idle CU costs more than the partial sums (fp8, us for 1/2/4/8 splits
+    // of 128x128 tiles: 96x4096x14336 68/41/28/24, 512x4096x14336 71/48/49/60, 96x8192x8192 43/31/25/28, 384x5120x13824
+    // 67/46/47/58, 512x5120x5120, 160 tiles, 30/37)
     int s = 1;
-    while (s < 8 && steps / (s * 2) >= 16 && tiles * (s * 2) <= 1024 &&
-           (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s < 256 ? 5 : 1))
+    while (s < 8 && steps / (s * 2) >= 12 && tiles * (s * 2) <= 256 && (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s <= 128 ? 5 : 1))
         s *= 2;
     return s;
 }
@@ -178,6 +179,12 @@ Plan plan_tiled(int M, int N, int kbytes, bool mx) {
     const long tiles_big = (long)((M + 127) / 128) * (long)((N + 255) / 256);
     const int steps = (kbytes + 127) / 128;
     if (!mx && tiles_big < 192 && steps >= 48) t = M <= 64 ? Tile{64, 64, 4} : Tile{128, 128, 4};
+    // Shorter rows (8..47 steps; K = 4096 one-byte elements is 32): while at most about 600 of them exist, 64x64 tiles beat
+    // every larger shape, with or without split-K: many small workgroups keep more bytes of W in flight than a few large ones
+    // (fp8, weights not cache-resident: M=128, N=K=4096 14.0 us against 19.4 with 128x128 tiles and two K splits; M=256,
+    // N=8192 22.0 against 23.7; M=384, N=8192, 768 tiles: 28.0 against 26.5, so the larger tile is kept there)
+    const long tiles64 = (long)((M + 63) / 64) * (long)((N + 63) / 64);
+    if (!mx && steps >= 8 && steps < 48 && tiles64 <= 600) t = Tile{64, 64, 4};
     return {t, pick_splits(M, N, kbytes, t)};
 }
 
