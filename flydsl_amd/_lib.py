@@ -11,7 +11,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsgemm.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 IN_DTYPE = {"int8": 0, "fp8": 1, "fp16": 2, "bf16": 3, "int4": 6}  # "int4": the MoE stages' int8 x packed-int4 weights
 OUT_DTYPE = {"bf16": 0, "fp16": 1}
@@ -33,6 +33,7 @@ EXPORTS = (
     "psg_tile_coords",
     "psg_debug_tile_order",
     "psg_moe_gemm",
+    "psg_moe_mx_gemm",
     "psg_moe_reduce",
     "psg_moe_reduce_masked",
     "psg_moe_sorting",
@@ -135,6 +136,33 @@ class MoeArgs(ctypes.Structure):
     ]
 
 
+class MoeMxArgs(ctypes.Structure):
+    _fields_ = [
+        ("out", ctypes.c_void_p),
+        ("out_scale", ctypes.c_void_p),
+        ("a", ctypes.c_void_p),
+        ("a_scale", ctypes.c_void_p),
+        ("w", ctypes.c_void_p),
+        ("w_scale", ctypes.c_void_p),
+        ("sorted_token_ids", ctypes.c_void_p),
+        ("sorted_expert_ids", ctypes.c_void_p),
+        ("sorted_weights", ctypes.c_void_p),
+        ("num_valid_ids", ctypes.c_void_p),
+        ("tokens", ctypes.c_int32),
+        ("experts", ctypes.c_int32),
+        ("model_dim", ctypes.c_int32),
+        ("inter_dim", ctypes.c_int32),
+        ("sorted_size", ctypes.c_int32),
+        ("blocks", ctypes.c_int32),
+        ("block_m", ctypes.c_int32),
+        ("a_dtype", ctypes.c_int32),
+        ("out_dtype", ctypes.c_int32),
+        ("stage", ctypes.c_int32),
+        ("atomic", ctypes.c_int32),
+        ("pad0", ctypes.c_int32),
+    ]
+
+
 class MoeSortArgs(ctypes.Structure):
     _fields_ = [
         ("topk_ids", ctypes.c_void_p),
@@ -211,7 +239,7 @@ def lib() -> ctypes.CDLL:
     handle.psg_moe_softmax_sorting.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     handle.psg_moe_softmax_sorting_fused.restype = ctypes.c_int
     handle.psg_moe_softmax_sorting_fused.argtypes = [ctypes.c_int32] * 3
-    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm", "psg_moe_sorting", "psg_moe_topk_gating"):
+    for name in ("psg_gemm_a8w8", "psg_gemm_mxfp4", "psg_gemm_a8w8_static", "psg_moe_gemm", "psg_moe_mx_gemm", "psg_moe_sorting", "psg_moe_topk_gating"):
         fn = getattr(handle, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]

@@ -1,0 +1,269 @@
+// MoE grouped GEMMs with MX operands for gfx950: activations in fp4 (e2m1) or fp8 (e4m3), expert weights in fp4, one e8m0
+// scale per 32 K elements on both sides (v_mfma_scale_f32_16x16x128_f8f6f4), over blocks of sorted token rows that all
+// belong to one expert.
+//   stage 1 (gate-up): g = a[t] . W1[e, n], u = a[t] . W1[e, inter + n]; y = silu(g) * u; y is quantised again per 32 columns
+//                      (scale byte = exponent of the smallest power of two >= amax / 6, e2m1 codes by nearest-even) and
+//                      written by SORTED position: codes row-major, scales in the shuffled layout stage 2 reads.
+//   stage 2 (down):    y[n] = a2[sorted row] . W2[e, n]; times the routing weight and added atomically into out[token], or
+//                      written unweighted to one row per sorted position.
+// Operand layouts (lane l = 16 g + i of a wavefront, one 128-element K step):
+//   A fp4: row i's 16 bytes at byte 16 g of its 64-byte step; fp8: the 16-byte pieces g and 4 + g of its 128-byte step.
+//   W: one preshuffled 1 KB block (16 rows x 64 bytes) is one operand: lane l reads bytes [16 l, 16 l + 16).
+//   Scales: per (32-row chunk, 256-K chunk) 64 dwords; lane l's dword holds the bytes (128-K half kh, 16-row half h) at
+//           byte 2 kh + h, selected with the MFMA's op_sel.  The A-side chunks count SORTED rows.
+// Operands are swapped (src0 = W, src1 = A) so a lane ends up with 4 consecutive columns of one row.  Four wavefronts side
+// by side along N; each covers 64 W rows: in stage 1 32 gate rows and the 32 up rows of the same columns, so a wavefront
+// owns whole 32-column quantisation groups.
+#include "psg_common.h"
+
+namespace {
+
+typedef __fp16 v2h __attribute__((ext_vector_type(2)));
+typedef __bf16 v2b __attribute__((ext_vector_type(2)));
+
+// adds the two 16-bit values packed in `bits` to o[0], o[1]
+template <int OUT>
+__device__ __forceinline__ void atomic_add2(uint16_t* o, int bits) {
+    if constexpr (OUT == OUT_BF16) __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) v2b*)o, __builtin_bit_cast(v2b, bits));
+    else __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) v2h*)o, __builtin_bit_cast(v2h, bits));
+}
+
+template <int AF, int MR, int STAGE>
+__global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
+    static_assert(MR % 2 == 0, "scale chunks cover 32 rows");
+    constexpr int NR = 4;
+    constexpr int TM = 16 * MR;
+    constexpr int TN = STAGE == 1 ? 128 : 256;     // output columns per workgroup
+    constexpr int AB = AF == MXF_FP4 ? 64 : 128;   // bytes of an A row per K step
+    constexpr int CPR = AB / 16;                   // 16-byte chunks per staged row
+    constexpr int A_LOADS = (TM * CPR + 255) / 256;
+    constexpr int ACODE = AF == MXF_FP4 ? 4 : 0;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * AB];
+
+    const int blk = blockIdx.y;
+    if (blk * TM >= p.num_valid[0]) return;
+    const int e = p.expert_ids[blk];
+    if ((unsigned)e >= (unsigned)p.experts) return;
+
+    const int tid = threadIdx.x;
+    const int wave = wave_id();
+    const int lane = tid & 63, li = lane & 15, lg = lane >> 4;
+    const int n0 = (int)blockIdx.x * TN;
+    const int KT = p.K >> 7;  // 128-element steps (even: K % 256 == 0)
+    const uint32_t a_row_bytes = AF == MXF_FP4 ? (uint32_t)p.K >> 1 : (uint32_t)p.K;
+    const uint32_t b_row_bytes = (uint32_t)p.K >> 1;
+    const uint32_t chunk_bytes = (uint32_t)(p.K >> 8) * 256u;  // one 32-row chunk of shuffled scales
+    const int w_rows = STAGE == 1 ? 2 * p.n_out : p.n_out;     // rows of one expert's matrix
+
+    // A: stage 1 gathers token rows, stage 2 reads the block's sorted rows; rows without a token read as zero
+    const int a_rows = STAGE == 1 ? p.tokens : p.sorted_size;
+    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)a_rows * a_row_bytes);
+    uint32_t arow[A_LOADS];
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) {
+        const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
+        arow[j] = 0xFFFFFFF0u;
+        if (row < TM) {
+            const int src = STAGE == 1 ? (p.sorted_ids[blk * TM + row] & 0xFFFFFF) : blk * TM + row;
+            if (src < a_rows) arow[j] = (uint32_t)src * a_row_bytes + (uint32_t)kc * 16u;
+        }
+    }
+    // W and its scales: this expert's matrix; the wavefront's four n-blocks
+    __amdgpu_buffer_rsrc_t rb = make_rsrc(p.w + (uint64_t)e * (uint64_t)w_rows * b_row_bytes, (uint64_t)w_rows * b_row_bytes);
+    __amdgpu_buffer_rsrc_t rsb = make_rsrc(p.w_scale + (uint64_t)e * (uint64_t)(w_rows >> 5) * chunk_bytes, (uint64_t)(w_rows >> 5) * chunk_bytes);
+    uint32_t boff[NR], sboff[NR / 2];
+#pragma unroll
+    for (int ni = 0; ni < NR; ni++) {
+        const int nb = STAGE == 1 ? (ni >> 1) * (p.n_out >> 4) + (n0 >> 4) + wave * 2 + (ni & 1) : (n0 >> 4) + wave * 4 + ni;
+        boff[ni] = (uint32_t)nb * 16u * b_row_bytes + (uint32_t)lane * 16u;
+    }
+#pragma unroll
+    for (int q = 0; q < NR / 2; q++) {
+        const int ch = STAGE == 1 ? q * (p.n_out >> 5) + (n0 >> 5) + wave : (n0 >> 5) + wave * 2 + q;
+        sboff[q] = (uint32_t)ch * chunk_bytes + (uint32_t)lane * 4u;
+    }
+    __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.a_scale + (uint64_t)((blk * TM) >> 5) * chunk_bytes, (uint64_t)(TM >> 5) * chunk_bytes);
+
+    // LDS: row-major AB-byte rows, the 16-byte chunk index XORed with a row-dependent term against bank conflicts
+    auto lds_off = [&](int row, int c) { return row * AB + ((c ^ ((AB == 128 ? (row >> 1) : (row >> 2)) & (CPR - 1))) << 4); };
+    v4i areg[A_LOADS];
+    auto load_a = [&](int kt) {
+        const bool ok = kt < KT;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++) areg[j] = buf_load16(ra, ok ? arow[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
+    };
+    auto store_a = [&](int stage) {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++) {
+            const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
+            if (row < TM) *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, kc)]) = areg[j];
+        }
+    };
+    v4i bw[2][NR];
+    auto load_b = [&](int kt, v4i* dst) {
+        const bool ok = kt < KT;
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) dst[ni] = buf_load16(rb, ok ? boff[ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 1024u : 0u);
+    };
+    int sav[2][MR / 2], sbv[2][NR / 2];
+    auto load_sc = [&](int kc, int* sa_dst, int* sb_dst) {
+        const bool ok = kc < (KT >> 1);
+#pragma unroll
+        for (int q = 0; q < MR / 2; q++) sa_dst[q] = buf_load4(rsa, ok ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u);
+#pragma unroll
+        for (int q = 0; q < NR / 2; q++) sb_dst[q] = buf_load4(rsb, ok ? sboff[q] : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u);
+    };
+    auto read_frag = [&](int stage, int mi) {
+        const int row = mi * 16 + li;
+        v8i v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (AF == MXF_FP4) {
+            const v4i x = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
+            v = __builtin_shufflevector(x, x, 0, 1, 2, 3, -1, -1, -1, -1);
+        } else {
+            const v4i x0 = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, lg)]);
+            const v4i x1 = *reinterpret_cast<const v4i*>(&lds[stage][lds_off(row, 4 + lg)]);
+            v = __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+        return v;
+    };
+
+    v4f acc[MR][NR];
+#pragma unroll
+    for (int mi = 0; mi < MR; mi++)
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // One K step of parity KH (= 128-K half of the current scale chunk): MFMAs on LDS stage KH, W set KH and scale set SET
+    auto step = [&](int kt, auto KHP, auto SETP) __attribute__((always_inline)) {
+        constexpr int KH = decltype(KHP)::value, SET = decltype(SETP)::value;
+        load_a(kt + 1);
+        load_b(kt + 1, bw[KH ^ 1]);
+        if constexpr (KH == 1) load_sc((kt >> 1) + 1, sav[SET ^ 1], sbv[SET ^ 1]);
+        const int* sa_cur = sav[SET];
+        const int* sb_cur = sbv[SET];
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            const v8i af = read_frag(KH, mi);
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                const v4i w4 = bw[KH][ni];
+                const v8i wf = __builtin_shufflevector(w4, w4, 0, 1, 2, 3, -1, -1, -1, -1);
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc[mi][ni], 4, ACODE, KH * 2 + (ni & 1), sb_cur[ni / 2],
+                                                                              KH * 2 + (mi & 1), sa_cur[mi / 2]);
+            });
+        });
+        store_a(KH ^ 1);
+        __syncthreads();
+    };
+
+    load_a(0);
+    load_b(0, bw[0]);
+    load_sc(0, sav[0], sbv[0]);
+    store_a(0);
+    __syncthreads();
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    for (int kt = 0; kt < KT; kt += 4) {  // two scale chunks per trip, so every register index is a constant
+        step(kt, I0{}, I0{});
+        step(kt + 1, I1{}, I0{});
+        if (kt + 2 < KT) {
+            step(kt + 2, I0{}, I1{});
+            step(kt + 3, I1{}, I1{});
+        }
+    }
+
+    if constexpr (STAGE == 1) {
+        // lane (i, g) holds, for row mi*16 + i, gate and up of the columns n0 + wave*32 + ni*16 + 4g + [0, 4), ni = 0, 1:
+        // the 32-column group of this wavefront is spread over the four lanes i, i+16, i+32, i+48
+        const uint32_t out_row_bytes = (uint32_t)p.n_out >> 1;
+        const uint32_t sc_chunk = (uint32_t)(p.n_out >> 8) * 256u;
+        const int c32 = (n0 >> 5) + wave;  // scale column
+        uint8_t* codes = static_cast<uint8_t*>(p.out);
+#pragma unroll
+        for (int mi = 0; mi < MR; mi++) {
+            float y[8];
+            float amax = 0.f;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float g = acc[mi][h][j], u = acc[mi][2 + h][j];
+                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+                    y[h * 4 + j] = g * sig * u;
+                    amax = fmaxf(amax, fabsf(y[h * 4 + j]));
+                }
+            amax = fmaxf(amax, __shfl_xor(amax, 16));
+            amax = fmaxf(amax, __shfl_xor(amax, 32));
+            uint32_t bexp = ((__float_as_uint(amax * (1.0f / 6.0f)) + 0x7FFFFFu) >> 23) & 0xFFu;
+            bexp = bexp < 254u ? bexp : 254u;
+            const float sf = bexp ? __uint_as_float(bexp << 23) : 1.0f;
+            int word = 0;
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, y[0], y[1], sf, 0);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, y[2], y[3], sf, 1);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, y[4], y[5], sf, 2);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, y[6], y[7], sf, 3);
+            const int r = mi * 16 + li;
+            const size_t sr = (size_t)blk * TM + r;
+            uint8_t* dst = codes + sr * out_row_bytes + (uint32_t)((n0 >> 1) + wave * 16 + lg * 2);
+            *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(word & 0xFFFF);
+            *reinterpret_cast<uint16_t*>(dst + 8) = (uint16_t)((uint32_t)word >> 16);
+            if (lg == 0) {
+                const size_t off = ((sr >> 5) * (size_t)sc_chunk) + (size_t)(c32 >> 3) * 256u + (size_t)((c32 & 3) * 16 + li) * 4u + (size_t)(((c32 >> 2) & 1) * 2 + ((r >> 4) & 1));
+                p.out_scale[off] = (uint8_t)bexp;
+            }
+        }
+    } else {
+        const size_t N = (size_t)p.n_out;
+        uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+        for (int mi = 0; mi < MR; mi++) {
+            const int sr = blk * TM + mi * 16 + li;
+            if (p.atomic) {
+                const int t = p.sorted_ids[sr] & 0xFFFFFF;
+                if (t >= p.tokens) continue;
+                const float wgt = p.sorted_w[sr];
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                    const v4f v = acc[mi][ni] * wgt;
+                    uint16_t* o = out + (size_t)t * N + n;
+                    if (p.out_dtype == OUT_BF16) {
+                        const v2i r = pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]);
+                        atomic_add2<OUT_BF16>(o, r[0]);
+                        atomic_add2<OUT_BF16>(o + 2, r[1]);
+                    } else {
+                        const v2i r = pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
+                        atomic_add2<OUT_FP16>(o, r[0]);
+                        atomic_add2<OUT_FP16>(o + 2, r[1]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                    const v4f v = acc[mi][ni];
+                    const v2i r = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]) : pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
+                    *reinterpret_cast<v2i*>(out + (size_t)sr * N + n) = r;
+                }
+            }
+        }
+    }
+}
+
+template <int AF, int STAGE>
+hipError_t launch_rows(const MoeMxParams& p, int block_m, int blocks, hipStream_t stream) {
+    const dim3 grid(p.n_out / (STAGE == 1 ? 128 : 256), blocks);
+    if (block_m == 32) hipLaunchKernelGGL((k_moe_mx<AF, 2, STAGE>), grid, dim3(256), 0, stream, p);
+    else if (block_m == 64) hipLaunchKernelGGL((k_moe_mx<AF, 4, STAGE>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((k_moe_mx<AF, 8, STAGE>), grid, dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// a_format: MXF_FP4 / MXF_FP8 (stage 1 only; stage 2 reads the fp4 rows stage 1 wrote); block_m: 32 / 64 / 128; blocks: blocks of
+// block_m sorted rows the launch covers (blocks past num_valid[0] exit at once)
+hipError_t psg_launch_moe_mx_gemm(const MoeMxParams& p, int a_format, int stage, int block_m, int blocks, hipStream_t stream) {
+    if (stage == 1) return a_format == MXF_FP8 ? launch_rows<MXF_FP8, 1>(p, block_m, blocks, stream) : launch_rows<MXF_FP4, 1>(p, block_m, blocks, stream);
+    return launch_rows<MXF_FP4, 2>(p, block_m, blocks, stream);
+}

@@ -14,6 +14,7 @@
 hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int tile_m, int tile_n, hipStream_t stream);
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
 hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream);
+hipError_t psg_launch_moe_mx_gemm(const MoeMxParams& p, int a_format, int stage, int block_m, int blocks, hipStream_t stream);
 hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream);
 uint64_t psg_moe_sort_workspace(int64_t pairs, int experts);
 int psg_moe_sort_max_experts();
@@ -686,6 +687,59 @@ int moe_reduce_common(const void* x, void* y, const int32_t* mask, const int32_t
     return 0;
 }
 }  // namespace
+
+int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
+    if (!a) return fail(PSG_E_NULL, "args is NULL");
+    if (!a->out || !a->a || !a->a_scale || !a->w || !a->w_scale || !a->sorted_token_ids || !a->sorted_expert_ids || !a->num_valid_ids)
+        return fail(PSG_E_NULL, "out, a, a_scale, w, w_scale, sorted_token_ids, sorted_expert_ids and num_valid_ids must be non-NULL");
+    if (a->stage != 1 && a->stage != 2) return fail(PSG_E_SHAPE, "stage=%d must be 1 or 2", a->stage);
+    if (a->stage == 1 && !a->out_scale) return fail(PSG_E_NULL, "out_scale must be non-NULL in stage 1");
+    if (a->stage == 2 && a->atomic && !a->sorted_weights) return fail(PSG_E_NULL, "sorted_weights must be non-NULL for the atomic epilogue");
+    if (a->pad0 != 0) return fail(PSG_E_SHAPE, "pad0 must be 0");
+    if (a->stage == 1 ? (a->a_dtype != PSG_MX_FP4 && a->a_dtype != PSG_MX_FP8) : a->a_dtype != PSG_MX_FP4)
+        return fail(PSG_E_DTYPE, "a_dtype %d: stage 1 takes 0 (fp4) or 2 (fp8), stage 2 takes 0 (fp4)", a->a_dtype);
+    if (a->stage == 2 && a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
+    if (a->block_m != 32 && a->block_m != 64 && a->block_m != 128) return fail(PSG_E_SHAPE, "block_m=%d must be 32, 64 or 128", a->block_m);
+    if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
+    if (a->experts < 1) return fail(PSG_E_SHAPE, "experts=%d must be positive", a->experts);
+    if (a->model_dim < 256 || a->model_dim % 256) return fail(PSG_E_SHAPE, "model_dim=%d must be a positive multiple of 256", a->model_dim);
+    if (a->inter_dim < 256 || a->inter_dim % 256) return fail(PSG_E_SHAPE, "inter_dim=%d must be a positive multiple of 256", a->inter_dim);
+    if (a->sorted_size < a->block_m) return fail(PSG_E_SHAPE, "sorted_size=%d is below one block of %d rows", a->sorted_size, a->block_m);
+    if (a->blocks < 1 || a->blocks > 65535) return fail(PSG_E_SHAPE, "blocks=%d outside [1, 65535]", a->blocks);
+    if ((int64_t)a->blocks * a->block_m > (int64_t)a->sorted_size)
+        return fail(PSG_E_SHAPE, "blocks=%d of %d rows exceed sorted_size=%d", a->blocks, a->block_m, a->sorted_size);
+    const int K = a->stage == 1 ? a->model_dim : a->inter_dim;
+    const int n_out = a->stage == 1 ? a->inter_dim : a->model_dim;
+    const uint64_t a_row = a->a_dtype == PSG_MX_FP8 ? (uint64_t)K : (uint64_t)K / 2;
+    const uint64_t a_rows = a->stage == 1 ? (uint64_t)a->tokens : (uint64_t)a->sorted_size;
+    const uint64_t rows_e = a->stage == 1 ? 2ull * (uint64_t)n_out : (uint64_t)n_out;
+    if (a_rows * a_row > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "a exceeds the 4 GiB descriptor range");
+    if (rows_e * (uint64_t)(K / 2) > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "one expert's weights exceed the 4 GiB descriptor range");
+    if (!aligned(a->a, 16) || !aligned(a->w, 16) || !aligned(a->a_scale, 4) || !aligned(a->w_scale, 4) || !aligned(a->out, 16))
+        return fail(PSG_E_ALIGN, "a, w and out must be 16-byte aligned, a_scale and w_scale 4-byte aligned");
+    MoeMxParams p;
+    p.out = a->out;
+    p.out_scale = static_cast<uint8_t*>(a->out_scale);
+    p.a = static_cast<const uint8_t*>(a->a);
+    p.a_scale = static_cast<const uint8_t*>(a->a_scale);
+    p.w = static_cast<const uint8_t*>(a->w);
+    p.w_scale = static_cast<const uint8_t*>(a->w_scale);
+    p.sorted_ids = a->sorted_token_ids;
+    p.expert_ids = a->sorted_expert_ids;
+    p.sorted_w = a->sorted_weights;
+    p.num_valid = a->num_valid_ids;
+    p.tokens = a->tokens;
+    p.experts = a->experts;
+    p.n_out = n_out;
+    p.K = K;
+    p.sorted_size = a->sorted_size;
+    p.out_dtype = a->out_dtype;
+    p.atomic = a->stage == 2 && a->atomic ? 1 : 0;
+    const hipError_t e = psg_launch_moe_mx_gemm(p, a->a_dtype == PSG_MX_FP8 ? MXF_FP8 : MXF_FP4, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_mx_gemm launch");
+    g_err[0] = 0;
+    return 0;
+}
 
 int psg_moe_reduce(const void* x, void* y, int32_t tokens, int32_t topk, int32_t model_dim, int32_t dtype, void* stream) {
     return moe_reduce_common(x, y, nullptr, nullptr, tokens, topk, model_dim, 0, dtype, stream);

@@ -172,6 +172,28 @@ struct MoeParams {
     int pair_blocks;            // blocks of 16 / 32 rows: multiply two consecutive blocks of one expert in one workgroup
 };
 
+// Arguments of the MX (fp4 weights, e8m0 scales per 32 K elements) MoE grouped GEMMs over sorted token blocks.
+struct MoeMxParams {
+    void* out;                  // stage 1: packed fp4 codes [sorted_size, inter/2]; stage 2: 16-bit [tokens, model_dim] (atomic) or
+                                // [sorted_size, model_dim] (one row per sorted position, unweighted)
+    uint8_t* out_scale;         // stage 1: e8m0 scales of `out` over sorted rows, shuffled: per (32 rows, 256 columns) 64 dwords
+    const uint8_t* a;           // stage 1: [tokens, K/2] fp4 or [tokens, K] fp8 (gathered by token id); stage 2: [sorted_size, K/2] fp4
+    const uint8_t* a_scale;     // shuffled e8m0 over SORTED rows: 32-row chunks of (K/256)*256 bytes
+    const uint8_t* w;           // preshuffled fp4 [experts * rows_per_expert, K/2] (rows_per_expert = 2*inter: gate rows then up
+                                // rows; or model_dim)
+    const uint8_t* w_scale;     // shuffled e8m0 over the experts * rows_per_expert rows of w
+    const int32_t* sorted_ids;  // (slot << 24) | token per sorted row; padding rows hold token >= tokens
+    const int32_t* expert_ids;  // expert of each block of block_m sorted rows
+    const float* sorted_w;      // routing weight per sorted row (stage 2, atomic)
+    const int32_t* num_valid;   // [0] = number of sorted rows in use (a multiple of block_m)
+    int tokens, experts;
+    int n_out;                  // inter_dim (stage 1) or model_dim (stage 2)
+    int K;                      // model_dim (stage 1) or inter_dim (stage 2)
+    int sorted_size;
+    int out_dtype;              // stage 2: OUT_BF16 / OUT_FP16
+    int atomic;                 // stage 2: weighted atomic add into out[token]
+};
+
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).
 struct MoeSortParams {
     const int32_t* topk_ids;     // [tokens, topk]

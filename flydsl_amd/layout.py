@@ -74,6 +74,46 @@ def shuffle_scale_w4(src: torch.Tensor, experts_cnt: int = 1, gate_up: bool = Fa
     return v.permute(0, 3, 5, 2, 4, 1).contiguous().reshape(r, kb)
 
 
+def e8m0_shuffle(scale: torch.Tensor) -> torch.Tensor:
+    """e8m0 scale bytes ``[R, C]`` padded to ``(ceil(R/256)*256, ceil(C/8)*8)`` and permuted like ``shuffle_scale_w4`` (the
+    reference's ``e8m0_shuffle``, tests/kernels/utils/gemm_common_utils.py:114-136; the padding bytes are zero here, the
+    reference leaves them uninitialised)."""
+    if scale is None or scale.dtype == torch.float32:
+        return scale
+    assert scale.ndim == 2, "scale must be a 2D tensor"
+    r, c = scale.shape
+    pad = torch.zeros((r + 255) // 256 * 256, (c + 7) // 8 * 8, dtype=torch.uint8, device=scale.device)
+    pad[:r, :c] = scale.view(torch.uint8)
+    v = pad.view(pad.shape[0] // 32, 2, 16, pad.shape[1] // 8, 2, 4)
+    return v.permute(0, 3, 5, 2, 4, 1).contiguous().view(pad.shape).view(scale.dtype)
+
+
+def moe_mxfp4_sort(blockscale_e8m0: torch.Tensor, sorted_ids: torch.Tensor, num_valid_ids: torch.Tensor, token_num: int,
+                   block_size: int = 32) -> torch.Tensor:
+    """Scales of the SORTED rows of an MoE stage in the shuffled order its kernel reads (the reference's ``moe_mxfp4_sort``,
+    tests/kernels/utils/gemm_common_utils.py:464-598): row ``i`` of the result's logical ``[rows, C]`` matrix is the scale
+    row of token ``sorted_ids[i] & 0xFFFFFF`` (``[tokens, C]`` input) or of ``token * topk + (sorted_ids[i] >> 24)``
+    (``[tokens, topk, C]`` input); padding rows and rows from ``num_valid_ids[0]`` on are zero (the reference leaves the
+    latter unwritten).  Returns ``[ceil(rows/32)*32, C]`` bytes in the ``e8m0_shuffle`` order; ``C % 8 == 0``."""
+    assert block_size % 32 == 0
+    topk = 1
+    s = blockscale_e8m0.view(torch.uint8)
+    if s.dim() == 3:
+        topk = s.shape[1]
+        s = s.reshape(-1, s.shape[-1])
+    rows_in, c = s.shape
+    assert c % 8 == 0, f"{c} scale columns: a multiple of 8 is required"
+    ids = sorted_ids.to(torch.int64)
+    tok, slot = ids & 0xFFFFFF, (ids >> 24) & 0xFF
+    src = tok if topk == 1 else tok * topk + slot
+    live = (tok < token_num) & (torch.arange(ids.numel(), device=ids.device) < num_valid_ids.reshape(-1)[0].to(ids.device)) & (src < rows_in)
+    rows = (ids.numel() + 31) // 32 * 32
+    out = torch.zeros(rows, c, dtype=torch.uint8, device=s.device)
+    out[: ids.numel()][live] = s[src[live]]
+    v = out.view(rows // 32, 2, 16, c // 8, 2, 4)
+    return v.permute(0, 3, 5, 2, 4, 1).contiguous().view(rows, c)
+
+
 def pack_shuffled_int8_to_int4(x_shuf: torch.Tensor) -> torch.Tensor:
     """Packed int4 weights of the W4A8 MoE stages from PRESHUFFLED int8 values in [-8, 7]: every 8 consecutive values
     ``v0..v7`` become 4 bytes, ``byte j = (v_j & 15) | (v_{j+4} << 4)`` (low nibbles v0..v3, high nibbles v4..v7; the

@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PSG_ABI_VERSION 6
+#define PSG_ABI_VERSION 7
 
 /* input element types of A and B */
 enum psg_in_dtype { PSG_IN_INT8 = 0, PSG_IN_FP8_E4M3FN = 1, PSG_IN_FP16 = 2, PSG_IN_BF16 = 3,
@@ -282,6 +282,51 @@ typedef struct psg_moe_args {
 } psg_moe_args;
 
 int psg_moe_gemm(const psg_moe_args *args, void *stream);
+
+/*
+ * MoE grouped GEMMs with MX operands over expert-sorted token blocks: the two stages of the reference's fused MX-FP4 MoE
+ * (kernels/moe/mxfp_moe/host.py:87-165 flydsl_mxfp4_gemm1, :168-231 flydsl_mxfp4_gemm2).  Weights are fp4 (e2m1 pairs, even
+ * column in the low nibble) in the shuffle_weight order with e8m0 scales per 32 K elements in the e8m0_shuffle order
+ * (tests/kernels/utils/gemm_common_utils.py:114-136), both over all experts * rows.
+ *   stage 1: y[r, n] = silu(g) * u, g = a[t_r] . W1[e, n], u = a[t_r] . W1[e, inter + n] for every sorted row r of token t_r;
+ *            y is quantised per 32 columns as the reference's kernel does (kernels/moe/mxfp_moe/mxfp4_gemm_common.py:221-230: scale byte =
+ *            exponent of the smallest power of two >= amax / 6, at most 254; codes = nearest-even e2m1 of y / 2^(byte-127))
+ *            and written BY SORTED POSITION: out [sorted_size, inter_dim/2] packed codes, out_scale the scales of those
+ *            rows in the e8m0_shuffle order over ceil(sorted_size/256)*256 rows x inter_dim/32 columns.
+ *            a [tokens, model_dim/2] fp4 (a_dtype PSG_MX_FP4) or [tokens, model_dim] e4m3fn (PSG_MX_FP8); a_scale the e8m0 scales
+ *            of the rows of a gathered by sorted position, in the same shuffled order (moe_mxfp4_sort,
+ *            gemm_common_utils.py:464-598); w = W1 [experts * 2*inter_dim, model_dim/2].
+ *   stage 2: y[r, n] = a[r] . W2[e, n] over the sorted rows stage 1 wrote (a = its out, a_scale = its out_scale);
+ *            atomic = 1: out[t_r, n] += y * sorted_weights[r] (out [tokens, model_dim] bf16 / fp16, zeroed by the caller, order
+ *            of the additions not fixed: the reference's "atomic" epilogue); atomic = 0: out[r, n] = y, out [sorted_size,
+ *            model_dim] (its "nonatomic" epilogue: the caller applies the weights); w = W2 [experts * model_dim, inter_dim/2].
+ *   block_m in {32, 64, 128}; model_dim % 256 == 0 and inter_dim % 256 == 0; tokens < 2^24; every operand below 4 GiB.
+ *   sorted_token_ids, sorted_expert_ids, sorted_weights, num_valid_ids as for psg_moe_gemm.
+ */
+typedef struct psg_moe_mx_args {
+    void *out;
+    void *out_scale;     /* stage 1 only */
+    const void *a;
+    const void *a_scale;
+    const void *w;
+    const void *w_scale;
+    const int32_t *sorted_token_ids;
+    const int32_t *sorted_expert_ids;
+    const float *sorted_weights; /* stage 2 with atomic = 1 only */
+    const int32_t *num_valid_ids;
+    int32_t tokens, experts;
+    int32_t model_dim, inter_dim;
+    int32_t sorted_size; /* entries of sorted_token_ids / sorted_weights = rows of the sorted intermediate */
+    int32_t blocks;      /* entries of sorted_expert_ids = grid size along the sorted rows */
+    int32_t block_m;
+    int32_t a_dtype;     /* stage 1: PSG_MX_FP4 or PSG_MX_FP8; stage 2: PSG_MX_FP4 */
+    int32_t out_dtype;   /* stage 2: PSG_OUT_BF16 / PSG_OUT_FP16 */
+    int32_t stage;       /* 1 or 2 */
+    int32_t atomic;      /* stage 2 only */
+    int32_t pad0;        /* 0 */
+} psg_moe_mx_args;
+
+int psg_moe_mx_gemm(const psg_moe_mx_args *args, void *stream);
 
 /* y[t, :] = sum over the topk slots of x[t, slot, :] (fp32 sum in slot order), the pass after stage 2 with accumulate = 0
  * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203 with use_mask = False).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16 / PSG_OUT_F32,

@@ -614,6 +614,128 @@ def moe_gemm2(a2_q, w2_q, scale_a2, scale_w2, topk_ids, topk_weights, model_dim:
 # ----------------------------------------------------------------------------------------------
 
 
+# ----------------------------------------------------------------------------------------------
+# Fused MX-FP4 MoE (kernels/moe/mxfp_moe, tests/kernels/test_moe_gemm.py:540-818)
+# ----------------------------------------------------------------------------------------------
+
+
+def e8m0_shuffle(scale: np.ndarray) -> np.ndarray:
+    """Scale bytes ``[R, C]`` zero-padded to ``(ceil(R/256)*256, ceil(C/8)*8)``, then ``view(R/32, 2, 16, C/8, 2, 4)``
+    permuted to ``(0, 3, 5, 2, 4, 1)`` (tests/kernels/utils/gemm_common_utils.py:114-136).  Pinned by explicit loops over the
+    closed-form offset ``((r/32 * C/8 + c/8) * 4 + c%4) * 64 + (r%16) * 4 + ((c%8)/4) * 2 + (r%32)/16`` and by equality with
+    ``shuffle_scale_w4`` on shapes that need no padding."""
+    sc = np.asarray(scale, dtype=np.uint8)
+    r, c = sc.shape
+    pad = np.zeros(((r + 255) // 256 * 256, (c + 7) // 8 * 8), dtype=np.uint8)
+    pad[:r, :c] = sc
+    v = pad.reshape(pad.shape[0] // 32, 2, 16, pad.shape[1] // 8, 2, 4)
+    return np.ascontiguousarray(v.transpose(0, 3, 5, 2, 4, 1)).reshape(pad.shape)
+
+
+def e8m0_unshuffle(shuf: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    """Inverse of the permutation of ``e8m0_shuffle`` on a flat byte array holding ``rows x cols`` (multiples of 32 and 8)."""
+    v = np.asarray(shuf, dtype=np.uint8).reshape(-1)[: rows * cols].reshape(rows // 32, cols // 8, 4, 16, 2, 2)
+    return np.ascontiguousarray(v.transpose(0, 5, 3, 1, 4, 2)).reshape(rows, cols)
+
+
+def moe_mxfp4_sort(scale: np.ndarray, sorted_ids: np.ndarray, num_valid: int, token_num: int) -> np.ndarray:
+    """Scales gathered by sorted position and shuffled (tests/kernels/utils/gemm_common_utils.py:464-598): logical row ``i``
+    = scale row of token ``sorted_ids[i] & 0xFFFFFF`` (2-D input) or of ``token * topk + (sorted_ids[i] >> 24)`` (3-D input)
+    when the token is below ``token_num`` and ``i < num_valid``, else zero; output ``[ceil(rows/32)*32, C]`` in the 32 x 8
+    blocked order (u32 ``[4][16]`` per block, byte = 16-row half + 2 * 4-column half).  Pinned by explicit loops."""
+    sc = np.asarray(scale, dtype=np.uint8)
+    topk = 1
+    if sc.ndim == 3:
+        topk = sc.shape[1]
+        sc = sc.reshape(-1, sc.shape[-1])
+    ids = np.asarray(sorted_ids).astype(np.int64)
+    rows = (ids.size + 31) // 32 * 32
+    c = sc.shape[1]
+    out = np.zeros((rows, c), dtype=np.uint8)
+    for i in range(min(ids.size, int(num_valid))):
+        tok, slot = int(ids[i]) & 0xFFFFFF, (int(ids[i]) >> 24) & 0xFF
+        if tok < token_num:
+            out[i] = sc[tok if topk == 1 else tok * topk + slot]
+    v = out.reshape(rows // 32, 2, 16, c // 8, 2, 4)
+    return np.ascontiguousarray(v.transpose(0, 3, 5, 2, 4, 1)).reshape(rows, c)
+
+
+def e8m0_roundup(amax: np.ndarray, fmt_max: float = 6.0) -> np.ndarray:
+    """Scale byte of the fused kernels' on-device quantiser: biased exponent of the smallest power of two that is
+    ``>= amax * (1 / fmt_max)`` (fp32 product), at most 254 (kernels/moe/mxfp_moe/mxfp4_gemm_common.py:221-224:
+    ``((bits + 0x7FFFFF) >> 23) & 0xFF``).  Pinned by the defining inequality ``2^(b-128) < amax/fmt_max <= 2^(b-127)`` on
+    random values, exact powers of two and zero."""
+    w = (np.asarray(amax, dtype=np.float32) * np.float32(1.0 / fmt_max)).astype(np.float32).view(np.uint32)
+    b = ((w.astype(np.uint64) + 0x7FFFFF) >> 23) & 0xFF
+    return np.minimum(b, 254).astype(np.uint8)
+
+
+def mxfp4_requant_roundup(y: np.ndarray):
+    """``[R, C]`` fp32 -> (packed e2m1 ``[R, C/2]``, scale bytes ``[R, C/32]``) with ``e8m0_roundup`` scales, the
+    quantiser at the end of the fused stage 1 (kernels/moe/mxfp_moe/gemm1.py:604-613; codes = nearest-even e2m1 of
+    ``y / 2^(byte-127)``, saturating)."""
+    y = np.asarray(y, dtype=np.float32)
+    r, c = y.shape
+    blocks = y.reshape(-1, 32)
+    sc = e8m0_roundup(np.abs(blocks).max(axis=1))
+    sf = np.ldexp(np.float32(1.0), sc.astype(np.int32) - 127).astype(np.float32)
+    q = np.where(sc[:, None] == 0, np.float32(0.0), blocks / np.where(sc == 0, np.float32(1.0), sf)[:, None]).astype(np.float32)
+    return pack_uint4(f32_to_e2m1(q).reshape(r, c)), sc.reshape(r, c // 32)
+
+
+def moe_mx_gemm1(a_q, a_scale, w1_q, w1_scale, sorted_ids, sorted_expert_ids, num_valid: int, tokens: int, inter_dim: int, block_m: int,
+                 a_fmt: str = "fp4"):
+    """Fused stage 1 by sorted position (kernels/moe/mxfp_moe/host.py:87-165; reference result
+    tests/kernels/test_moe_gemm.py:780-784 = ``torch_moe_gemm1`` without routing weights, then a 1x32 fp4 quantisation):
+    for sorted row ``i`` of token ``t`` in a block of expert ``e``: ``g = a[t] . W1[e, :inter]``, ``u = a[t] . W1[e, inter:]``,
+    ``y = silu(g) * u``.  Operands un-shuffled: ``a_q [tokens, K/2 or K]``, ``a_scale [tokens, K/32]``, ``w1_q [E*2*inter, K/2]``,
+    ``w1_scale [E*2*inter, K/32]``.  Returns ``(y fp32 [rows, inter], packed [rows, inter/2], scale [rows, inter/32])`` with
+    zero rows for padding; the quantiser is ``mxfp4_requant_roundup``.  Pinned against ``run_torch_mx`` per (token, expert)
+    pair in token-major order."""
+    ids = np.asarray(sorted_ids).astype(np.int64)
+    rows = ids.size
+    x = mx_operand_to_f32(a_q, a_fmt) * e8m0_to_f32(np.repeat(np.asarray(a_scale, dtype=np.uint8), 32, axis=1))
+    y = np.zeros((rows, inter_dim), dtype=np.float32)
+    for blk in range(min(rows, int(num_valid)) // block_m):
+        e = int(sorted_expert_ids[blk])
+        if e < 0:
+            continue
+        sl = slice(e * 2 * inter_dim, (e + 1) * 2 * inter_dim)
+        w = mxfp4_to_f32(w1_q[sl]) * e8m0_to_f32(np.repeat(np.asarray(w1_scale, dtype=np.uint8)[sl], 32, axis=1))
+        tok = ids[blk * block_m : (blk + 1) * block_m] & 0xFFFFFF
+        live = tok < tokens
+        gu = (x[tok[live]] @ w.T).astype(np.float32)
+        g, u = gu[:, :inter_dim], gu[:, inter_dim:]
+        y[blk * block_m : (blk + 1) * block_m][live] = (g / (1.0 + np.exp(-g.astype(np.float64)))).astype(np.float32) * u
+    packed, sc = mxfp4_requant_roundup(y)
+    return y, packed, sc
+
+
+def moe_mx_gemm2(a2_packed, a2_scale, w2_q, w2_scale, sorted_ids, sorted_weights, sorted_expert_ids, num_valid: int, tokens: int,
+                 model_dim: int, block_m: int):
+    """Fused stage 2 over the sorted fp4 rows (kernels/moe/mxfp_moe/host.py:168-231; reference result
+    tests/kernels/test_moe_gemm.py:785-795): ``flat[i] = a2[i] . W2[e]`` per sorted row, ``out[t] = sum_i weight[i] * flat[i]``
+    over the rows of token ``t``.  Returns ``(flat fp32 [rows, model_dim], out fp32 [tokens, model_dim])``."""
+    ids = np.asarray(sorted_ids).astype(np.int64)
+    rows = ids.size
+    a = mxfp4_to_f32(a2_packed) * e8m0_to_f32(np.repeat(np.asarray(a2_scale, dtype=np.uint8), 32, axis=1))
+    flat = np.zeros((rows, model_dim), dtype=np.float32)
+    out = np.zeros((tokens, model_dim), dtype=np.float32)
+    for blk in range(min(rows, int(num_valid)) // block_m):
+        e = int(sorted_expert_ids[blk])
+        if e < 0:
+            continue
+        sl = slice(e * model_dim, (e + 1) * model_dim)
+        w = mxfp4_to_f32(w2_q[sl]) * e8m0_to_f32(np.repeat(np.asarray(w2_scale, dtype=np.uint8)[sl], 32, axis=1))
+        rs = slice(blk * block_m, (blk + 1) * block_m)
+        flat[rs] = (a[rs] @ w.T).astype(np.float32)
+        for i in range(blk * block_m, (blk + 1) * block_m):
+            t = int(ids[i]) & 0xFFFFFF
+            if t < tokens:
+                out[t] += np.float32(sorted_weights[i]) * flat[i]
+    return flat, out
+
+
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     """fp32 -> bf16 bit pattern (uint16), round-to-nearest-even, NaN kept quiet."""
     u = np.asarray(x, dtype=np.float32).view(np.uint32)

@@ -1,0 +1,157 @@
+"""GPU parity of the fused MX-FP4 MoE stages against the CPU oracle, through the reference's call shapes
+(kernels/moe/mxfp_moe/host.py; the reference's end-to-end check is tests/kernels/test_moe_gemm.py:540-818).
+
+Stage 1 ends in a quantiser, so it is compared in three ways: the scale bytes (equal but for blocks whose maximum sits on a
+power-of-two boundary, where the fp32 summation order decides: at most 0.5 % of the blocks, off by one), the codes (equal for
+at least 99 % of the elements) and the dequantised values against the oracle's unquantised fp32 result (within one scale unit,
+the widest half-step of e2m1, plus 1e-3 relative).  Stage 2 is checked on the DEVICE's stage-1 output, so its own error is
+what is measured: |out-ref| <= 1e-2*|ref| + 1e-2*max|ref| for one row per sorted position, 3e-2*max|ref| for the atomic
+epilogue (its 16-bit additions round in arrival order)."""
+
+import numpy as np
+import pytest
+import torch
+
+from flydsl_amd import layout
+from kernels.moe.mxfp_moe import flydsl_mxfp4_gemm1, flydsl_mxfp4_gemm2
+from oracle import psg_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(tokens, model_dim, inter, experts, topk, bm, a_fmt, seed, hot_expert=False):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((tokens, model_dim)).astype(np.float32)
+    w1 = (rng.standard_normal((experts * 2 * inter, model_dim)) / np.sqrt(model_dim)).astype(np.float32)
+    w2 = (rng.standard_normal((experts * model_dim, inter)) / np.sqrt(inter)).astype(np.float32)
+    a_q, a_s = O.per_1x32_f4_quant(x) if a_fmt == "fp4" else O.per_1x32_f8_quant(x)
+    w1_q, w1_s = O.per_1x32_f4_quant(w1)
+    w2_q, w2_s = O.per_1x32_f4_quant(w2)
+    ids = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    if hot_expert:
+        ids[:, 0] = 1  # every token also goes to expert 1: several blocks of one expert
+        ids[:, 1:] = np.where(ids[:, 1:] == 1, 0, ids[:, 1:])
+    wts = rng.uniform(0.1, 1.0, size=(tokens, topk)).astype(np.float32)
+    return dict(a_q=a_q, a_s=a_s[:tokens], w1_q=w1_q, w1_s=w1_s, w2_q=w2_q, w2_s=w2_s, ids=ids, wts=wts, sort=O.moe_sorting(ids, wts, experts, bm))
+
+
+def _device_inputs(p, tokens, bm, dev):
+    sid, sw, se, npp = p["sort"]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    d = dict(a=t(p["a_q"]), w1=t(O.shuffle_weight_w4(p["w1_q"])), w2=t(O.shuffle_weight_w4(p["w2_q"])),
+             w1_s=layout.e8m0_shuffle(t(p["w1_s"])), w2_s=layout.e8m0_shuffle(t(p["w2_s"])),
+             sid=t(sid), sw=t(sw), se=t(se), cumsum=t(npp[:1].astype(np.int32)))
+    d["a_s"] = layout.moe_mxfp4_sort(t(p["a_s"]).view(tokens, 1, -1), d["sid"], d["cumsum"], tokens, block_size=bm)
+    return d
+
+
+def _stage1(p, d, tokens, model_dim, inter, experts, topk, bm, a_fmt, dev):
+    rows = int(d["sid"].numel())
+    codes = torch.full((rows, inter // 2), 0x77, dtype=torch.uint8, device=dev)
+    scales = torch.full(((rows + 255) // 256 * 256 * (inter // 32),), 0x77, dtype=torch.uint8, device=dev)
+    flydsl_mxfp4_gemm1(a_quant=d["a"], a_scale_sorted_shuffled=d["a_s"], w1_u8=d["w1"], w1_scale_u8=d["w1_s"], sorted_expert_ids=d["se"],
+                       cumsum_tensor=d["cumsum"], m_indices=d["sid"], inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales,
+                       hidden_states=None, n_tokens=tokens, BM=bm, use_nt=bm == 32, inline_quant=False, NE=experts, D_HIDDEN=model_dim,
+                       D_INTER=inter, topk=topk, a_dtype=a_fmt)
+    torch.cuda.synchronize()
+    return codes, scales
+
+
+def _check_stage1(p, codes, scales, tokens, inter, bm, a_fmt):
+    sid, sw, se, npp = p["sort"]
+    nv = int(npp[0])
+    y, want_q, want_s = O.moe_mx_gemm1(p["a_q"], p["a_s"], p["w1_q"], p["w1_s"], sid, se, nv, tokens, inter, bm, a_fmt)
+    got_q = codes.cpu().numpy()
+    rows32 = (sid.size + 31) // 32 * 32
+    got_s = O.e8m0_unshuffle(scales.cpu().numpy(), rows32, inter // 32)
+    assert np.all(got_q[nv:] == 0x77), "rows past num_valid must stay untouched"
+    live = (sid[:nv] & 0xFFFFFF) < tokens
+    assert not got_q[:nv][~live].any() and not got_s[:nv][~live].any(), "padding rows hold zero codes and zero scales"
+    ds = got_s[:nv][live].astype(np.int32) - want_s[:nv][live].astype(np.int32)
+    assert np.abs(ds).max() <= 1 and np.mean(ds != 0) <= 5e-3, (np.abs(ds).max(), np.mean(ds != 0))
+    assert np.mean(got_q[:nv][live] == want_q[:nv][live]) >= 0.99
+    unit = np.repeat(np.ldexp(1.0, got_s[:nv].astype(np.int32) - 127), 32, axis=1) * (got_s[:nv] != 0).repeat(32, axis=1)
+    deq = O.mxfp4_to_f32(got_q[:nv]) * unit
+    assert np.all(np.abs(deq - y[:nv]) <= unit * 1.0 + 1e-3 * np.abs(y[:nv]) + 1e-30)
+    return got_q, got_s
+
+
+@pytest.mark.parametrize("a_fmt", ["fp4", "fp8"])
+@pytest.mark.parametrize("bm", [32, 64, 128])
+def test_fused_stages_match_the_oracle(bm, a_fmt):
+    tokens, model_dim, inter, experts, topk = 70, 512, 256, 5, 2
+    dev = torch.device("cuda")
+    p = _problem(tokens, model_dim, inter, experts, topk, bm, a_fmt, seed=bm + len(a_fmt), hot_expert=True)
+    d = _device_inputs(p, tokens, bm, dev)
+    codes, scales = _stage1(p, d, tokens, model_dim, inter, experts, topk, bm, a_fmt, dev)
+    got_q, got_s = _check_stage1(p, codes, scales, tokens, inter, bm, a_fmt)
+    sid, sw, se, npp = p["sort"]
+    nv, rows = int(npp[0]), sid.size
+    clean_q, clean_s = got_q.copy(), got_s.copy()
+    clean_q[nv:], clean_s[nv:] = 0, 0
+    flat_ref, out_ref = O.moe_mx_gemm2(clean_q, clean_s[:rows], p["w2_q"], p["w2_s"], sid, sw, se, nv, tokens, model_dim, bm)
+    common = dict(inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales, w2_u8=d["w2"], w2_scale_u8=d["w2_s"], sorted_expert_ids=d["se"],
+                  cumsum_tensor=d["cumsum"], sorted_token_ids=d["sid"], sorted_weights=d["sw"], M_logical=tokens, max_sorted=rows, BM=bm,
+                  NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+    for dt in (torch.bfloat16, torch.float16):
+        flat = torch.full((rows, model_dim), 7.0, dtype=dt, device=dev)
+        flydsl_mxfp4_gemm2(flat_out=flat, use_nt=False, epilog="nonatomic", **common)
+        out = torch.zeros(tokens, model_dim, dtype=dt, device=dev)
+        flydsl_mxfp4_gemm2(flat_out=out, use_nt=True, epilog="atomic", **common)
+        torch.cuda.synchronize()
+        f = flat.float().cpu().numpy()
+        assert np.all(f[nv:] == 7.0)
+        live = (sid[:nv] & 0xFFFFFF) < tokens
+        tol = 1e-2 * np.abs(flat_ref[:nv][live]) + 1e-2 * np.abs(flat_ref).max()
+        assert np.all(np.abs(f[:nv][live] - flat_ref[:nv][live]) <= tol)
+        o = out.float().cpu().numpy()
+        assert np.abs(o - out_ref).max() <= 3e-2 * np.abs(out_ref).max(), np.abs(o - out_ref).max() / np.abs(out_ref).max()
+
+
+def test_blocks_of_masked_experts_are_skipped_and_longer_dims_work():
+    tokens, model_dim, inter, experts, topk, bm = 33, 1024, 512, 4, 2, 32
+    dev = torch.device("cuda")
+    p = _problem(tokens, model_dim, inter, experts, topk, bm, "fp4", seed=9)
+    sid, sw, se, npp = p["sort"]
+    se = se.copy()
+    masked = int(se[0])
+    se[se == masked] = -1  # expert parallelism: blocks of experts that live elsewhere carry -1
+    p["sort"] = (sid, sw, se, npp)
+    d = _device_inputs(p, tokens, bm, dev)
+    codes, scales = _stage1(p, d, tokens, model_dim, inter, experts, topk, bm, "fp4", dev)
+    got_q = codes.cpu().numpy()
+    nv = int(npp[0])
+    skipped = np.repeat(se[: nv // bm] < 0, bm)
+    assert np.all(got_q[:nv][skipped] == 0x77), "blocks of a masked expert are not written"
+    y, want_q, want_s = O.moe_mx_gemm1(p["a_q"], p["a_s"], p["w1_q"], p["w1_s"], sid, se, nv, tokens, inter, bm, "fp4")
+    assert np.mean(got_q[:nv][~skipped] == want_q[:nv][~skipped]) >= 0.99
+    out = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+    flydsl_mxfp4_gemm2(inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales, w2_u8=d["w2"], w2_scale_u8=d["w2_s"], sorted_expert_ids=d["se"],
+                       cumsum_tensor=d["cumsum"], sorted_token_ids=d["sid"], sorted_weights=d["sw"], flat_out=out, M_logical=tokens,
+                       max_sorted=sid.size, BM=bm, use_nt=True, epilog="atomic", NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+    torch.cuda.synchronize()
+    got_s = O.e8m0_unshuffle(scales.cpu().numpy(), (sid.size + 31) // 32 * 32, inter // 32)
+    q, s = got_q.copy(), got_s.copy()
+    q[nv:], s[nv:] = 0, 0
+    q[:nv][skipped], s[:nv][skipped] = 0, 0
+    _, out_ref = O.moe_mx_gemm2(q, s[: sid.size], p["w2_q"], p["w2_s"], sid, sw, se, nv, tokens, model_dim, bm)
+    assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * np.abs(out_ref).max()
+
+
+def test_unbuilt_variants_raise_like_the_reference():
+    dev = torch.device("cuda")
+    z = torch.zeros(64, dtype=torch.uint8, device=dev)
+    base = dict(a_quant=z, a_scale_sorted_shuffled=z, w1_u8=z, w1_scale_u8=z, sorted_expert_ids=z, cumsum_tensor=z, m_indices=z,
+                inter_sorted_quant=z, inter_sorted_shuffled_scale=z, hidden_states=z, n_tokens=4, use_nt=False, NE=2, D_HIDDEN=512, D_INTER=256, topk=1)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm1(BM=16, inline_quant=True, **base)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm1(BM=32, inline_quant=False, interleave=True, **base)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm1(BM=32, inline_quant=False, **{**base, "D_HIDDEN": 384})
+    g2 = dict(inter_sorted_quant=z, inter_sorted_shuffled_scale=z, w2_u8=z, w2_scale_u8=z, sorted_expert_ids=z, cumsum_tensor=z, sorted_token_ids=z,
+              sorted_weights=z, flat_out=z, M_logical=4, max_sorted=32, BM=32, use_nt=False, NE=2, D_HIDDEN=512, D_INTER=256, topk=1)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm2(epilog="nonatomic_mxfp4", **g2)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm2(epilog="atomic", **{**g2, "D_INTER": 320})

@@ -388,6 +388,8 @@ def test_struct_layouts_match_header():
                offsetof(psg_moe_sort_args, blocks));
         printf("%zu %zu %zu %zu\n", sizeof(psg_moe_gating_args), offsetof(psg_moe_gating_args, token_expert_indices),
                offsetof(psg_moe_gating_args, tokens), offsetof(psg_moe_gating_args, renormalize));
+        printf("%zu %zu %zu %zu\n", sizeof(psg_moe_mx_args), offsetof(psg_moe_mx_args, num_valid_ids), offsetof(psg_moe_mx_args, tokens),
+               offsetof(psg_moe_mx_args, atomic));
         return 0;
     }'''
     with tempfile.TemporaryDirectory() as d:
@@ -406,7 +408,32 @@ def test_struct_layouts_match_header():
     want += [ctypes.sizeof(so), so.workspace_bytes.offset, so.tokens.offset, so.blocks.offset]
     ga = _lib.MoeGatingArgs
     want += [ctypes.sizeof(ga), ga.token_expert_indices.offset, ga.tokens.offset, ga.renormalize.offset]
+    mx = _lib.MoeMxArgs
+    want += [ctypes.sizeof(mx), mx.num_valid_ids.offset, mx.tokens.offset, mx.atomic.offset]
     assert [int(v) for v in out] == want
+
+
+def test_mx_moe_validation_errors_without_a_gpu():
+    handle = _lib.lib()
+    assert handle.psg_moe_mx_gemm(None, None) == -1
+
+    def args(**kw):
+        a = _lib.MoeMxArgs()
+        for f in ("out", "out_scale", "a", "a_scale", "w", "w_scale", "sorted_token_ids", "sorted_expert_ids", "sorted_weights", "num_valid_ids"):
+            setattr(a, f, 0x10000)
+        a.tokens, a.experts, a.model_dim, a.inter_dim, a.sorted_size, a.blocks, a.block_m = 8, 2, 512, 256, 128, 4, 32
+        a.a_dtype, a.out_dtype, a.stage, a.atomic, a.pad0 = 0, 0, 1, 0, 0
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    bad = [dict(stage=3), dict(block_m=16), dict(model_dim=384), dict(inter_dim=128), dict(a_dtype=1), dict(stage=2, a_dtype=2), dict(stage=2, out_dtype=2),
+           dict(blocks=5), dict(blocks=0), dict(tokens=0), dict(experts=0), dict(pad0=1), dict(out_scale=None), dict(stage=2, atomic=1, sorted_weights=None),
+           dict(a=0x10008), dict(w=None), dict(sorted_size=16)]
+    for kw in bad:
+        a = args(**kw)
+        assert handle.psg_moe_mx_gemm(ctypes.byref(a), None) != 0, kw
+        assert handle.psg_last_error()
 
 
 def test_gating_validation_errors_without_a_gpu():
