@@ -339,6 +339,34 @@ def run_next_row_workloads():
                     "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s1 / 1e9})
         out.append({"workload": f"moe_w4a8_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
                     "weight_gb_per_s": experts * model_dim * inter_dim / 2 / s2 / 1e9})
+    # the fused MX-FP4 stages (fp4 activations and weights, one e8m0 scale per 32 elements; stage 1 quantises its output again and writes
+    # it by sorted position, stage 2 adds weight * row into the token's output row); blocks of at least 32 sorted rows
+    from kernels.moe.mxfp_moe import flydsl_mxfp4_gemm1, flydsl_mxfp4_gemm2
+
+    for tokens, model_dim, inter_dim, experts, topk, bm in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 32)):
+        g = torch.Generator().manual_seed(0)
+        vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
+        sid, swt, se, npp = moe_sorting(ids.int().to(dev), torch.softmax(vals, 1).to(dev), num_experts=experts, block_size=bm)
+        rows = int(sid.numel())
+        rb = lambda *shape: torch.randint(0, 256, shape, dtype=torch.uint8, generator=g).to(dev)  # noqa: E731
+        sc = lambda n: torch.randint(120, 130, (n,), dtype=torch.uint8, generator=g).to(dev)  # noqa: E731
+        a4, a4s = rb(tokens, model_dim // 2), sc((rows + 31) // 32 * 32 * (model_dim // 32))
+        w1m, w1s = rb(experts * 2 * inter_dim, model_dim // 2), sc(experts * 2 * inter_dim * (model_dim // 32))
+        w2m, w2s = rb(experts * model_dim, inter_dim // 2), sc(experts * model_dim * (inter_dim // 32))
+        iq = torch.zeros(rows, inter_dim // 2, dtype=torch.uint8, device=dev)
+        iqs = torch.zeros((rows + 255) // 256 * 256 * (inter_dim // 32), dtype=torch.uint8, device=dev)
+        outm = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+        nv = npp[:1].contiguous()
+        kw = dict(sorted_expert_ids=se, cumsum_tensor=nv, BM=bm, NE=experts, D_HIDDEN=model_dim, D_INTER=inter_dim, topk=topk)
+        s1 = timed(lambda: flydsl_mxfp4_gemm1(a_quant=a4, a_scale_sorted_shuffled=a4s, w1_u8=w1m, w1_scale_u8=w1s, m_indices=sid, inter_sorted_quant=iq,
+                                              inter_sorted_shuffled_scale=iqs, n_tokens=tokens, **kw))
+        s2 = timed(lambda: flydsl_mxfp4_gemm2(inter_sorted_quant=iq, inter_sorted_shuffled_scale=iqs, w2_u8=w2m, w2_scale_u8=w2s, sorted_token_ids=sid,
+                                              sorted_weights=swt, flat_out=outm, M_logical=tokens, max_sorted=rows, epilog="atomic", **kw))
+        tag = f"tokens{tokens}_e{experts}_top{topk}_model{model_dim}_inter{inter_dim}_block{bm}"
+        out.append({"workload": f"moe_mxfp4_stage1_{tag}", "us_per_launch_events": s1 * 1e6, "tflops": 2.0 * tokens * topk * 2 * inter_dim * model_dim / s1 / 1e12,
+                    "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s1 / 1e9})
+        out.append({"workload": f"moe_mxfp4_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
+                    "weight_gb_per_s": experts * model_dim * inter_dim / 2 / s2 / 1e9})
     # the device-side expert sorter in front of the stages (outputs pre-allocated, accumulate buffer cleared by the same launch)
     for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)):
         g = torch.Generator().manual_seed(0)

@@ -29,7 +29,7 @@ __device__ __forceinline__ void atomic_add2(uint16_t* o, int bits) {
 }
 
 template <int AF, int MR, int STAGE>
-__global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 4 ? 2 : 1))) k_moe_mx(MoeMxParams p) {
     static_assert(MR % 2 == 0, "scale chunks cover 32 rows");
     constexpr int NR = 4;
     constexpr int TM = 16 * MR;
@@ -38,11 +38,14 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
     constexpr int CPR = AB / 16;                   // 16-byte chunks per staged row
     constexpr int A_LOADS = (TM * CPR + 255) / 256;
     constexpr int ACODE = AF == MXF_FP4 ? 4 : 0;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][TM * AB];
+    constexpr int EPI_BYTES = TM * (STAGE == 1 ? 64 : 512);  // the epilogue's tile: TM rows of 64 code bytes or 256 16-bit values
+    constexpr int LDS_BYTES = 2 * TM * AB > EPI_BYTES ? 2 * TM * AB : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    uint8_t(*lds)[TM * AB] = reinterpret_cast<uint8_t(*)[TM * AB]>(lds_raw);
 
-    const int blk = blockIdx.y;
+    const int blk = blockIdx.y;  // block of TM sorted rows; the sorter's blocks hold TM << eshift rows
     if (blk * TM >= p.num_valid[0]) return;
-    const int e = p.expert_ids[blk];
+    const int e = p.expert_ids[blk >> p.eshift];
     if ((unsigned)e >= (unsigned)p.experts) return;
 
     const int tid = threadIdx.x;
@@ -86,20 +89,23 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
 
     // LDS: row-major AB-byte rows, the 16-byte chunk index XORed with a row-dependent term against bank conflicts
     auto lds_off = [&](int row, int c) { return row * AB + ((c ^ ((AB == 128 ? (row >> 1) : (row >> 2)) & (CPR - 1))) << 4); };
-    v4i areg[A_LOADS];
-    auto load_a = [&](int kt) {
+    // Loads run PF steps ahead of the MFMAs in rings of RING register sets: one step of a 64-row tile is 256 MFMA cycles per
+    // wavefront, far less than the latency of a load from HBM
+    constexpr int RING = AF == MXF_FP4 ? 4 : 2, PF = RING - 1;
+    v4i areg[RING][A_LOADS];
+    auto load_a = [&](int kt, v4i* dst) {
         const bool ok = kt < KT;
 #pragma unroll
-        for (int j = 0; j < A_LOADS; j++) areg[j] = buf_load16(ra, ok ? arow[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
+        for (int j = 0; j < A_LOADS; j++) dst[j] = buf_load16(ra, ok ? arow[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
     };
-    auto store_a = [&](int stage) {
+    auto store_a = [&](int stage, const v4i* src) {
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
             const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
-            if (row < TM) *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, kc)]) = areg[j];
+            if (row < TM) *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, kc)]) = src[j];
         }
     };
-    v4i bw[2][NR];
+    v4i bw[RING][NR];
     auto load_b = [&](int kt, v4i* dst) {
         const bool ok = kt < KT;
 #pragma unroll
@@ -133,12 +139,13 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    // One K step of parity KH (= 128-K half of the current scale chunk): MFMAs on LDS stage KH, W set KH and scale set SET
-    auto step = [&](int kt, auto KHP, auto SETP) __attribute__((always_inline)) {
-        constexpr int KH = decltype(KHP)::value, SET = decltype(SETP)::value;
-        load_a(kt + 1);
-        load_b(kt + 1, bw[KH ^ 1]);
-        if constexpr (KH == 1) load_sc((kt >> 1) + 1, sav[SET ^ 1], sbv[SET ^ 1]);
+    // One K step of parity KH (= 128-K half of the current scale chunk): MFMAs on LDS stage KH, W set WS = kt % RING and scale
+    // set SET; requests the operands of step kt + PF and the scales of the next chunk, stages the A rows of step kt + 1
+    auto step = [&](int kt, auto KHP, auto SETP, auto WSP) __attribute__((always_inline)) {
+        constexpr int KH = decltype(KHP)::value, SET = decltype(SETP)::value, WS = decltype(WSP)::value;
+        load_a(kt + PF, areg[(WS + PF) % RING]);
+        load_b(kt + PF, bw[(WS + PF) % RING]);
+        if constexpr (KH == 0) load_sc((kt >> 1) + 1, sav[SET ^ 1], sbv[SET ^ 1]);
         const int* sa_cur = sav[SET];
         const int* sb_cur = sbv[SET];
         static_for<MR>([&](auto MI) {
@@ -146,29 +153,34 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
             const v8i af = read_frag(KH, mi);
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
-                const v4i w4 = bw[KH][ni];
+                const v4i w4 = bw[WS][ni];
                 const v8i wf = __builtin_shufflevector(w4, w4, 0, 1, 2, 3, -1, -1, -1, -1);
                 acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc[mi][ni], 4, ACODE, KH * 2 + (ni & 1), sb_cur[ni / 2],
                                                                               KH * 2 + (mi & 1), sa_cur[mi / 2]);
             });
         });
-        store_a(KH ^ 1);
+        store_a(KH ^ 1, areg[(WS + 1) % RING]);
         __syncthreads();
     };
 
-    load_a(0);
-    load_b(0, bw[0]);
-    load_sc(0, sav[0], sbv[0]);
-    store_a(0);
-    __syncthreads();
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2 % RING>;
+    using I3 = std::integral_constant<int, 3 % RING>;
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        load_a(i, areg[i]);
+        load_b(i, bw[i]);
+    }
+    load_sc(0, sav[0], sbv[0]);
+    store_a(0, areg[0]);
+    __syncthreads();
     for (int kt = 0; kt < KT; kt += 4) {  // two scale chunks per trip, so every register index is a constant
-        step(kt, I0{}, I0{});
-        step(kt + 1, I1{}, I0{});
+        step(kt, I0{}, I0{}, I0{});
+        step(kt + 1, I1{}, I0{}, I1{});
         if (kt + 2 < KT) {
-            step(kt + 2, I0{}, I1{});
-            step(kt + 3, I1{}, I1{});
+            step(kt + 2, I0{}, I1{}, I2{});
+            step(kt + 3, I1{}, I1{}, I3{});
         }
     }
 
@@ -204,7 +216,8 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
             word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, y[6], y[7], sf, 3);
             const int r = mi * 16 + li;
             const size_t sr = (size_t)blk * TM + r;
-            uint8_t* dst = codes + sr * out_row_bytes + (uint32_t)((n0 >> 1) + wave * 16 + lg * 2);
+            // the tile's codes go through LDS (64 bytes per row, free after the loop's last barrier) so that they leave in 16-byte pieces
+            uint8_t* dst = lds_raw + r * 64 + wave * 16 + lg * 2;
             *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(word & 0xFFFF);
             *reinterpret_cast<uint16_t*>(dst + 8) = (uint16_t)((uint32_t)word >> 16);
             if (lg == 0) {
@@ -212,50 +225,59 @@ __global__ void __launch_bounds__(256) k_moe_mx(MoeMxParams p) {
                 p.out_scale[off] = (uint8_t)bexp;
             }
         }
+        __syncthreads();
+        for (int q = tid; q < TM * 4; q += 256) {
+            const int r = q >> 2, c = q & 3;
+            *reinterpret_cast<v4i*>(codes + ((size_t)blk * TM + r) * out_row_bytes + (uint32_t)((n0 >> 1) + c * 16)) = *reinterpret_cast<const v4i*>(lds_raw + r * 64 + c * 16);
+        }
     } else {
+        // The tile goes through LDS as 16-bit values (512 bytes per row, 16-byte granules XOR-swizzled by the row; the A stages are
+        // free after the loop's last barrier); then the workgroup walks it row by row, so that one store or atomic instruction
+        // covers 256 or 1024 contiguous bytes of the output instead of 16 rows x 8 bytes.
         const size_t N = (size_t)p.n_out;
         uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) {
-            const int sr = blk * TM + mi * 16 + li;
-            if (p.atomic) {
-                const int t = p.sorted_ids[sr] & 0xFFFFFF;
+            const int r = mi * 16 + li;
+            const float wgt = p.atomic ? p.sorted_w[blk * TM + r] : 1.0f;
+#pragma unroll
+            for (int ni = 0; ni < NR; ni++) {
+                const int cb = ((wave * NR + ni) * 16 + lg * 4) * 2;
+                const v4f v = acc[mi][ni] * wgt;
+                const v2i pk = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]) : pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<v2i*>(lds_raw + r * 512 + ((((cb >> 4) ^ r) & 31) << 4) + (cb & 15)) = pk;
+            }
+        }
+        __syncthreads();
+        if (p.atomic) {
+            for (int q = tid; q < TM * 128; q += 256) {
+                const int r = q >> 7, cb = (q & 127) * 4;
+                const int t = p.sorted_ids[blk * TM + r] & 0xFFFFFF;
                 if (t >= p.tokens) continue;
-                const float wgt = p.sorted_w[sr];
-#pragma unroll
-                for (int ni = 0; ni < NR; ni++) {
-                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-                    const v4f v = acc[mi][ni] * wgt;
-                    uint16_t* o = out + (size_t)t * N + n;
-                    if (p.out_dtype == OUT_BF16) {
-                        const v2i r = pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]);
-                        atomic_add2<OUT_BF16>(o, r[0]);
-                        atomic_add2<OUT_BF16>(o + 2, r[1]);
-                    } else {
-                        const v2i r = pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
-                        atomic_add2<OUT_FP16>(o, r[0]);
-                        atomic_add2<OUT_FP16>(o + 2, r[1]);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int ni = 0; ni < NR; ni++) {
-                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-                    const v4f v = acc[mi][ni];
-                    const v2i r = p.out_dtype == OUT_BF16 ? pack4_out16<OUT_BF16>(v[0], v[1], v[2], v[3]) : pack4_out16<OUT_FP16>(v[0], v[1], v[2], v[3]);
-                    *reinterpret_cast<v2i*>(out + (size_t)sr * N + n) = r;
-                }
+                const int bits = *reinterpret_cast<const int*>(lds_raw + r * 512 + ((((cb >> 4) ^ r) & 31) << 4) + (cb & 15));
+                uint16_t* o = out + (size_t)t * N + n0 + (cb >> 1);
+                if (p.out_dtype == OUT_BF16) atomic_add2<OUT_BF16>(o, bits);
+                else atomic_add2<OUT_FP16>(o, bits);
+            }
+        } else {
+            for (int q = tid; q < TM * 32; q += 256) {
+                const int r = q >> 5, g = q & 31;
+                *reinterpret_cast<v4i*>(out + ((size_t)blk * TM + r) * N + n0 + g * 8) = *reinterpret_cast<const v4i*>(lds_raw + r * 512 + (((g ^ r) & 31) << 4));
             }
         }
     }
 }
 
+// Blocks of 128 sorted rows run as two workgroups of 64 rows each: a 128-row tile needs every register of the wavefront for its
+// accumulators, so one workgroup per CU would run with nothing to overlap its loads and its epilogue with (measured, 4096
+// tokens x top-8 on 32 experts, 4096 x 1536: stage 1 399 us with 128-row tiles against 339 with 64-row tiles, stage 2 with the
+// atomic epilogue 667 against 434).
 template <int AF, int STAGE>
-hipError_t launch_rows(const MoeMxParams& p, int block_m, int blocks, hipStream_t stream) {
-    const dim3 grid(p.n_out / (STAGE == 1 ? 128 : 256), blocks);
+hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t stream) {
+    p.eshift = block_m == 128 ? 1 : 0;
+    const dim3 grid(p.n_out / (STAGE == 1 ? 128 : 256), blocks << p.eshift);
     if (block_m == 32) hipLaunchKernelGGL((k_moe_mx<AF, 2, STAGE>), grid, dim3(256), 0, stream, p);
-    else if (block_m == 64) hipLaunchKernelGGL((k_moe_mx<AF, 4, STAGE>), grid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((k_moe_mx<AF, 8, STAGE>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((k_moe_mx<AF, 4, STAGE>), grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -735,6 +735,8 @@ int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     p.sorted_size = a->sorted_size;
     p.out_dtype = a->out_dtype;
     p.atomic = a->stage == 2 && a->atomic ? 1 : 0;
+    p.eshift = 0;
+    if (((int64_t)a->blocks << 1) > 65535 && a->block_m == 128) return fail(PSG_E_SHAPE, "blocks=%d of 128 rows exceed the grid", a->blocks);
     const hipError_t e = psg_launch_moe_mx_gemm(p, a->a_dtype == PSG_MX_FP8 ? MXF_FP8 : MXF_FP4, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_mx_gemm launch");
     g_err[0] = 0;

@@ -192,6 +192,7 @@ struct MoeMxParams {
     int sorted_size;
     int out_dtype;              // stage 2: OUT_BF16 / OUT_FP16
     int atomic;                 // stage 2: weighted atomic add into out[token]
+    int eshift;                 // set by the launcher: log2(sorter block rows / rows per workgroup)
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).
