@@ -28,19 +28,24 @@ __device__ __forceinline__ void atomic_add2(uint16_t* o, int bits) {
     else __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) v2h*)o, __builtin_bit_cast(v2h, bits));
 }
 
-template <int AF, int MR, int STAGE>
+// IQ (stage 1, 16-row blocks): `a` holds bf16 activations [tokens, K]; every 32 of them are quantised to fp4 on their way into
+// LDS with the same scale rule as the output (kernels/moe/mxfp_moe/gemm1.py:324-412), and no A-side scales are read.
+template <int AF, int MR, int STAGE, bool IQ = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 4 ? 2 : 1))) k_moe_mx(MoeMxParams p) {
-    static_assert(MR % 2 == 0, "scale chunks cover 32 rows");
+    static_assert(MR % 2 == 0 || MR == 1, "scale chunks cover 32 rows; a single 16-row block picks its half at run time");
+    static_assert(!IQ || (MR == 1 && STAGE == 1 && AF == MXF_FP4), "inline quantisation: 16-row blocks of stage 1");
     constexpr int NR = 4;
     constexpr int TM = 16 * MR;
     constexpr int TN = STAGE == 1 ? 128 : 256;     // output columns per workgroup
     constexpr int AB = AF == MXF_FP4 ? 64 : 128;   // bytes of an A row per K step
     constexpr int CPR = AB / 16;                   // 16-byte chunks per staged row
-    constexpr int A_LOADS = (TM * CPR + 255) / 256;
+    constexpr int A_LOADS = IQ ? 1 : (TM * CPR + 255) / 256;
+    constexpr int SC = (MR + 1) / 2;               // A-side scale dwords per 256-K chunk
     constexpr int ACODE = AF == MXF_FP4 ? 4 : 0;
     constexpr int EPI_BYTES = TM * (STAGE == 1 ? 64 : 512);  // the epilogue's tile: TM rows of 64 code bytes or 256 16-bit values
     constexpr int LDS_BYTES = 2 * TM * AB > EPI_BYTES ? 2 * TM * AB : EPI_BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    __shared__ uint8_t iq_scale[2][IQ ? 64 : 1];   // IQ: scale byte of (row, 32-element group) of each LDS stage
     uint8_t(*lds)[TM * AB] = reinterpret_cast<uint8_t(*)[TM * AB]>(lds_raw);
 
     const int blk = blockIdx.y;  // block of TM sorted rows; the sorter's blocks hold TM << eshift rows
@@ -60,15 +65,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
 
     // A: stage 1 gathers token rows, stage 2 reads the block's sorted rows; rows without a token read as zero
     const int a_rows = STAGE == 1 ? p.tokens : p.sorted_size;
-    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)a_rows * a_row_bytes);
+    const uint32_t a_src_bytes = IQ ? (uint32_t)p.K * 2u : a_row_bytes;  // bytes of a row of `a`
+    constexpr uint32_t A_STEP = IQ ? 256u : (uint32_t)AB;                // ... and of one K step of it
+    __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)a_rows * a_src_bytes);
     uint32_t arow[A_LOADS];
 #pragma unroll
     for (int j = 0; j < A_LOADS; j++) {
-        const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
+        // IQ: thread t takes 8 bf16 (16 bytes) of row t / 16: four neighbouring lanes hold one 32-element group
+        const int c = tid + 256 * j, row = IQ ? c >> 4 : c / CPR, kc = IQ ? c & 15 : c % CPR;
         arow[j] = 0xFFFFFFF0u;
         if (row < TM) {
             const int src = STAGE == 1 ? (p.sorted_ids[blk * TM + row] & 0xFFFFFF) : blk * TM + row;
-            if (src < a_rows) arow[j] = (uint32_t)src * a_row_bytes + (uint32_t)kc * 16u;
+            if (src < a_rows) arow[j] = (uint32_t)src * a_src_bytes + (uint32_t)kc * 16u;
         }
     }
     // W and its scales: this expert's matrix; the wavefront's four n-blocks
@@ -85,7 +93,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
         const int ch = STAGE == 1 ? q * (p.n_out >> 5) + (n0 >> 5) + wave : (n0 >> 5) + wave * 2 + q;
         sboff[q] = (uint32_t)ch * chunk_bytes + (uint32_t)lane * 4u;
     }
-    __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.a_scale + (uint64_t)((blk * TM) >> 5) * chunk_bytes, (uint64_t)(TM >> 5) * chunk_bytes);
+    __amdgpu_buffer_rsrc_t rsa = make_rsrc(IQ ? p.w_scale : p.a_scale + (uint64_t)((blk * TM) >> 5) * chunk_bytes, IQ ? 0 : (uint64_t)SC * chunk_bytes);
+    const int sa_shift = MR == 1 ? ((blk * TM) >> 4 & 1) * 8 : 0;  // a 16-row block in the upper half of its 32-row scale chunk
 
     // LDS: row-major AB-byte rows, the 16-byte chunk index XORed with a row-dependent term against bank conflicts
     auto lds_off = [&](int row, int c) { return row * AB + ((c ^ ((AB == 128 ? (row >> 1) : (row >> 2)) & (CPR - 1))) << 4); };
@@ -96,9 +105,34 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
     auto load_a = [&](int kt, v4i* dst) {
         const bool ok = kt < KT;
 #pragma unroll
-        for (int j = 0; j < A_LOADS; j++) dst[j] = buf_load16(ra, ok ? arow[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
+        for (int j = 0; j < A_LOADS; j++) dst[j] = buf_load16(ra, ok ? arow[j] : 0xFFFFFFF0u, ok ? (uint32_t)kt * A_STEP : 0u);
     };
     auto store_a = [&](int stage, const v4i* src) {
+        if constexpr (IQ) {
+            // 8 bf16 -> block maximum over the four lanes of the group -> scale byte -> 8 fp4 codes = one dword of the row's step
+            float x[8];
+            float amax = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                x[2 * j] = __uint_as_float((uint32_t)src[0][j] << 16);
+                x[2 * j + 1] = __uint_as_float((uint32_t)src[0][j] & 0xFFFF0000u);
+                amax = fmaxf(amax, fmaxf(fabsf(x[2 * j]), fabsf(x[2 * j + 1])));
+            }
+            amax = fmaxf(amax, __uint_as_float(__builtin_amdgcn_update_dpp(0, __float_as_uint(amax), 0xB1, 0xF, 0xF, true)));
+            amax = fmaxf(amax, __uint_as_float(__builtin_amdgcn_update_dpp(0, __float_as_uint(amax), 0x4E, 0xF, 0xF, true)));
+            uint32_t bexp = ((__float_as_uint(amax * (1.0f / 6.0f)) + 0x7FFFFFu) >> 23) & 0xFFu;
+            bexp = bexp < 254u ? bexp : 254u;
+            const float sf = bexp ? __uint_as_float(bexp << 23) : 1.0f;
+            int word = 0;
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, x[0], x[1], sf, 0);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, x[2], x[3], sf, 1);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, x[4], x[5], sf, 2);
+            word = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, x[6], x[7], sf, 3);
+            const int row = tid >> 4, grp = (tid >> 2) & 3, q = tid & 3;
+            *reinterpret_cast<int*>(&lds[stage][lds_off(row, grp) + q * 4]) = word;
+            if (q == 0) iq_scale[stage][row * 4 + grp] = (uint8_t)bexp;
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
             const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
@@ -111,11 +145,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) dst[ni] = buf_load16(rb, ok ? boff[ni] : 0xFFFFFFF0u, ok ? (uint32_t)kt * 1024u : 0u);
     };
-    int sav[2][MR / 2], sbv[2][NR / 2];
+    int sav[2][SC], sbv[2][NR / 2];
     auto load_sc = [&](int kc, int* sa_dst, int* sb_dst) {
         const bool ok = kc < (KT >> 1);
 #pragma unroll
-        for (int q = 0; q < MR / 2; q++) sa_dst[q] = buf_load4(rsa, ok ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u);
+        for (int q = 0; q < SC; q++)
+            sa_dst[q] = IQ ? 0 : buf_load4(rsa, ok ? (uint32_t)q * chunk_bytes + (uint32_t)lane * 4u : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u) >> sa_shift;
 #pragma unroll
         for (int q = 0; q < NR / 2; q++) sb_dst[q] = buf_load4(rsb, ok ? sboff[q] : 0xFFFFFFF0u, ok ? (uint32_t)kc * 256u : 0u);
     };
@@ -151,12 +186,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
             const v8i af = read_frag(KH, mi);
+            // A-side scale: IQ keeps the byte of (row, group) of this stage in LDS; a single 16-row block has shifted its half down
+            const int sa_op = IQ ? (int)iq_scale[KH][li * 4 + lg] : sa_cur[mi / 2];
+            constexpr int sa_sel = IQ ? 0 : KH * 2 + (MR == 1 ? 0 : (mi & 1));
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
                 const v4i w4 = bw[WS][ni];
                 const v8i wf = __builtin_shufflevector(w4, w4, 0, 1, 2, 3, -1, -1, -1, -1);
-                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc[mi][ni], 4, ACODE, KH * 2 + (ni & 1), sb_cur[ni / 2],
-                                                                              KH * 2 + (mi & 1), sa_cur[mi / 2]);
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc[mi][ni], 4, ACODE, KH * 2 + (ni & 1), sb_cur[ni / 2], sa_sel, sa_op);
             });
         });
         store_a(KH ^ 1, areg[(WS + 1) % RING]);
@@ -221,7 +258,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
             *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(word & 0xFFFF);
             *reinterpret_cast<uint16_t*>(dst + 8) = (uint16_t)((uint32_t)word >> 16);
             if (lg == 0) {
-                const size_t off = ((sr >> 5) * (size_t)sc_chunk) + (size_t)(c32 >> 3) * 256u + (size_t)((c32 & 3) * 16 + li) * 4u + (size_t)(((c32 >> 2) & 1) * 2 + ((r >> 4) & 1));
+                const size_t off = ((sr >> 5) * (size_t)sc_chunk) + (size_t)(c32 >> 3) * 256u + (size_t)((c32 & 3) * 16 + li) * 4u + (size_t)(((c32 >> 2) & 1) * 2 + ((sr >> 4) & 1));
                 p.out_scale[off] = (uint8_t)bexp;
             }
         }
@@ -276,14 +313,19 @@ template <int AF, int STAGE>
 hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t stream) {
     p.eshift = block_m == 128 ? 1 : 0;
     const dim3 grid(p.n_out / (STAGE == 1 ? 128 : 256), blocks << p.eshift);
-    if (block_m == 32) hipLaunchKernelGGL((k_moe_mx<AF, 2, STAGE>), grid, dim3(256), 0, stream, p);
+    if (block_m == 16) {
+        if constexpr (STAGE == 2) hipLaunchKernelGGL((k_moe_mx<MXF_FP4, 1, 2>), grid, dim3(256), 0, stream, p);
+        else if constexpr (AF == MXF_FP4) hipLaunchKernelGGL((k_moe_mx<MXF_FP4, 1, 1, true>), grid, dim3(256), 0, stream, p);
+        else return hipErrorInvalidValue;
+    } else if (block_m == 32) hipLaunchKernelGGL((k_moe_mx<AF, 2, STAGE>), grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((k_moe_mx<AF, 4, STAGE>), grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// a_format: MXF_FP4 / MXF_FP8 (stage 1 only; stage 2 reads the fp4 rows stage 1 wrote); block_m: 32 / 64 / 128; blocks: blocks of
+// a_format: MXF_FP4 / MXF_FP8 (stage 1 only; stage 2 reads the fp4 rows stage 1 wrote); block_m: 32 / 64 / 128, or 16: stage 1 then
+// takes bf16 activations in p.a and quantises them itself (a_format MXF_FP4); blocks: blocks of
 // block_m sorted rows the launch covers (blocks past num_valid[0] exit at once)
 hipError_t psg_launch_moe_mx_gemm(const MoeMxParams& p, int a_format, int stage, int block_m, int blocks, hipStream_t stream) {
     if (stage == 1) return a_format == MXF_FP8 ? launch_rows<MXF_FP8, 1>(p, block_m, blocks, stream) : launch_rows<MXF_FP4, 1>(p, block_m, blocks, stream);

@@ -690,16 +690,19 @@ int moe_reduce_common(const void* x, void* y, const int32_t* mask, const int32_t
 
 int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     if (!a) return fail(PSG_E_NULL, "args is NULL");
-    if (!a->out || !a->a || !a->a_scale || !a->w || !a->w_scale || !a->sorted_token_ids || !a->sorted_expert_ids || !a->num_valid_ids)
+    const bool inline_quant = a->stage == 1 && a->a_dtype == PSG_MX_BF16_QUANT;
+    if (!a->out || !a->a || (!a->a_scale && !inline_quant) || !a->w || !a->w_scale || !a->sorted_token_ids || !a->sorted_expert_ids || !a->num_valid_ids)
         return fail(PSG_E_NULL, "out, a, a_scale, w, w_scale, sorted_token_ids, sorted_expert_ids and num_valid_ids must be non-NULL");
     if (a->stage != 1 && a->stage != 2) return fail(PSG_E_SHAPE, "stage=%d must be 1 or 2", a->stage);
     if (a->stage == 1 && !a->out_scale) return fail(PSG_E_NULL, "out_scale must be non-NULL in stage 1");
     if (a->stage == 2 && a->atomic && !a->sorted_weights) return fail(PSG_E_NULL, "sorted_weights must be non-NULL for the atomic epilogue");
     if (a->pad0 != 0) return fail(PSG_E_SHAPE, "pad0 must be 0");
-    if (a->stage == 1 ? (a->a_dtype != PSG_MX_FP4 && a->a_dtype != PSG_MX_FP8) : a->a_dtype != PSG_MX_FP4)
-        return fail(PSG_E_DTYPE, "a_dtype %d: stage 1 takes 0 (fp4) or 2 (fp8), stage 2 takes 0 (fp4)", a->a_dtype);
+    if (a->stage == 1 ? (a->a_dtype != PSG_MX_FP4 && a->a_dtype != PSG_MX_FP8 && a->a_dtype != PSG_MX_BF16_QUANT) : a->a_dtype != PSG_MX_FP4)
+        return fail(PSG_E_DTYPE, "a_dtype %d: stage 1 takes 0 (fp4), 2 (fp8) or 3 (bf16, quantised by the kernel), stage 2 takes 0 (fp4)", a->a_dtype);
     if (a->stage == 2 && a->out_dtype != PSG_OUT_BF16 && a->out_dtype != PSG_OUT_FP16) return fail(PSG_E_DTYPE, "out_dtype %d unknown", a->out_dtype);
-    if (a->block_m != 32 && a->block_m != 64 && a->block_m != 128) return fail(PSG_E_SHAPE, "block_m=%d must be 32, 64 or 128", a->block_m);
+    if (a->block_m != 16 && a->block_m != 32 && a->block_m != 64 && a->block_m != 128) return fail(PSG_E_SHAPE, "block_m=%d must be 16, 32, 64 or 128", a->block_m);
+    if (a->stage == 1 && (a->block_m == 16) != inline_quant)
+        return fail(PSG_E_SHAPE, "stage 1: blocks of 16 rows go with a_dtype 3 (bf16 activations quantised by the kernel) and only with it, got block_m=%d a_dtype=%d", a->block_m, a->a_dtype);
     if (a->tokens < 1 || a->tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", a->tokens);
     if (a->experts < 1) return fail(PSG_E_SHAPE, "experts=%d must be positive", a->experts);
     if (a->model_dim < 256 || a->model_dim % 256) return fail(PSG_E_SHAPE, "model_dim=%d must be a positive multiple of 256", a->model_dim);
@@ -710,12 +713,12 @@ int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
         return fail(PSG_E_SHAPE, "blocks=%d of %d rows exceed sorted_size=%d", a->blocks, a->block_m, a->sorted_size);
     const int K = a->stage == 1 ? a->model_dim : a->inter_dim;
     const int n_out = a->stage == 1 ? a->inter_dim : a->model_dim;
-    const uint64_t a_row = a->a_dtype == PSG_MX_FP8 ? (uint64_t)K : (uint64_t)K / 2;
+    const uint64_t a_row = inline_quant ? 2ull * (uint64_t)K : a->a_dtype == PSG_MX_FP8 ? (uint64_t)K : (uint64_t)K / 2;
     const uint64_t a_rows = a->stage == 1 ? (uint64_t)a->tokens : (uint64_t)a->sorted_size;
     const uint64_t rows_e = a->stage == 1 ? 2ull * (uint64_t)n_out : (uint64_t)n_out;
     if (a_rows * a_row > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "a exceeds the 4 GiB descriptor range");
     if (rows_e * (uint64_t)(K / 2) > 0xFFFFFFF0ull) return fail(PSG_E_SHAPE, "one expert's weights exceed the 4 GiB descriptor range");
-    if (!aligned(a->a, 16) || !aligned(a->w, 16) || !aligned(a->a_scale, 4) || !aligned(a->w_scale, 4) || !aligned(a->out, 16))
+    if (!aligned(a->a, 16) || !aligned(a->w, 16) || (!inline_quant && !aligned(a->a_scale, 4)) || !aligned(a->w_scale, 4) || !aligned(a->out, 16))
         return fail(PSG_E_ALIGN, "a, w and out must be 16-byte aligned, a_scale and w_scale 4-byte aligned");
     MoeMxParams p;
     p.out = a->out;

@@ -6,8 +6,9 @@ of W1 (MX-FP4), applies ``silu(gate) * up``, quantises the result to MX-FP4 agai
 position; stage 2 multiplies those sorted rows by W2 and either adds ``weight * y`` atomically into the token's output row
 (``epilog="atomic"``) or writes one unweighted row per sorted position (``epilog="nonatomic"`` / ``"nonatomic_cshuffle"``).
 
-Built: ``BM`` 32 / 64 / 128, weights in the separate gate / up row order (``interleave=False``), pre-quantised activations
-(``inline_quant=False``).  ``use_nt``, ``BN``, ``BK`` and ``xcd_swizzle`` are tuning hints of the reference's kernels: they are
+Built: ``BM`` 32 / 64 / 128 with pre-quantised activations, ``BM`` 16 with ``inline_quant=True`` (stage 1 reads the bf16
+``hidden_states`` and quantises them itself; fp4 only) and, for stage 2, ``BM`` 16 as well; weights in the separate gate / up
+row order (``interleave=False``).  ``use_nt``, ``BN``, ``BK`` and ``xcd_swizzle`` are tuning hints of the reference's kernels: they are
 checked like the reference checks them and otherwise ignored.  Everything else raises ``NotImplementedError``, as the
 reference does for the variants it does not build (host.py:142-146, :203-204).
 """
@@ -62,7 +63,8 @@ def flydsl_mxfp4_gemm1(*, a_quant, a_scale_sorted_shuffled, w1_u8, w1_scale_u8, 
         raise NotImplementedError(f"mxfp_moe gemm1 requires D_HIDDEN (K) % {BK} == 0, got H={D_HIDDEN}")
     if (2 * D_INTER) % BN != 0:
         raise NotImplementedError(f"mxfp_moe gemm1 requires 2*D_INTER (N_OUT) % {BN} == 0, got D_INTER={D_INTER}")
-    if inline_quant or interleave or BM not in (32, 64, 128) or a_dtype not in _A_DTYPE:
+    inline_quant = bool(inline_quant)
+    if interleave or a_dtype not in _A_DTYPE or (BM not in (32, 64, 128) if not inline_quant else (BM != 16 or a_dtype != "fp4")):
         raise NotImplementedError(
             f"mxfp_moe gemm1 unsupported variant (BM={BM}, use_nt={use_nt}, inline_quant={inline_quant}, interleave={interleave}, a_dtype={a_dtype})")
     if D_HIDDEN % 256 or D_INTER % 256:
@@ -70,7 +72,12 @@ def flydsl_mxfp4_gemm1(*, a_quant, a_scale_sorted_shuffled, w1_u8, w1_scale_u8, 
     sorted_size = int(m_indices.numel())
     args = _lib.MoeMxArgs()
     args.out, args.out_scale = _ptr(inter_sorted_quant), _ptr(inter_sorted_shuffled_scale)
-    args.a, args.a_scale = _ptr(a_quant), _ptr(a_scale_sorted_shuffled)
+    if inline_quant:
+        if hidden_states is None or hidden_states.dtype != torch.bfloat16 or hidden_states.numel() < int(n_tokens) * int(D_HIDDEN):
+            raise ValueError("inline_quant needs hidden_states: bf16 [n_tokens, D_HIDDEN]")
+        args.a, args.a_scale = _ptr(hidden_states), None
+    else:
+        args.a, args.a_scale = _ptr(a_quant), _ptr(a_scale_sorted_shuffled)
     args.w, args.w_scale = _ptr(w1_u8), _ptr(w1_scale_u8)
     args.sorted_token_ids, args.sorted_expert_ids = _ptr(m_indices), _ptr(sorted_expert_ids)
     args.sorted_weights, args.num_valid_ids = None, _ptr(cumsum_tensor)
@@ -78,7 +85,7 @@ def flydsl_mxfp4_gemm1(*, a_quant, a_scale_sorted_shuffled, w1_u8, w1_scale_u8, 
     args.model_dim, args.inter_dim = int(D_HIDDEN), int(D_INTER)
     args.sorted_size = sorted_size
     args.blocks = min(int(sorted_expert_ids.numel()), sorted_size // int(BM))
-    args.block_m, args.a_dtype, args.out_dtype = int(BM), _A_DTYPE[a_dtype], 0
+    args.block_m, args.a_dtype, args.out_dtype = int(BM), 3 if inline_quant else _A_DTYPE[a_dtype], 0
     args.stage, args.atomic, args.pad0 = 1, 0, 0
     if _rows(inter_sorted_quant, D_INTER // 2) < sorted_size:
         raise ValueError(f"inter_sorted_quant holds {_rows(inter_sorted_quant, D_INTER // 2)} rows, the sorted list {sorted_size}")
@@ -98,7 +105,7 @@ def flydsl_mxfp4_gemm2(*, inter_sorted_quant, inter_sorted_shuffled_scale, w2_u8
         raise NotImplementedError(f"mxfp_moe gemm2 contraction D_INTER (inter_dim) must be a multiple of {BK}, got D_INTER={D_INTER}")
     if D_HIDDEN % BN != 0:
         raise NotImplementedError(f"mxfp_moe gemm2 requires D_HIDDEN (N_OUT=model_dim) % {BN} == 0, got H={D_HIDDEN}")
-    if epilog not in _G2_EPILOGS or BM not in (32, 64, 128) or (D_INTER_REAL is not None and int(D_INTER_REAL) != int(D_INTER)):
+    if epilog not in _G2_EPILOGS or BM not in (16, 32, 64, 128) or (D_INTER_REAL is not None and int(D_INTER_REAL) != int(D_INTER)):
         raise NotImplementedError(f"mxfp_moe gemm2 unsupported variant (BM={BM}, use_nt={use_nt}, epilog={epilog}, D_INTER_REAL={D_INTER_REAL})")
     if D_HIDDEN % 256 or D_INTER % 256:
         raise NotImplementedError(f"mxfp_moe gemm2 requires D_HIDDEN and D_INTER % 256 == 0, got {D_HIDDEN}, {D_INTER}")

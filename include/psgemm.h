@@ -109,7 +109,8 @@ typedef struct psg_a8w8_args {
 } psg_a8w8_args;
 
 /* Element formats of the MX GEMM's operands (kernels/gemm/mxfp4_preshuffle.py:70-72, a_dtype / b_dtype). */
-enum psg_mx_dtype { PSG_MX_FP4 = 0, PSG_MX_FP6 = 1, PSG_MX_FP8 = 2 };
+enum psg_mx_dtype { PSG_MX_FP4 = 0, PSG_MX_FP6 = 1, PSG_MX_FP8 = 2,
+                    PSG_MX_BF16_QUANT = 3 /* psg_moe_mx_gemm stage 1 only: bf16 activations, quantised to fp4 by the kernel */ };
 
 /*
  * Arguments of the MX preshuffle GEMM: A in fp4 (e2m1), fp6 (e2m3) or fp8 (e4m3fn), W in fp4 or fp8, one e8m0 scale
@@ -300,7 +301,11 @@ int psg_moe_gemm(const psg_moe_args *args, void *stream);
  *            atomic = 1: out[t_r, n] += y * sorted_weights[r] (out [tokens, model_dim] bf16 / fp16, zeroed by the caller, order
  *            of the additions not fixed: the reference's "atomic" epilogue); atomic = 0: out[r, n] = y, out [sorted_size,
  *            model_dim] (its "nonatomic" epilogue: the caller applies the weights); w = W2 [experts * model_dim, inter_dim/2].
- *   block_m in {32, 64, 128}; model_dim % 256 == 0 and inter_dim % 256 == 0; tokens < 2^24; every operand below 4 GiB.
+ *            With a_dtype PSG_MX_BF16_QUANT (the reference's inline_quant variant, gemm1.py:324-412; block_m 16 only) a is
+ *            [tokens, model_dim] bf16 and every 32 elements are quantised to fp4 inside the kernel with the same scale rule as
+ *            the output; a_scale is not read.
+ *   block_m in {32, 64, 128}, or 16 (stage 1: only with PSG_MX_BF16_QUANT); model_dim % 256 == 0 and inter_dim % 256 == 0;
+ *   tokens < 2^24; every operand below 4 GiB.
  *   sorted_token_ids, sorted_expert_ids, sorted_weights, num_valid_ids as for psg_moe_gemm.
  */
 typedef struct psg_moe_mx_args {
@@ -319,7 +324,7 @@ typedef struct psg_moe_mx_args {
     int32_t sorted_size; /* entries of sorted_token_ids / sorted_weights = rows of the sorted intermediate */
     int32_t blocks;      /* entries of sorted_expert_ids = grid size along the sorted rows */
     int32_t block_m;
-    int32_t a_dtype;     /* stage 1: PSG_MX_FP4 or PSG_MX_FP8; stage 2: PSG_MX_FP4 */
+    int32_t a_dtype;     /* stage 1: PSG_MX_FP4, PSG_MX_FP8 or PSG_MX_BF16_QUANT; stage 2: PSG_MX_FP4 */
     int32_t out_dtype;   /* stage 2: PSG_OUT_BF16 / PSG_OUT_FP16 */
     int32_t stage;       /* 1 or 2 */
     int32_t atomic;      /* stage 2 only */

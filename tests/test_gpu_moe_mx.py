@@ -138,13 +138,62 @@ def test_blocks_of_masked_experts_are_skipped_and_longer_dims_work():
     assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * np.abs(out_ref).max()
 
 
+@pytest.mark.parametrize("tokens", [5, 70])
+def test_blocks_of_16_rows_quantise_bf16_activations_in_the_kernel(tokens):
+    """The reference's inline_quant variant (gemm1.py:324-412; tests/kernels/test_moe_gemm.py:856): stage 1 reads bf16 rows and
+    quantises them itself.  The oracle quantises the same bf16 values with the same rule and runs the pre-quantised path."""
+    model_dim, inter, experts, topk, bm = 512, 256, 6, 3, 16
+    dev = torch.device("cuda")
+    p = _problem(tokens, model_dim, inter, experts, topk, bm, "fp4", seed=40 + tokens, hot_expert=tokens > 16)
+    g = torch.Generator().manual_seed(tokens)
+    hidden = (torch.randn(tokens, model_dim, generator=g) * torch.exp(torch.randn(tokens, 1, generator=g))).to(torch.bfloat16)
+    hidden[0, 32:64] = 0
+    p["a_q"], p["a_s"] = O.mxfp4_requant_roundup(hidden.float().numpy())
+    sid, sw, se, npp = p["sort"]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    d = dict(w1=t(O.shuffle_weight_w4(p["w1_q"])), w2=t(O.shuffle_weight_w4(p["w2_q"])), w1_s=layout.e8m0_shuffle(t(p["w1_s"])),
+             w2_s=layout.e8m0_shuffle(t(p["w2_s"])), sid=t(sid), sw=t(sw), se=t(se), cumsum=t(npp[:1].astype(np.int32)))
+    rows = sid.size
+    codes = torch.full((rows, inter // 2), 0x77, dtype=torch.uint8, device=dev)
+    scales = torch.full(((rows + 255) // 256 * 256 * (inter // 32),), 0x77, dtype=torch.uint8, device=dev)
+    dummy = torch.zeros(16, dtype=torch.uint8, device=dev)
+    flydsl_mxfp4_gemm1(a_quant=dummy, a_scale_sorted_shuffled=dummy, w1_u8=d["w1"], w1_scale_u8=d["w1_s"], sorted_expert_ids=d["se"],
+                       cumsum_tensor=d["cumsum"], m_indices=d["sid"], inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales,
+                       hidden_states=hidden.to(dev), n_tokens=tokens, BM=bm, use_nt=True, inline_quant=True, NE=experts, D_HIDDEN=model_dim,
+                       D_INTER=inter, topk=topk, a_dtype="fp4")
+    torch.cuda.synchronize()
+    got_q, got_s = _check_stage1(p, codes, scales, tokens, inter, bm, "fp4")
+    nv = int(npp[0])
+    q, s = got_q.copy(), got_s.copy()
+    q[nv:], s[nv:] = 0, 0
+    flat_ref, out_ref = O.moe_mx_gemm2(q, s[:rows], p["w2_q"], p["w2_s"], sid, sw, se, nv, tokens, model_dim, bm)
+    common = dict(inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales, w2_u8=d["w2"], w2_scale_u8=d["w2_s"], sorted_expert_ids=d["se"],
+                  cumsum_tensor=d["cumsum"], sorted_token_ids=d["sid"], sorted_weights=d["sw"], M_logical=tokens, max_sorted=rows, BM=bm,
+                  NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+    flat = torch.full((rows, model_dim), 7.0, dtype=torch.bfloat16, device=dev)
+    flydsl_mxfp4_gemm2(flat_out=flat, use_nt=False, epilog="nonatomic", **common)
+    out = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+    flydsl_mxfp4_gemm2(flat_out=out, use_nt=True, epilog="atomic", **common)
+    torch.cuda.synchronize()
+    f = flat.float().cpu().numpy()
+    assert np.all(f[nv:] == 7.0)
+    live = (sid[:nv] & 0xFFFFFF) < tokens
+    tol = 1e-2 * np.abs(flat_ref[:nv][live]) + 1e-2 * np.abs(flat_ref).max()
+    assert np.all(np.abs(f[:nv][live] - flat_ref[:nv][live]) <= tol)
+    assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * np.abs(out_ref).max()
+
+
 def test_unbuilt_variants_raise_like_the_reference():
     dev = torch.device("cuda")
     z = torch.zeros(64, dtype=torch.uint8, device=dev)
     base = dict(a_quant=z, a_scale_sorted_shuffled=z, w1_u8=z, w1_scale_u8=z, sorted_expert_ids=z, cumsum_tensor=z, m_indices=z,
                 inter_sorted_quant=z, inter_sorted_shuffled_scale=z, hidden_states=z, n_tokens=4, use_nt=False, NE=2, D_HIDDEN=512, D_INTER=256, topk=1)
     with pytest.raises(NotImplementedError):
-        flydsl_mxfp4_gemm1(BM=16, inline_quant=True, **base)
+        flydsl_mxfp4_gemm1(BM=32, inline_quant=True, **base)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm1(BM=16, inline_quant=False, **base)
+    with pytest.raises(NotImplementedError):
+        flydsl_mxfp4_gemm1(BM=16, inline_quant=True, a_dtype="fp8", **base)
     with pytest.raises(NotImplementedError):
         flydsl_mxfp4_gemm1(BM=32, inline_quant=False, interleave=True, **base)
     with pytest.raises(NotImplementedError):

@@ -427,7 +427,7 @@ def test_mx_moe_validation_errors_without_a_gpu():
             setattr(a, k, v)
         return a
 
-    bad = [dict(stage=3), dict(block_m=16), dict(model_dim=384), dict(inter_dim=128), dict(a_dtype=1), dict(stage=2, a_dtype=2), dict(stage=2, out_dtype=2),
+    bad = [dict(stage=3), dict(block_m=16), dict(block_m=24), dict(block_m=32, a_dtype=3), dict(stage=2, a_dtype=3, block_m=16), dict(model_dim=384), dict(inter_dim=128), dict(a_dtype=1), dict(stage=2, a_dtype=2), dict(stage=2, out_dtype=2),
            dict(blocks=5), dict(blocks=0), dict(tokens=0), dict(experts=0), dict(pad0=1), dict(out_scale=None), dict(stage=2, atomic=1, sorted_weights=None),
            dict(a=0x10008), dict(w=None), dict(sorted_size=16)]
     for kw in bad:
