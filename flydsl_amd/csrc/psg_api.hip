@@ -708,7 +708,7 @@ int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     if (a->model_dim < 256 || a->model_dim % 256) return fail(PSG_E_SHAPE, "model_dim=%d must be a positive multiple of 256", a->model_dim);
     if (a->inter_dim < 256 || a->inter_dim % 256) return fail(PSG_E_SHAPE, "inter_dim=%d must be a positive multiple of 256", a->inter_dim);
     if (a->sorted_size < a->block_m) return fail(PSG_E_SHAPE, "sorted_size=%d is below one block of %d rows", a->sorted_size, a->block_m);
-    if (a->blocks < 1 || a->blocks > 65535) return fail(PSG_E_SHAPE, "blocks=%d outside [1, 65535]", a->blocks);
+    if (a->blocks < 1) return fail(PSG_E_SHAPE, "blocks=%d must be positive", a->blocks);
     if ((int64_t)a->blocks * a->block_m > (int64_t)a->sorted_size)
         return fail(PSG_E_SHAPE, "blocks=%d of %d rows exceed sorted_size=%d", a->blocks, a->block_m, a->sorted_size);
     const int K = a->stage == 1 ? a->model_dim : a->inter_dim;
@@ -739,7 +739,8 @@ int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     p.out_dtype = a->out_dtype;
     p.atomic = a->stage == 2 && a->atomic ? 1 : 0;
     p.eshift = 0;
-    if (((int64_t)a->blocks << 1) > 65535 && a->block_m == 128) return fail(PSG_E_SHAPE, "blocks=%d of 128 rows exceed the grid", a->blocks);
+    p.n_tiles = p.n_groups = p.by_expert = 0;
+    if (((int64_t)a->blocks << 1) * (int64_t)((n_out / 128 + 7) / 8 * 8) > 0x7FFFFFFFll) return fail(PSG_E_SHAPE, "blocks=%d times the column tiles exceed the grid", a->blocks);
     const hipError_t e = psg_launch_moe_mx_gemm(p, a->a_dtype == PSG_MX_FP8 ? MXF_FP8 : MXF_FP4, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_mx_gemm launch");
     g_err[0] = 0;

@@ -193,6 +193,8 @@ struct MoeMxParams {
     int out_dtype;              // stage 2: OUT_BF16 / OUT_FP16
     int atomic;                 // stage 2: weighted atomic add into out[token]
     int eshift;                 // set by the launcher: log2(sorter block rows / rows per workgroup)
+    int n_tiles, n_groups;      // set by the launcher: column tiles of the output, and groups of 8 of them
+    int by_expert;              // set by the launcher: workgroup ids are mapped to XCDs by (expert, column tile)
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).

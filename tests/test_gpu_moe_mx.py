@@ -138,11 +138,12 @@ def test_blocks_of_masked_experts_are_skipped_and_longer_dims_work():
     assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * np.abs(out_ref).max()
 
 
-@pytest.mark.parametrize("tokens", [5, 70])
-def test_blocks_of_16_rows_quantise_bf16_activations_in_the_kernel(tokens):
+@pytest.mark.parametrize("tokens,model_dim", [(5, 512), (70, 512), (21, 7424)])
+def test_blocks_of_16_rows_quantise_bf16_activations_in_the_kernel(tokens, model_dim):
     """The reference's inline_quant variant (gemm1.py:324-412; tests/kernels/test_moe_gemm.py:856): stage 1 reads bf16 rows and
-    quantises them itself.  The oracle quantises the same bf16 values with the same rule and runs the pre-quantised path."""
-    model_dim, inter, experts, topk, bm = 512, 256, 6, 3, 16
+    quantises them itself.  The oracle quantises the same bf16 values with the same rule and runs the pre-quantised path.
+    One case has long rows (7424 elements: 58 K steps, an odd number of 256-element scale chunks)."""
+    inter, experts, topk, bm = 256, 6, 3, 16
     dev = torch.device("cuda")
     p = _problem(tokens, model_dim, inter, experts, topk, bm, "fp4", seed=40 + tokens, hot_expert=tokens > 16)
     g = torch.Generator().manual_seed(tokens)
