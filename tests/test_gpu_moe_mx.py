@@ -68,8 +68,9 @@ def _check_stage1(p, codes, scales, tokens, inter, bm, a_fmt):
     live = (sid[:nv] & 0xFFFFFF) < tokens
     assert not got_q[:nv][~live].any() and not got_s[:nv][~live].any(), "padding rows hold zero codes and zero scales"
     ds = got_s[:nv][live].astype(np.int32) - want_s[:nv][live].astype(np.int32)
-    assert np.abs(ds).max() <= 1 and np.mean(ds != 0) <= 5e-3, (np.abs(ds).max(), np.mean(ds != 0))
-    assert np.mean(got_q[:nv][live] == want_q[:nv][live]) >= 0.99
+    if ds.size:  # small problems: one block on a boundary, a handful of elements on a rounding tie
+        assert np.abs(ds).max() <= 1 and np.count_nonzero(ds) <= max(5e-3 * ds.size, 1), (np.abs(ds).max(), np.mean(ds != 0))
+        assert np.count_nonzero(got_q[:nv][live] != want_q[:nv][live]) <= max(0.01 * got_q[:nv][live].size, 4)
     unit = np.repeat(np.ldexp(1.0, got_s[:nv].astype(np.int32) - 127), 32, axis=1) * (got_s[:nv] != 0).repeat(32, axis=1)
     deq = O.mxfp4_to_f32(got_q[:nv]) * unit
     assert np.all(np.abs(deq - y[:nv]) <= unit * 1.0 + 1e-3 * np.abs(y[:nv]) + 1e-30)
@@ -182,6 +183,56 @@ def test_blocks_of_16_rows_quantise_bf16_activations_in_the_kernel(tokens, model
     tol = 1e-2 * np.abs(flat_ref[:nv][live]) + 1e-2 * np.abs(flat_ref).max()
     assert np.all(np.abs(f[:nv][live] - flat_ref[:nv][live]) <= tol)
     assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * np.abs(out_ref).max()
+
+
+def test_random_problems_over_every_block_size_and_activation_format():
+    """Sixteen seeded problems: token counts from 1 up, experts without tokens, top-k up to the expert count, widths from the
+    smallest (256) to several column tiles with tile counts that are and are not multiples of 8, every block size with each of its
+    activation formats, both stage-2 epilogues."""
+    dev = torch.device("cuda")
+    rng = np.random.default_rng(2024)
+    variants = [(32, "fp4"), (64, "fp4"), (128, "fp4"), (32, "fp8"), (64, "fp8"), (128, "fp8"), (16, "bf16")]
+    for case in range(16):
+        bm, a_fmt = variants[case % len(variants)]
+        tokens = int(rng.choice([1, 2, 7, 16, 33, 100, 257]))
+        experts = int(rng.choice([1, 3, 8, 24]))
+        topk = int(rng.integers(1, min(experts, 6) + 1))
+        model_dim = 256 * int(rng.choice([1, 2, 3, 5]))
+        inter = 256 * int(rng.choice([1, 2, 3, 5]))
+        print(f"case {case}: bm={bm} a={a_fmt} tokens={tokens} experts={experts} topk={topk} model_dim={model_dim} inter={inter}", flush=True)
+        p = _problem(tokens, model_dim, inter, experts, topk, bm, "fp8" if a_fmt == "fp8" else "fp4", seed=1000 + case)
+        sid, sw, se, npp = p["sort"]
+        rows, nv = sid.size, int(npp[0])
+        if a_fmt == "bf16":
+            g = torch.Generator().manual_seed(case)
+            hidden = torch.randn(tokens, model_dim, generator=g).to(torch.bfloat16)
+            p["a_q"], p["a_s"] = O.mxfp4_requant_roundup(hidden.float().numpy())
+        d = _device_inputs(p, tokens, max(bm, 32), dev)
+        codes = torch.full((rows, inter // 2), 0x77, dtype=torch.uint8, device=dev)
+        scales = torch.full(((rows + 255) // 256 * 256 * (inter // 32),), 0x77, dtype=torch.uint8, device=dev)
+        extra = dict(inline_quant=True, hidden_states=hidden.to(dev), a_dtype="fp4") if a_fmt == "bf16" else dict(a_dtype=a_fmt)
+        flydsl_mxfp4_gemm1(a_quant=d["a"], a_scale_sorted_shuffled=d["a_s"], w1_u8=d["w1"], w1_scale_u8=d["w1_s"], sorted_expert_ids=d["se"],
+                           cumsum_tensor=d["cumsum"], m_indices=d["sid"], inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales,
+                           n_tokens=tokens, BM=bm, NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk, **extra)
+        torch.cuda.synchronize()
+        got_q, got_s = _check_stage1(p, codes, scales, tokens, inter, bm, "fp8" if a_fmt == "fp8" else "fp4")
+        q, s2 = got_q.copy(), got_s.copy()
+        q[nv:], s2[nv:] = 0, 0
+        flat_ref, out_ref = O.moe_mx_gemm2(q, s2[:rows], p["w2_q"], p["w2_s"], sid, sw, se, nv, tokens, model_dim, bm)
+        common = dict(inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales, w2_u8=d["w2"], w2_scale_u8=d["w2_s"], sorted_expert_ids=d["se"],
+                      cumsum_tensor=d["cumsum"], sorted_token_ids=d["sid"], sorted_weights=d["sw"], M_logical=tokens, max_sorted=rows, BM=bm,
+                      NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+        flat = torch.full((rows, model_dim), 7.0, dtype=torch.bfloat16, device=dev)
+        flydsl_mxfp4_gemm2(flat_out=flat, epilog="nonatomic", **common)
+        out = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+        flydsl_mxfp4_gemm2(flat_out=out, epilog="atomic", **common)
+        torch.cuda.synchronize()
+        f = flat.float().cpu().numpy()
+        assert np.all(f[nv:] == 7.0)
+        live = (sid[:nv] & 0xFFFFFF) < tokens
+        scale = max(float(np.abs(flat_ref).max()), 1e-30)
+        assert np.all(np.abs(f[:nv][live] - flat_ref[:nv][live]) <= 1e-2 * np.abs(flat_ref[:nv][live]) + 1e-2 * scale), case
+        assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * max(float(np.abs(out_ref).max()), 1e-30), case
 
 
 def test_unbuilt_variants_raise_like_the_reference():
