@@ -34,6 +34,7 @@ EXPORTS = (
     "psg_debug_tile_order",
     "psg_moe_gemm",
     "psg_moe_mx_gemm",
+    "psg_moe_mx_scale_sort",
     "psg_moe_reduce",
     "psg_moe_reduce_masked",
     "psg_moe_sorting",
@@ -233,6 +234,8 @@ def lib() -> ctypes.CDLL:
     handle.psg_moe_reduce_masked.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int32] * 5 + [ctypes.c_void_p]
     handle.psg_moe_sorting_workspace_bytes.restype = ctypes.c_uint64
     handle.psg_moe_sorting_workspace_bytes.argtypes = [ctypes.c_int32] * 3
+    handle.psg_moe_mx_scale_sort.restype = ctypes.c_int
+    handle.psg_moe_mx_scale_sort.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int32] * 4 + [ctypes.c_void_p]
     handle.psg_moe_reduce.restype = ctypes.c_int
     handle.psg_moe_reduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int32] * 4 + [ctypes.c_void_p]
     handle.psg_moe_softmax_sorting.restype = ctypes.c_int

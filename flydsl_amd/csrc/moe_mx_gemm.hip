@@ -360,10 +360,43 @@ hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t strea
 
 }  // namespace
 
+// Scales of the sorted rows in the shuffled order stage 1 reads: one thread per output dword = the scale bytes of the rows r16 and
+// r16 + 16 of a 32-row chunk at the columns c4 and c4 + 4 of an 8-column chunk (byte = 2 * column half + row half).
+__global__ void __launch_bounds__(256) k_moe_mx_scale_sort(const uint8_t* scale, const int32_t* sorted_ids, const int32_t* num_valid, uint32_t* out,
+                                                            int tokens, int topk, int cols, int sorted_size, int dwords) {
+    const int d = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    if (d >= dwords) return;
+    const int r16 = d & 15, c4 = (d >> 4) & 3, blk = d >> 6;  // blk = chunk * (cols / 8) + column chunk
+    const int ncc = cols >> 3, chunk = blk / ncc, cc = blk % ncc;
+    const int nv = num_valid[0];
+    uint32_t word = 0;
+#pragma unroll
+    for (int rh = 0; rh < 2; rh++) {
+        const int i = chunk * 32 + rh * 16 + r16;
+        if (i >= sorted_size || i >= nv) continue;
+        const uint32_t id = (uint32_t)sorted_ids[i];
+        const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
+        if (tok >= tokens || (topk > 1 && slot >= topk)) continue;
+        const uint8_t* row = scale + (size_t)(topk > 1 ? tok * topk + slot : tok) * (size_t)cols + cc * 8 + c4;
+        word |= (uint32_t)row[0] << (8 * rh);
+        word |= (uint32_t)row[4] << (8 * (2 + rh));
+    }
+    out[d] = word;
+}
+
 // a_format: MXF_FP4 / MXF_FP8 (stage 1 only; stage 2 reads the fp4 rows stage 1 wrote); block_m: 32 / 64 / 128, or 16: stage 1 then
 // takes bf16 activations in p.a and quantises them itself (a_format MXF_FP4); blocks: blocks of
 // block_m sorted rows the launch covers (blocks past num_valid[0] exit at once)
 hipError_t psg_launch_moe_mx_gemm(const MoeMxParams& p, int a_format, int stage, int block_m, int blocks, hipStream_t stream) {
     if (stage == 1) return a_format == MXF_FP8 ? launch_rows<MXF_FP8, 1>(p, block_m, blocks, stream) : launch_rows<MXF_FP4, 1>(p, block_m, blocks, stream);
     return launch_rows<MXF_FP4, 2>(p, block_m, blocks, stream);
+}
+
+// out: ceil(sorted_size / 32) * 32 rows x cols bytes, every byte written
+hipError_t psg_launch_moe_mx_scale_sort(const void* scale, const int32_t* sorted_ids, const int32_t* num_valid, void* out, int tokens, int topk, int cols,
+                                        int sorted_size, hipStream_t stream) {
+    const int dwords = (sorted_size + 31) / 32 * 8 * cols;
+    hipLaunchKernelGGL(k_moe_mx_scale_sort, dim3((dwords + 255) / 256), dim3(256), 0, stream, static_cast<const uint8_t*>(scale), sorted_ids, num_valid,
+                       static_cast<uint32_t*>(out), tokens, topk, cols, sorted_size, dwords);
+    return hipGetLastError();
 }

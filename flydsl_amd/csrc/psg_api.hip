@@ -15,6 +15,8 @@ hipError_t psg_launch_a8w8_tiled(const A8W8Params& p, int kind, int store, int t
 hipError_t psg_launch_a8w8_stream(const A8W8Params& p, int kind, int store, hipStream_t stream);
 hipError_t psg_launch_moe_gemm(const MoeParams& p, int kind, int stage, int block_m, int blocks, hipStream_t stream);
 hipError_t psg_launch_moe_mx_gemm(const MoeMxParams& p, int a_format, int stage, int block_m, int blocks, hipStream_t stream);
+hipError_t psg_launch_moe_mx_scale_sort(const void* scale, const int32_t* sorted_ids, const int32_t* num_valid, void* out, int tokens, int topk, int cols,
+                                        int sorted_size, hipStream_t stream);
 hipError_t psg_launch_moe_sort(const MoeSortParams& p, void* workspace, uint64_t workspace_bytes, hipStream_t stream);
 uint64_t psg_moe_sort_workspace(int64_t pairs, int experts);
 int psg_moe_sort_max_experts();
@@ -687,6 +689,21 @@ int moe_reduce_common(const void* x, void* y, const int32_t* mask, const int32_t
     return 0;
 }
 }  // namespace
+
+int psg_moe_mx_scale_sort(const void* scale, const int32_t* sorted_token_ids, const int32_t* num_valid_ids, void* out, int32_t tokens, int32_t topk,
+                          int32_t cols, int32_t sorted_size, void* stream) {
+    if (!scale || !sorted_token_ids || !num_valid_ids || !out) return fail(PSG_E_NULL, "scale, sorted_token_ids, num_valid_ids and out must be non-NULL");
+    if (tokens < 1 || tokens >= (1 << 24)) return fail(PSG_E_SHAPE, "tokens=%d outside [1, 2^24)", tokens);
+    if (topk < 1 || topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", topk);
+    if (cols < 8 || cols % 8) return fail(PSG_E_SHAPE, "cols=%d must be a positive multiple of 8", cols);
+    if (sorted_size < 1) return fail(PSG_E_SHAPE, "sorted_size=%d must be positive", sorted_size);
+    if (((int64_t)sorted_size + 31) / 32 * 8 * (int64_t)cols > 0x7FFFFFFFll) return fail(PSG_E_SHAPE, "sorted_size * cols exceeds 2^33 bytes");
+    if (!aligned(out, 4)) return fail(PSG_E_ALIGN, "out must be 4-byte aligned");
+    const hipError_t e = psg_launch_moe_mx_scale_sort(scale, sorted_token_ids, num_valid_ids, out, tokens, topk, cols, sorted_size, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "psg_moe_mx_scale_sort launch");
+    g_err[0] = 0;
+    return 0;
+}
 
 int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     if (!a) return fail(PSG_E_NULL, "args is NULL");

@@ -134,3 +134,26 @@ def flydsl_mxfp4_gemm2(*, inter_sorted_quant, inter_sorted_shuffled_scale, w2_u8
     lib = _lib.lib()
     _lib.check(lib.psg_moe_mx_gemm(ctypes.byref(args), _stream_handle(stream)), "psg_moe_mx_gemm (stage 2)")
     return flat_out
+
+
+def moe_mxfp4_sort(blockscale_e8m0, sorted_ids, num_valid_ids, token_num, block_size=32, out=None, stream=None):
+    """The ``a_scale_sorted_shuffled`` input of stage 1 from the scales of the quantised activations, on the device in one launch
+    (the reference's ``moe_mxfp4_sort``, tests/kernels/utils/gemm_common_utils.py:545-598, same arguments): ``blockscale_e8m0``
+    ``[tokens, C]`` or ``[tokens, topk, C]`` bytes, ``C % 8 == 0``; returns ``[ceil(len(sorted_ids)/32)*32, C]`` uint8 (``out`` when
+    given, which keeps the call allocation-free).  Rows of padding ids and rows past ``num_valid_ids[0]`` are zero."""
+    if block_size % 32:
+        raise AssertionError(f"block_size={block_size} must be a multiple of 32")
+    s = blockscale_e8m0.view(torch.uint8)
+    topk = 1 if s.dim() == 2 else int(s.shape[1])
+    cols = int(s.shape[-1])
+    if not s.is_contiguous():
+        raise ValueError("blockscale_e8m0 must be contiguous")
+    rows = (int(sorted_ids.numel()) + 31) // 32 * 32
+    if out is None:
+        out = torch.empty(rows, cols, dtype=torch.uint8, device=s.device)
+    elif out.numel() * out.element_size() < rows * cols:
+        raise ValueError(f"out holds {out.numel() * out.element_size()} bytes, {rows * cols} are written")
+    lib = _lib.lib()
+    _lib.check(lib.psg_moe_mx_scale_sort(_ptr(s), _ptr(sorted_ids), _ptr(num_valid_ids), _ptr(out), int(token_num), topk, cols, int(sorted_ids.numel()),
+                                         _stream_handle(stream)), "psg_moe_mx_scale_sort")
+    return out

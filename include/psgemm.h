@@ -333,6 +333,14 @@ typedef struct psg_moe_mx_args {
 
 int psg_moe_mx_gemm(const psg_moe_mx_args *args, void *stream);
 
+/* a_scale of psg_moe_mx_gemm stage 1 from the scales of the quantised activations: the reference's moe_mxfp4_sort
+ * (tests/kernels/utils/gemm_common_utils.py:464-598).  scale [tokens, cols] e8m0 bytes (topk = 1) or [tokens, topk, cols] (then the
+ * row of a sorted id is token * topk + slot); out: ceil(sorted_size/32)*32 rows x cols bytes in the shuffled order, row i = the scale
+ * row of sorted_token_ids[i]; rows of padding ids and rows from num_valid_ids[0] on are zero (every byte of out is written; the
+ * reference leaves the rows past num_valid_ids[0] untouched).  cols % 8 == 0. */
+int psg_moe_mx_scale_sort(const void *scale, const int32_t *sorted_token_ids, const int32_t *num_valid_ids, void *out, int32_t tokens,
+                          int32_t topk, int32_t cols, int32_t sorted_size, void *stream);
+
 /* y[t, :] = sum over the topk slots of x[t, slot, :] (fp32 sum in slot order), the pass after stage 2 with accumulate = 0
  * (kernels/moe/moe_gemm_2stage/moe_reduce.py:164-203 with use_mask = False).  dtype: PSG_OUT_BF16 / PSG_OUT_FP16 / PSG_OUT_F32,
  * the type of both x and y (the reference's dense variants, :57-61); model_dim % 4 == 0. */

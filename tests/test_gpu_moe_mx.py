@@ -235,6 +235,88 @@ def test_random_problems_over_every_block_size_and_activation_format():
         assert np.abs(out.float().cpu().numpy() - out_ref).max() <= 3e-2 * max(float(np.abs(out_ref).max()), 1e-30), case
 
 
+def test_device_scale_sort_matches_the_oracle_byte_for_byte():
+    from kernels.moe.mxfp_moe import moe_mxfp4_sort
+
+    dev = torch.device("cuda")
+    rng = np.random.default_rng(77)
+    for tokens, topk, cols, n_ids, nv in ((11, 3, 16, 58, 48), (1, 1, 8, 32, 32), (300, 8, 128, 4000, 3968), (40, 2, 24, 100, 100)):
+        ids = rng.integers(0, tokens + 3, size=n_ids).astype(np.int64)  # some ids at or past `tokens`: padding
+        ids = (ids | (rng.integers(0, topk, size=n_ids) << 24)).astype(np.int32)
+        for sc in (rng.integers(1, 255, size=(tokens, cols), dtype=np.uint8), rng.integers(1, 255, size=(tokens, topk, cols), dtype=np.uint8)):
+            want = O.moe_mxfp4_sort(sc, ids, nv, tokens)
+            out = torch.full((want.shape[0] + 32, cols), 0x5A, dtype=torch.uint8, device=dev)
+            got = moe_mxfp4_sort(torch.from_numpy(sc).to(dev), torch.from_numpy(ids).to(dev), torch.tensor([nv, tokens], dtype=torch.int32, device=dev),
+                                 tokens, out=out)
+            torch.cuda.synchronize()
+            g = got.cpu().numpy()
+            assert np.array_equal(g.reshape(-1)[: want.size], want.reshape(-1))
+            assert np.all(g.reshape(-1)[want.size :] == 0x5A), "nothing past ceil(rows/32)*32 rows is written"
+
+
+def test_layer_from_bf16_activations_runs_on_the_device_and_replays_in_a_graph():
+    """bf16 hidden state -> device MX-FP4 quantiser -> device scale sort -> stage 1 -> stage 2 (atomic), caller-owned buffers only;
+    eager once, then captured into a HIP graph and replayed three times with eager work in between.  The oracle quantises the same
+    hidden state with the host rule the device quantiser is byte-equal to."""
+    from flydsl_amd import quant_device
+    from kernels.moe.mxfp_moe import moe_mxfp4_sort
+
+    tokens, model_dim, inter, experts, topk, bm = 45, 768, 512, 7, 3, 32
+    dev = torch.device("cuda")
+    p = _problem(tokens, model_dim, inter, experts, topk, bm, "fp4", seed=91)
+    hidden = torch.randn(tokens, model_dim, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    p["a_q"], a_s = O.per_1x32_f4_quant(hidden.float().numpy())
+    p["a_s"] = a_s[:tokens]
+    sid, sw, se, npp = p["sort"]
+    rows, nv = sid.size, int(npp[0])
+    d = _device_inputs(p, tokens, bm, dev)
+    hid = hidden.to(dev)
+    a_q = torch.empty(tokens, model_dim // 2, dtype=torch.uint8, device=dev)
+    a_s_rm = torch.empty((tokens + 31) // 32 * 32, model_dim // 32, dtype=torch.uint8, device=dev)
+    a_s_sorted = torch.empty((rows + 31) // 32 * 32, model_dim // 32, dtype=torch.uint8, device=dev)
+    codes = torch.full((rows, inter // 2), 0x77, dtype=torch.uint8, device=dev)
+    scales = torch.full(((rows + 255) // 256 * 256 * (inter // 32),), 0x77, dtype=torch.uint8, device=dev)
+    out = torch.zeros(tokens, model_dim, dtype=torch.bfloat16, device=dev)
+
+    def layer():
+        out.zero_()
+        quant_device.per_1x32_f4_quant(hid, shuffle=False, out=(a_q, a_s_rm))
+        moe_mxfp4_sort(a_s_rm[:tokens], d["sid"], d["cumsum"], tokens, block_size=bm, out=a_s_sorted)
+        flydsl_mxfp4_gemm1(a_quant=a_q, a_scale_sorted_shuffled=a_s_sorted, w1_u8=d["w1"], w1_scale_u8=d["w1_s"], sorted_expert_ids=d["se"],
+                           cumsum_tensor=d["cumsum"], m_indices=d["sid"], inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales,
+                           n_tokens=tokens, BM=bm, NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+        flydsl_mxfp4_gemm2(inter_sorted_quant=codes, inter_sorted_shuffled_scale=scales, w2_u8=d["w2"], w2_scale_u8=d["w2_s"], sorted_expert_ids=d["se"],
+                           cumsum_tensor=d["cumsum"], sorted_token_ids=d["sid"], sorted_weights=d["sw"], flat_out=out, M_logical=tokens,
+                           max_sorted=rows, BM=bm, epilog="atomic", NE=experts, D_HIDDEN=model_dim, D_INTER=inter, topk=topk)
+
+    layer()
+    torch.cuda.synchronize()
+    assert np.array_equal(a_q.cpu().numpy(), p["a_q"]) and np.array_equal(a_s_sorted.cpu().numpy(), d["a_s"].cpu().numpy())
+    got_q, got_s = _check_stage1(p, codes, scales, tokens, inter, bm, "fp4")
+    q, s2 = got_q.copy(), got_s.copy()
+    q[nv:], s2[nv:] = 0, 0
+    _, out_ref = O.moe_mx_gemm2(q, s2[:rows], p["w2_q"], p["w2_s"], sid, sw, se, nv, tokens, model_dim, bm)
+    tol = 3e-2 * float(np.abs(out_ref).max())
+    assert np.abs(out.float().cpu().numpy() - out_ref).max() <= tol
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        layer()
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            layer()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        out.fill_(5.0)
+        codes.fill_(0x33)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(codes.cpu().numpy()[:nv], got_q[:nv])
+        assert np.abs(out.float().cpu().numpy() - out_ref).max() <= tol
+
+
 def test_unbuilt_variants_raise_like_the_reference():
     dev = torch.device("cuda")
     z = torch.zeros(64, dtype=torch.uint8, device=dev)

@@ -436,6 +436,16 @@ def test_mx_moe_validation_errors_without_a_gpu():
         assert handle.psg_last_error()
 
 
+def test_mx_scale_sort_validation_errors_without_a_gpu():
+    handle = _lib.lib()
+    ok = dict(scale=0x1000, ids=0x1000, nv=0x1000, out=0x1000, tokens=4, topk=1, cols=16, rows=64)
+    for kw in (dict(scale=None), dict(ids=None), dict(nv=None), dict(out=None), dict(tokens=0), dict(topk=0), dict(topk=256), dict(cols=12), dict(cols=0),
+               dict(rows=0), dict(out=0x1002)):
+        a = {**ok, **kw}
+        assert handle.psg_moe_mx_scale_sort(a["scale"], a["ids"], a["nv"], a["out"], a["tokens"], a["topk"], a["cols"], a["rows"], None) < 0, kw
+        assert handle.psg_last_error()
+
+
 def test_gating_validation_errors_without_a_gpu():
     handle = _lib.lib()
     assert handle.psg_moe_topk_gating(None, None) == -1
