@@ -72,24 +72,27 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
 
     // LDS: row-major AB-byte rows, the 16-byte chunk index XORed with a row-dependent term against bank conflicts
     auto lds_off = [&](int row, int c) { return row * AB + ((c ^ ((AB == 128 ? (row >> 1) : (row >> 2)) & (CPR - 1))) << 4); };
-    v4i areg[A_LOADS];
-    auto load_a = [&](int kt) {
+    // Operands are requested PF steps ahead of their MFMAs in rings of RING register sets (small tiles: a K step is a few hundred
+    // MFMA cycles per wavefront, far below the latency of a load; the 128 x 256 tile needs its registers for accumulators)
+    constexpr int RING = MR * NR <= 8 ? 4 : 2, PF = RING - 1;
+    v4i areg[RING][A_LOADS];
+    auto load_a = [&](int kt, v4i* dst) {
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
             const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
             const bool ok = row < TM && kt < kt_end;
-            areg[j] = buf_load16(ra, ok ? (uint32_t)row * a_rs + (uint32_t)kc * 16u : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
+            dst[j] = buf_load16(ra, ok ? (uint32_t)row * a_rs + (uint32_t)kc * 16u : 0xFFFFFFF0u, ok ? (uint32_t)kt * AB : 0u);
         }
     };
-    auto store_a = [&](int stage) {
+    auto store_a = [&](int stage, const v4i* src) {
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++) {
             const int c = tid + 256 * j, row = c / CPR, kc = c % CPR;
-            if (row < TM) *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, kc)]) = areg[j];
+            if (row < TM) *reinterpret_cast<v4i*>(&lds[stage][lds_off(row, kc)]) = src[j];
         }
     };
     // W operand of n-block ni for step kt -> 8 dwords (fp4 uses the low four)
-    v8i bw[2][NR];
+    v8i bw[RING][NR];
     auto load_b = [&](int kt, v8i* dst) {
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) {
@@ -137,13 +140,14 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    // One K step of parity KH (= 128-K half of the current scale chunk): MFMAs on LDS stage KH and W set KH
-    // and the scale set SET (scale chunks alternate between the two sets)
-    auto step = [&](int kt, auto KHP, auto SETP) __attribute__((always_inline)) {
-        constexpr int KH = decltype(KHP)::value, SET = decltype(SETP)::value;
-        load_a(kt + 1);
-        load_b(kt + 1, bw[KH ^ 1]);
-        if constexpr (KH == 1) load_sc((kt >> 1) + 1, sav[SET ^ 1], sbv[SET ^ 1]);
+    // One K step of parity KH (= 128-K half of the current scale chunk): MFMAs on LDS stage KH, W set WS = step % RING and the
+    // scale set SET (scale chunks alternate between the two sets); requests the operands of step kt + PF and, in the first half of
+    // a chunk, the scales of the next one; stages the A rows of step kt + 1
+    auto step = [&](int kt, auto KHP, auto SETP, auto WSP) __attribute__((always_inline)) {
+        constexpr int KH = decltype(KHP)::value, SET = decltype(SETP)::value, WS = decltype(WSP)::value;
+        load_a(kt + PF, areg[(WS + PF) % RING]);
+        load_b(kt + PF, bw[(WS + PF) % RING]);
+        if constexpr (KH == 0) load_sc((kt >> 1) + 1, sav[SET ^ 1], sbv[SET ^ 1]);
         const int* sa_cur = sav[SET];
         const int* sb_cur = sbv[SET];
         static_for<MR>([&](auto MI) {
@@ -151,27 +155,32 @@ __global__ void __launch_bounds__(256) k_mx_generic(MxGenParams p) {
             const v8i af = read_frag(KH, mi);
             static_for<NR>([&](auto NI) {
                 constexpr int ni = decltype(NI)::value;
-                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bw[KH][ni], af, acc[mi][ni], MxCode<BF>::value, MxCode<AF>::value,
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bw[WS][ni], af, acc[mi][ni], MxCode<BF>::value, MxCode<AF>::value,
                                                                               KH * 2 + (ni & 1), sb_cur[ni / 2], KH * 2 + (mi & 1), sa_cur[mi / 2]);
             });
         });
-        store_a(KH ^ 1);
+        store_a(KH ^ 1, areg[(WS + 1) % RING]);
         __syncthreads();
     };
 
-    load_a(kt_begin);
-    load_b(kt_begin, bw[0]);
-    load_sc(kt_begin >> 1, sav[0], sbv[0]);
-    store_a(0);
-    __syncthreads();
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2 % RING>;
+    using I3 = std::integral_constant<int, 3 % RING>;
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        load_a(kt_begin + i, areg[i]);
+        load_b(kt_begin + i, bw[i]);
+    }
+    load_sc(kt_begin >> 1, sav[0], sbv[0]);
+    store_a(0, areg[0]);
+    __syncthreads();
     for (int kt = kt_begin; kt < kt_end; kt += 4) {  // two scale chunks per trip, so every register index is a constant
-        step(kt, I0{}, I0{});
-        step(kt + 1, I1{}, I0{});
+        step(kt, I0{}, I0{}, I0{});
+        step(kt + 1, I1{}, I0{}, I1{});
         if (kt + 2 < kt_end) {
-            step(kt + 2, I0{}, I1{});
-            step(kt + 3, I1{}, I1{});
+            step(kt + 2, I0{}, I1{}, I2{});
+            step(kt + 3, I1{}, I1{}, I3{});
         }
     }
 
