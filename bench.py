@@ -367,6 +367,35 @@ def run_next_row_workloads():
                     "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s1 / 1e9})
         out.append({"workload": f"moe_mxfp4_stage2_atomic_{tag}", "us_per_launch_events": s2 * 1e6, "tflops": 2.0 * tokens * topk * model_dim * inter_dim / s2 / 1e12,
                     "weight_gb_per_s": experts * model_dim * inter_dim / 2 / s2 / 1e9})
+        # the launches in front of stage 1 when the activations arrive as bf16: the MX-FP4 quantiser and the scale sort
+        from flydsl_amd import quant_device
+        from kernels.moe.mxfp_moe import moe_mxfp4_sort
+
+        hid = torch.randn(tokens, model_dim, generator=g).to(torch.bfloat16).to(dev)
+        xq_buf = torch.empty(tokens, model_dim // 2, dtype=torch.uint8, device=dev)
+        xs_buf = torch.empty((tokens + 31) // 32 * 32, model_dim // 32, dtype=torch.uint8, device=dev)
+        xs_sorted = torch.empty((rows + 31) // 32 * 32, model_dim // 32, dtype=torch.uint8, device=dev)
+
+        def front():
+            quant_device.per_1x32_f4_quant(hid, shuffle=False, out=(xq_buf, xs_buf))
+            moe_mxfp4_sort(xs_buf[:tokens], sid, nv, tokens, block_size=bm, out=xs_sorted)
+
+        sf = timed(front, iters=50)
+        out.append({"workload": f"moe_mxfp4_quant_and_scale_sort_tokens{tokens}_model{model_dim}_block{bm}", "us_per_launch_events": sf * 1e6, "tflops": 0.0,
+                    "weight_gb_per_s": 0.0})
+        if tokens <= 64:
+            # the same stage 1 on blocks of 16 rows reading the bf16 rows itself (no launches in front of it)
+            sid16, swt16, se16, npp16 = moe_sorting(ids.int().to(dev), torch.softmax(vals, 1).to(dev), num_experts=experts, block_size=16)
+            rows16 = int(sid16.numel())
+            iq16 = torch.zeros(rows16, inter_dim // 2, dtype=torch.uint8, device=dev)
+            iqs16 = torch.zeros((rows16 + 255) // 256 * 256 * (inter_dim // 32), dtype=torch.uint8, device=dev)
+            nv16 = npp16[:1].contiguous()
+            s16 = timed(lambda: flydsl_mxfp4_gemm1(a_quant=a4, a_scale_sorted_shuffled=a4s, w1_u8=w1m, w1_scale_u8=w1s, m_indices=sid16, inter_sorted_quant=iq16,
+                                                   inter_sorted_shuffled_scale=iqs16, n_tokens=tokens, inline_quant=True, hidden_states=hid,
+                                                   sorted_expert_ids=se16, cumsum_tensor=nv16, BM=16, NE=experts, D_HIDDEN=model_dim, D_INTER=inter_dim, topk=topk))
+            out.append({"workload": f"moe_mxfp4_stage1_inline_quant_tokens{tokens}_e{experts}_top{topk}_model{model_dim}_inter{inter_dim}_block16",
+                        "us_per_launch_events": s16 * 1e6, "tflops": 2.0 * tokens * topk * 2 * inter_dim * model_dim / s16 / 1e12,
+                        "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s16 / 1e9})
     # the device-side expert sorter in front of the stages (outputs pre-allocated, accumulate buffer cleared by the same launch)
     for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)):
         g = torch.Generator().manual_seed(0)
