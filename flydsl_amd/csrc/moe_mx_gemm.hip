@@ -134,16 +134,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
     constexpr uint32_t A_STEP = IQ ? 256u : (uint32_t)AB;                // ... and of one K step of it
     __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)a_rows * a_src_bytes);
     uint32_t arow[A_LOADS];
-#pragma unroll
-    for (int j = 0; j < A_LOADS; j++) {
-        // IQ: thread t takes 8 bf16 (16 bytes) of row t / 16: four neighbouring lanes hold one 32-element group
-        const int c = tid + 256 * j, row = IQ ? c >> 4 : c / CPR, kc = IQ ? c & 15 : c % CPR;
-        arow[j] = 0xFFFFFFF0u;
-        if (row < TM) {
-            const int src = STAGE == 1 ? (p.sorted_ids[blk * TM + row] & 0xFFFFFF) : blk * TM + row;
-            if (src < a_rows) arow[j] = (uint32_t)src * a_src_bytes + (uint32_t)kc * 16u;
-        }
-    }
     // W and its scales: this expert's matrix; the wavefront's four n-blocks
     __amdgpu_buffer_rsrc_t rb = make_rsrc(p.w + (uint64_t)e * (uint64_t)w_rows * b_row_bytes, (uint64_t)w_rows * b_row_bytes);
     __amdgpu_buffer_rsrc_t rsb = make_rsrc(p.w_scale + (uint64_t)e * (uint64_t)(w_rows >> 5) * chunk_bytes, (uint64_t)(w_rows >> 5) * chunk_bytes);
@@ -253,11 +243,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2 % RING>;
     using I3 = std::integral_constant<int, 3 % RING>;
+    // the first W fragments are requested before the list of sorted rows is fetched: they only depend on the expert
 #pragma unroll
-    for (int i = 0; i < PF; i++) {
-        load_a(i, areg[i]);
-        load_b(i, bw[i]);
+    for (int i = 0; i < PF; i++) load_b(i, bw[i]);
+#pragma unroll
+    for (int j = 0; j < A_LOADS; j++) {
+        // IQ: thread t takes 8 bf16 (16 bytes) of row t / 16: four neighbouring lanes hold one 32-element group
+        const int c = tid + 256 * j, row = IQ ? c >> 4 : c / CPR, kc = IQ ? c & 15 : c % CPR;
+        arow[j] = 0xFFFFFFF0u;
+        if (row < TM) {
+            const int src = STAGE == 1 ? (p.sorted_ids[blk * TM + row] & 0xFFFFFF) : blk * TM + row;
+            if (src < a_rows) arow[j] = (uint32_t)src * a_src_bytes + (uint32_t)kc * 16u;
+        }
     }
+#pragma unroll
+    for (int i = 0; i < PF; i++) load_a(i, areg[i]);
     load_sc(0, sav[0], sbv[0]);
     store_a(0, areg[0]);
     __syncthreads();
