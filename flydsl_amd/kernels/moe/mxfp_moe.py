@@ -49,6 +49,16 @@ def _stream_handle(stream):
     return ctypes.c_void_p(stream.cuda_stream)
 
 
+def _need(t, name, dtype=None, itemsize=None):
+    """A pointer is all the library gets: refuse tensors whose element type, device or layout it would misread."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or not t.is_contiguous():
+        raise TypeError(f"{name} must be a contiguous device tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if itemsize is not None and t.element_size() != itemsize:
+        raise TypeError(f"{name} must have {itemsize}-byte elements, got {t.dtype}")
+
+
 def _rows(t, row_bytes):
     return t.numel() * t.element_size() // row_bytes
 
@@ -69,12 +79,26 @@ def flydsl_mxfp4_gemm1(*, a_quant, a_scale_sorted_shuffled, w1_u8, w1_scale_u8, 
             f"mxfp_moe gemm1 unsupported variant (BM={BM}, use_nt={use_nt}, inline_quant={inline_quant}, interleave={interleave}, a_dtype={a_dtype})")
     if D_HIDDEN % 256 or D_INTER % 256:
         raise NotImplementedError(f"mxfp_moe gemm1 requires D_HIDDEN and D_INTER % 256 == 0, got {D_HIDDEN}, {D_INTER}")
+    for t, name in ((m_indices, "m_indices"), (sorted_expert_ids, "sorted_expert_ids"), (cumsum_tensor, "cumsum_tensor")):
+        _need(t, name, dtype=torch.int32)
+    for t, name in ((w1_u8, "w1_u8"), (w1_scale_u8, "w1_scale_u8"), (inter_sorted_quant, "inter_sorted_quant"),
+                    (inter_sorted_shuffled_scale, "inter_sorted_shuffled_scale")):
+        _need(t, name, itemsize=1)
+    if not inline_quant:
+        _need(a_quant, "a_quant", itemsize=1)
+        _need(a_scale_sorted_shuffled, "a_scale_sorted_shuffled", itemsize=1)
+        a_row = int(D_HIDDEN) // 2 if a_dtype == "fp4" else int(D_HIDDEN)
+        if _rows(a_quant, a_row) < int(n_tokens):
+            raise ValueError(f"a_quant holds {_rows(a_quant, a_row)} rows of {a_row} bytes, n_tokens={n_tokens}")
+    if w1_u8.numel() < int(NE) * 2 * int(D_INTER) * (int(D_HIDDEN) // 2) or w1_scale_u8.numel() < int(NE) * 2 * int(D_INTER) * (int(D_HIDDEN) // 32):
+        raise ValueError("w1_u8 / w1_scale_u8 are smaller than NE * 2*D_INTER rows of D_HIDDEN/2 code bytes and D_HIDDEN/32 scale bytes")
     sorted_size = int(m_indices.numel())
     args = _lib.MoeMxArgs()
     args.out, args.out_scale = _ptr(inter_sorted_quant), _ptr(inter_sorted_shuffled_scale)
     if inline_quant:
-        if hidden_states is None or hidden_states.dtype != torch.bfloat16 or hidden_states.numel() < int(n_tokens) * int(D_HIDDEN):
+        if hidden_states is None or hidden_states.numel() < int(n_tokens) * int(D_HIDDEN):
             raise ValueError("inline_quant needs hidden_states: bf16 [n_tokens, D_HIDDEN]")
+        _need(hidden_states, "hidden_states", dtype=torch.bfloat16)
         args.a, args.a_scale = _ptr(hidden_states), None
     else:
         args.a, args.a_scale = _ptr(a_quant), _ptr(a_scale_sorted_shuffled)
@@ -111,13 +135,24 @@ def flydsl_mxfp4_gemm2(*, inter_sorted_quant, inter_sorted_shuffled_scale, w2_u8
         raise NotImplementedError(f"mxfp_moe gemm2 requires D_HIDDEN and D_INTER % 256 == 0, got {D_HIDDEN}, {D_INTER}")
     if flat_out.dtype not in (torch.bfloat16, torch.float16):
         raise TypeError(f"flat_out must be bf16 or fp16, got {flat_out.dtype}")
+    for t, name in ((sorted_token_ids, "sorted_token_ids"), (sorted_expert_ids, "sorted_expert_ids"), (cumsum_tensor, "cumsum_tensor")):
+        _need(t, name, dtype=torch.int32)
+    _need(sorted_weights, "sorted_weights", dtype=torch.float32)
+    for t, name in ((w2_u8, "w2_u8"), (w2_scale_u8, "w2_scale_u8"), (inter_sorted_quant, "inter_sorted_quant"),
+                    (inter_sorted_shuffled_scale, "inter_sorted_shuffled_scale")):
+        _need(t, name, itemsize=1)
+    _need(flat_out, "flat_out")
+    if w2_u8.numel() < int(NE) * int(D_HIDDEN) * (int(D_INTER) // 2) or w2_scale_u8.numel() < int(NE) * int(D_HIDDEN) * (int(D_INTER) // 32):
+        raise ValueError("w2_u8 / w2_scale_u8 are smaller than NE * D_HIDDEN rows of D_INTER/2 code bytes and D_INTER/32 scale bytes")
     atomic = epilog == "atomic"
     max_sorted = int(max_sorted)
     need = (int(M_logical) if atomic else max_sorted) * int(D_HIDDEN)
     if flat_out.numel() < need:
         raise ValueError(f"flat_out holds {flat_out.numel()} elements, epilog {epilog!r} writes {need}")
-    if sorted_token_ids.numel() < max_sorted or _rows(inter_sorted_quant, D_INTER // 2) < max_sorted:
-        raise ValueError("sorted_token_ids / inter_sorted_quant are shorter than max_sorted rows")
+    if sorted_token_ids.numel() < max_sorted or sorted_weights.numel() < max_sorted or _rows(inter_sorted_quant, D_INTER // 2) < max_sorted:
+        raise ValueError("sorted_token_ids / sorted_weights / inter_sorted_quant are shorter than max_sorted rows")
+    if inter_sorted_shuffled_scale.numel() < (max_sorted + 31) // 32 * 32 * (int(D_INTER) // 32):
+        raise ValueError("inter_sorted_shuffled_scale is smaller than ceil(max_sorted / 32) * 32 * D_INTER/32 bytes")
     args = _lib.MoeMxArgs()
     args.out, args.out_scale = _ptr(flat_out), None
     args.a, args.a_scale = _ptr(inter_sorted_quant), _ptr(inter_sorted_shuffled_scale)
@@ -143,7 +178,12 @@ def moe_mxfp4_sort(blockscale_e8m0, sorted_ids, num_valid_ids, token_num, block_
     given, which keeps the call allocation-free).  Rows of padding ids and rows past ``num_valid_ids[0]`` are zero."""
     if block_size % 32:
         raise AssertionError(f"block_size={block_size} must be a multiple of 32")
+    _need(blockscale_e8m0, "blockscale_e8m0", itemsize=1)
+    _need(sorted_ids, "sorted_ids", dtype=torch.int32)
+    _need(num_valid_ids, "num_valid_ids", dtype=torch.int32)
     s = blockscale_e8m0.view(torch.uint8)
+    if s.dim() not in (2, 3) or s.shape[0] < int(token_num) or s.shape[-1] % 8:
+        raise ValueError(f"blockscale_e8m0 must be [tokens, C] or [tokens, topk, C] with C % 8 == 0 and at least token_num rows, got {tuple(s.shape)}")
     topk = 1 if s.dim() == 2 else int(s.shape[1])
     cols = int(s.shape[-1])
     if not s.is_contiguous():

@@ -338,3 +338,14 @@ def test_unbuilt_variants_raise_like_the_reference():
         flydsl_mxfp4_gemm2(epilog="nonatomic_mxfp4", **g2)
     with pytest.raises(NotImplementedError):
         flydsl_mxfp4_gemm2(epilog="atomic", **{**g2, "D_INTER": 320})
+    # a pointer is all the library sees: wrong element types are refused before anything is launched
+    i32 = torch.zeros(64, dtype=torch.int32, device=dev)
+    ok1 = {**base, "sorted_expert_ids": i32, "cumsum_tensor": i32, "m_indices": i32}
+    with pytest.raises(TypeError):
+        flydsl_mxfp4_gemm1(BM=32, **{**ok1, "m_indices": i32.long()})
+    with pytest.raises(TypeError):
+        flydsl_mxfp4_gemm1(BM=32, **{**ok1, "cumsum_tensor": i32.cpu()})
+    with pytest.raises(ValueError):
+        flydsl_mxfp4_gemm1(BM=32, **ok1)  # 64 bytes of weights
+    with pytest.raises(TypeError):
+        flydsl_mxfp4_gemm2(epilog="atomic", **{**g2, "sorted_expert_ids": i32, "cumsum_tensor": i32, "sorted_token_ids": i32, "sorted_weights": i32})
