@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the preshuffle quantized GEMM on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu] [--next-rows] [--reference-shapes]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu] [--next-rows [--next-rows-only SECTION]] [--reference-shapes]
 
 A step is one GEMM launch on one set of synthetic operands (seed 0; activations N(0,1), weights
 N(0,0.02), quantised and preshuffled on the host, resident in HBM before the timed region).
@@ -252,7 +252,7 @@ def run_quant_workload(name, steps=50, warmup=5):
                          "traffic": None, "algorithmic_bytes": nbytes}}
 
 
-def run_next_row_workloads():
+def run_next_row_workloads(only=None):
     """Timings of the kernels of the rows next to the hot path (``--next-rows``): the general MX kernel on the reference's
     test shapes and the two MoE stages.  HIP events around plain launch loops (every kernel here runs for >= 15 us, so
     launch gaps hide behind the previous kernel); weights sized beyond the Infinity Cache where the shape allows."""
@@ -284,7 +284,8 @@ def run_next_row_workloads():
         return best
 
     out = []
-    for af, bf in (("fp8", "fp8"), ("fp6", "fp4"), ("fp8", "fp4")):
+    want = lambda section: only is None or only == section  # noqa: E731  (--next-rows-only: one section, e.g. under a profiler)
+    for af, bf in (("fp8", "fp8"), ("fp6", "fp4"), ("fp8", "fp4")) if want("mx") else ():
         for M in (1024, 64, 32):
             N = K = 8192
             d = make_mx(min(M, 256), 512, K, af, bf, seed=0)
@@ -297,7 +298,7 @@ def run_next_row_workloads():
             wbytes = N * K // (2 if bf == "fp4" else 1)
             out.append({"workload": f"mx_{af}x{bf}_m{M}_n8192_k8192", "us_per_launch_events": sec * 1e6, "tflops": 2.0 * M * N * K / sec / 1e12,
                         "weight_gb_per_s": wbytes / sec / 1e9})
-    for tokens, model_dim, inter_dim, experts, topk, tile_m in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 16), (333, 4096, 2048, 17, 9, 64)):
+    for tokens, model_dim, inter_dim, experts, topk, tile_m in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 16), (333, 4096, 2048, 17, 9, 64)) if want("moe_fp8") else ():
         g = torch.Generator().manual_seed(0)
         vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
         sid, swt, se, npp = moe_sorting(ids.int().to(dev), torch.softmax(vals, 1).to(dev), num_experts=experts, block_size=tile_m)  # device sorter
@@ -343,7 +344,7 @@ def run_next_row_workloads():
     # it by sorted position, stage 2 adds weight * row into the token's output row); blocks of at least 32 sorted rows
     from kernels.moe.mxfp_moe import flydsl_mxfp4_gemm1, flydsl_mxfp4_gemm2
 
-    for tokens, model_dim, inter_dim, experts, topk, bm in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 32)):
+    for tokens, model_dim, inter_dim, experts, topk, bm in ((4096, 4096, 1536, 32, 8, 128), (64, 4096, 1536, 32, 8, 32)) if want("moe_mxfp4") else ():
         g = torch.Generator().manual_seed(0)
         vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
         sid, swt, se, npp = moe_sorting(ids.int().to(dev), torch.softmax(vals, 1).to(dev), num_experts=experts, block_size=bm)
@@ -397,7 +398,7 @@ def run_next_row_workloads():
                         "us_per_launch_events": s16 * 1e6, "tflops": 2.0 * tokens * topk * 2 * inter_dim * model_dim / s16 / 1e12,
                         "weight_gb_per_s": experts * 2 * inter_dim * model_dim / 2 / s16 / 1e9})
     # the device-side expert sorter in front of the stages (outputs pre-allocated, accumulate buffer cleared by the same launch)
-    for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)):
+    for tokens, model_dim, experts, topk, tile_m in ((64, 4096, 32, 8, 16), (4096, 4096, 32, 8, 128), (4096, 4096, 256, 8, 32), (16384, 4096, 256, 8, 32)) if want("moe_sorting") else ():
         g = torch.Generator().manual_seed(0)
         vals, ids = torch.topk(torch.rand(tokens, experts, generator=g), k=topk, dim=1)
         d_ids, d_w = ids.int().to(dev), torch.softmax(vals, 1).to(dev)
@@ -438,7 +439,7 @@ def run_next_row_workloads():
             best = min(best, e0.elapsed_time(e1) / 1e3 / steps / 10)
         return best
 
-    for tokens, experts, topk in ((16, 256, 8), (16, 128, 6), (1024, 128, 6), (16384, 256, 8)):
+    for tokens, experts, topk in ((16, 256, 8), (16, 128, 6), (1024, 128, 6), (16384, 256, 8)) if want("moe_gating") else ():
         g = torch.Generator().manual_seed(0)
         x = (torch.rand(tokens, experts, generator=g) * 4 - 2).to(torch.bfloat16).to(dev)
         w = torch.empty(tokens, topk, dtype=torch.float32, device=dev)
@@ -603,6 +604,8 @@ def main():
                     help="also time the shapes of the reference's own tests for this path; adds a reference_test_shapes list")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the general MX kernel and the MoE stages (rows next to the hot path); adds a next_rows list")
+    ap.add_argument("--next-rows-only", default=None, choices=("mx", "moe_fp8", "moe_mxfp4", "moe_sorting", "moe_gating"),
+                    help="with --next-rows: run one section of them only (for profiler runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy a few times (the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against)")
@@ -655,7 +658,7 @@ def main():
             others.append(r)
         for name in ("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"):
             others.append(run_quant_workload(name))
-    next_rows = run_next_row_workloads() if args.next_rows else None
+    next_rows = run_next_row_workloads(args.next_rows_only) if args.next_rows else None
     ref_shapes = run_reference_test_shapes() if args.reference_shapes else None
 
     line = {
