@@ -109,6 +109,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
         const int wg_slot = (int)blockIdx.x >> 3;
         blk = wg_slot / p.n_groups;
         n_tile = wg_slot % p.n_groups * 8;
+    } else if (p.quad_tiles) {
+        // XCD x = id % 8 takes the row blocks of parity x / 4 and the column tiles t with t % 4 == x % 4: the tiles of a block meet in
+        // four L2s instead of eight, a slice of the weights alternates between two
+        const int x = (int)blockIdx.x & 7, s = (int)blockIdx.x >> 3, nq = p.n_tiles >> 2;
+        blk = 2 * (s / nq) + (x >> 2);
+        n_tile = (x & 3) + 4 * (s % nq);
     } else {
         blk = (int)blockIdx.x / p.n_tiles;  // block of TM sorted rows; the sorter's blocks hold TM << eshift rows
         n_tile = (int)blockIdx.x % p.n_tiles;
@@ -350,7 +356,9 @@ hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t strea
     // blocks of 32, stage 1 66 -> 49 us); with many blocks per expert the plain order measured better (4096 tokens: 297 us against 330)
     const int rows_wg = block_m >> p.eshift;
     p.by_expert = p.n_tiles % 8 != 0 && (long)p.sorted_size <= 6L * p.experts * rows_wg;
-    const dim3 grid((unsigned)(p.by_expert ? p.n_groups * 8 : p.n_tiles) * (unsigned)(blocks << p.eshift));
+    p.quad_tiles = !p.by_expert && p.n_tiles % 4 == 0 && p.n_tiles % 8 != 0;
+    const unsigned row_blocks = (unsigned)(blocks << p.eshift);
+    const dim3 grid((unsigned)(p.by_expert ? p.n_groups * 8 : p.n_tiles) * (p.quad_tiles ? (row_blocks + 1) / 2 * 2 : row_blocks));
     if (block_m == 16) {
         if constexpr (STAGE == 2) hipLaunchKernelGGL((k_moe_mx<MXF_FP4, 1, 2>), grid, dim3(256), 0, stream, p);
         else if constexpr (AF == MXF_FP4) hipLaunchKernelGGL((k_moe_mx<MXF_FP4, 1, 1, true>), grid, dim3(256), 0, stream, p);

@@ -756,7 +756,7 @@ int psg_moe_mx_gemm(const psg_moe_mx_args* a, void* stream) {
     p.out_dtype = a->out_dtype;
     p.atomic = a->stage == 2 && a->atomic ? 1 : 0;
     p.eshift = 0;
-    p.n_tiles = p.n_groups = p.by_expert = 0;
+    p.n_tiles = p.n_groups = p.by_expert = p.quad_tiles = 0;
     if (((int64_t)a->blocks << 1) * (int64_t)((n_out / 128 + 7) / 8 * 8) > 0x7FFFFFFFll) return fail(PSG_E_SHAPE, "blocks=%d times the column tiles exceed the grid", a->blocks);
     const hipError_t e = psg_launch_moe_mx_gemm(p, a->a_dtype == PSG_MX_FP8 ? MXF_FP8 : MXF_FP4, a->stage, a->block_m, a->blocks, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "psg_moe_mx_gemm launch");

@@ -195,6 +195,7 @@ struct MoeMxParams {
     int eshift;                 // set by the launcher: log2(sorter block rows / rows per workgroup)
     int n_tiles, n_groups;      // set by the launcher: column tiles of the output, and groups of 8 of them
     int by_expert;              // set by the launcher: workgroup ids are mapped to XCDs by (expert, column tile)
+    int quad_tiles;             // set by the launcher: workgroup ids are mapped to XCDs by (row block parity, column tile % 4)
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).
