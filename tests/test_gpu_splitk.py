@@ -174,3 +174,22 @@ def test_workspace_growth_during_capture_is_refused():
         with torch.cuda.graph(g, stream=s):
             fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, torch.cuda.current_stream())
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 2048, 4096), (128, 4096, 4096), (300, 1040, 2048), (512, 4096, 1024), (200, 4112, 5120), (384, 5120, 5120),
+                                   (512, 5120, 5120), (96, 4096, 14336), (33, 28672, 4096)])
+def test_mid_m_plans_stay_bit_exact_for_int8(M, N, K):
+    """The automatic plan between the streaming kernel and GPU-filling problems: 64x64 tiles on short rows (with and without two K
+    splits), 128x128 tiles with up to eight splits on long rows, and the shapes on either side of each rule's border.  int8 sums are
+    exact, so whatever the plan the bf16 output equals the C oracle bit for bit; guard rows behind M stay untouched."""
+    d = make_a8w8(M, N, K, "int8", seed=M + N)
+    dev = torch.device("cuda")
+    fn = _fn("int8", N, K)
+    ref = C.a8w8(np_bytes(d["a_q"]), np_bytes(d["b_shuf"]), d["sa"].numpy(), d["sb"].numpy(), "int8")["c_bf16_bits"]
+    t = {k: d[k].to(dev) for k in ("a_q", "b_shuf", "sa", "sb")}
+    bias = torch.empty(0, dtype=torch.bfloat16, device=dev)
+    c = torch.full((M + 3, N), 7.0, dtype=torch.bfloat16, device=dev)
+    fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(c[:M]), ref)
+    assert torch.all(c[M:] == 7.0)
