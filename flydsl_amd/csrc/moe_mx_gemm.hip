@@ -352,10 +352,10 @@ hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t strea
     p.eshift = block_m == 128 ? 1 : 0;
     p.n_tiles = p.n_out / (STAGE == 1 ? 128 : 256);
     p.n_groups = (p.n_tiles + 7) / 8;
-    // Keyed by expert while an expert has few row blocks (then sharing an L2 is what saves re-reads: 256 tokens x top-8 on 32 experts,
-    // blocks of 32, stage 1 66 -> 49 us); with many blocks per expert the plain order measured better (4096 tokens: 297 us against 330)
-    const int rows_wg = block_m >> p.eshift;
-    p.by_expert = p.n_tiles % 8 != 0 && (long)p.sorted_size <= 6L * p.experts * rows_wg;
+    // Keyed by expert while an expert has few rows (then sharing an L2 is what saves re-reads: 256 tokens x top-8 on 32 experts,
+    // blocks of 32, stage 1 66 -> 49 us; blocks of 16: 84 -> 71); from about 200 sorted rows per expert on the other orders measured
+    // better (1024 tokens, blocks of 64: 93 us against 103; 4096 tokens: 297 against 330)
+    p.by_expert = p.n_tiles % 8 != 0 && (long)p.sorted_size <= 192L * p.experts;
     p.quad_tiles = !p.by_expert && p.n_tiles % 4 == 0 && p.n_tiles % 8 != 0;
     const unsigned row_blocks = (unsigned)(blocks << p.eshift);
     const dim3 grid((unsigned)(p.by_expert ? p.n_groups * 8 : p.n_tiles) * (p.quad_tiles ? (row_blocks + 1) / 2 * 2 : row_blocks));
