@@ -1,0 +1,430 @@
+// 256x256 tile of the compute-bound mainloop, eight wavefronts side by side along N (gfx950).
+//
+// Same operand paths as gemm_tiled.h (W fragments straight from memory into MFMA operand registers, every fragment read
+// from memory once per workgroup; the A tile shared through LDS and read by all eight wavefronts), with a different way
+// of moving A and of synchronising:
+//   * A goes global -> LDS by DMA (buffer_load_dwordx4 ... lds): no staging registers, no ds_write.  A DMA instruction
+//     writes 64 x 16 bytes to consecutive LDS addresses (M0 + 16*lane), i.e. eight 128-byte rows of the stage, so the XOR
+//     swizzle of the 16-byte chunks is applied to the SOURCE address of each lane (lane l of a 1 KB block fills physical
+//     chunk l%8 of row l/8 and therefore fetches logical chunk (l%8) ^ ((row/2)%8) of that row).  Lanes redirected past
+//     the descriptor bound (rows >= M, K tail, steps past the end) write zeros.
+//   * Four LDS stages of 32 KB: the A tile of step kt+3 is requested during step kt, is waited for (vmcnt, by the
+//     wavefront that requested it) before the barrier that ends step kt+1, and is therefore complete for everybody one
+//     whole step before its MFMAs.  That lets every wavefront read the first A fragments of step kt+1 BEFORE the barrier
+//     that ends step kt, so the MFMAs continue right behind the barrier instead of waiting for LDS.  The one barrier per
+//     step that is left only keeps a stage from being overwritten while a slower wavefront still reads it.
+//   * The DMA is issued from inline assembly: the compiler does not know that it writes LDS (it would otherwise put a
+//     full vmcnt wait in front of every LDS read that follows), so the kernel does that bookkeeping itself.  Loads
+//     return in order, and the compiler counts only the W loads it knows about, so within a step the DMAs are issued
+//     before the W loads and only behind the first MFMAs (where the compiler waits for this step's W fragments): a
+//     compiler-made vmcnt then never covers a DMA that was issued a moment ago.
+#pragma once
+#include "gemm_tiled.h"
+
+namespace {
+
+constexpr int T8_STAGE = 256 * TK;  // bytes of one A stage (256 rows x 128 bytes)
+constexpr int T8_NS = 4;            // LDS stages
+
+// descriptor built from values forced into scalar registers (an inline-asm "s" operand must not end up in vector registers)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_uniform(const void* base, uint64_t bytes) {
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint32_t n = (uint32_t)__builtin_amdgcn_readfirstlane((int)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>((uintptr_t)(((uint64_t)hi << 32) | lo)), 0, (int)n, 0x00020000);
+}
+
+// one DMA instruction: 64 lanes x 16 bytes from (descriptor, voff + soff) to LDS [lds_addr, lds_addr + 1024)
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voff), "s"(r), "s"(__builtin_amdgcn_readfirstlane((int)soff))
+                 : "memory");
+}
+
+#ifndef T8_DBG
+#define T8_DBG 0
+#endif
+#ifdef T8_TIMING
+__device__ unsigned long long* t8_dbg;  // per workgroup: 8 x (core clock, 10 ns wall clock) at start / loop begin / loop end / kernel end
+#define T8_STAMP(i) do { if (threadIdx.x == 0) { t8_dbg[blockIdx.x * 16 + 2 * (i)] = clock64(); t8_dbg[blockIdx.x * 16 + 2 * (i) + 1] = wall_clock64(); } } while (0)
+#else
+#define T8_STAMP(i) do { } while (0)
+#endif
+
+// 4 bytes per lane: 64 lanes x 4 bytes to LDS [lds_addr, lds_addr + 256)
+__device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voff), "s"(r), "s"(__builtin_amdgcn_readfirstlane((int)soff))
+                 : "memory");
+}
+
+// PFW = K steps the W fragments are fetched ahead of their MFMAs (1 or 3; PFW + 1 register sets)
+template <int KIND, int STORE, int PFW>
+__global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
+    using acc_t = typename Acc<KIND>::type;
+    constexpr int MR = 16, NR = 2, WAVES = 8;
+    constexpr int TM = 256, TN = 256;
+    constexpr int NB = PFW + 1;
+    static_assert(NB == 2 || NB == 4, "W register sets");
+    constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
+    constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;
+    constexpr bool MX = KIND == KIND_MXFP4 || KIND == KIND_MXFP8;
+
+    // LDS: four A stages; behind them four slots of MX scale dwords (per slot 8 A-side chunks + 8 W-side chunks of 256 bytes)
+    // or the per-token / per-channel scales of the epilogue (256 + 256 floats)
+    constexpr int SC_SLOT = 4096;
+    constexpr int LDS_EXTRA = MX ? T8_NS * SC_SLOT : 2048;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[T8_NS * T8_STAGE + LDS_EXTRA];
+    uint8_t* const lds_x = lds + T8_NS * T8_STAGE;
+
+    T8_STAMP(0);
+    const int tid = threadIdx.x;
+    const int wave = wave_id();
+    const int lane = tid & 63;
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+
+    const int tiles_m = (p.M + TM - 1) / TM;
+    const int tiles_n = (p.N + TN - 1) / TN;
+    int tm, tn;
+    tile_coords((int)blockIdx.x, tiles_m, tiles_n, p.group_m, tm, tn);
+    const int m0 = tm * TM;
+    const int n0 = tn * TN;
+    const int K = KIND == KIND_MXFP4 ? (p.K >> 1) : (IS16 ? (p.K << 1) : p.K);  // BYTES of one operand row
+    const int KT = (K + TK - 1) / TK;
+    const int kt_per = (KT + p.splits - 1) / p.splits;
+    const int kt_begin = (int)blockIdx.y * kt_per;
+    const int kt_end = (kt_begin + kt_per) < KT ? (kt_begin + kt_per) : KT;
+
+    const uint64_t a_rows = (uint64_t)(p.M - m0);
+    __amdgpu_buffer_rsrc_t ra = make_rsrc_uniform(p.a + (uint64_t)m0 * K, a_rows * (uint64_t)K);
+    const int nb0 = (n0 >> 4) + wave * NR;
+    const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)K;
+    const uint64_t b_total = (uint64_t)p.N * (uint64_t)K;
+    __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
+
+    // MX scales: per (32-row chunk, 256-element K chunk) 64 dwords, one per lane.  Wavefront w brings A-side chunk w of the
+    // tile and its own W-side chunk (32 columns) into the slot of the step by two 4-byte DMAs; chunks past the end read
+    // as zero (scale byte 0 = 2^-127, multiplied by operands that are zero too).
+    constexpr int MP = MR / 2, NP = 1;
+    __amdgpu_buffer_rsrc_t rsa = ra, rsb = ra;
+    if constexpr (MX) {
+        const uint32_t chunk_bytes = KIND == KIND_MXFP4 ? (uint32_t)KT * 256u : (uint32_t)(p.K >> 8) * 256u;
+        const uint64_t sa_chunks = (uint64_t)((p.M + 31) >> 5), sa_mine = (uint64_t)((m0 >> 5) + wave);
+        rsa = make_rsrc_uniform(p.mx_sa + (sa_mine < sa_chunks ? sa_mine : sa_chunks) * chunk_bytes, sa_mine < sa_chunks ? chunk_bytes : 0);
+        const uint64_t sb_chunks = (uint64_t)(p.N >> 5), sb_mine = (uint64_t)((n0 >> 5) + wave);
+        rsb = make_rsrc_uniform(p.mx_sb + (sb_mine < sb_chunks ? sb_mine : sb_chunks) * chunk_bytes, sb_mine < sb_chunks ? chunk_bytes : 0);
+    }
+    int sav[2][MP], sbv[2][NP];
+
+    acc_t acc[MR][NR];
+#pragma unroll
+    for (int mi = 0; mi < MR; mi++)
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) acc[mi][ni] = (acc_t){0, 0, 0, 0};
+
+    v4i blo[NB][NR], bhi[NB][NR];
+
+    // A by DMA: this wavefront fills the four 1 KB blocks 4*wave + j (rows 8*(4*wave + j) .. + 7) of a stage
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    uint32_t a_voff[4];
+    int a_kc[2];  // logical 16-byte chunk this lane fetches, by the parity of the block
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int row = (wave * 4 + j) * 8 + (lane >> 3);
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        a_voff[j] = (uint32_t)row * (uint32_t)K + (uint32_t)kc * 16u;
+        a_kc[j & 1] = kc;
+    }
+    // CHK = false: the step is known to lie inside [kt_begin, kt_end) and not to be the K tail, so nothing is redirected (the
+    // selects and compares of the checked form are ten instructions per load in front of the MFMAs of both wavefronts of a SIMD)
+    auto dma_a1 = [&](int kt, int stage, int j, auto CHK) {
+        const uint32_t dst = lds_base + (uint32_t)(stage * T8_STAGE + (wave * 4 + j) * 1024);
+        if constexpr (decltype(CHK)::value) {
+            const bool in_k = kt < kt_end && (uint32_t)(kt * TK + a_kc[j & 1] * 16) < (uint32_t)K;
+            dma16(ra, dst, in_k ? a_voff[j] : 0xFFFFFFF0u, (kt < kt_end && !(T8_DBG & 64)) ? (uint32_t)kt * TK : 0u);
+        } else {
+            dma16(ra, dst, a_voff[j], (T8_DBG & 64) ? 0u : (uint32_t)kt * TK);
+        }
+    };
+
+    // scale dwords of step kt -> slot (two DMAs per wavefront), and slot -> registers
+    auto dma_sc = [&](int kt, int slot, int which) {
+        const bool has = kt < kt_end;
+        const uint32_t dst = lds_base + (uint32_t)(T8_NS * T8_STAGE + slot * SC_SLOT + which * 2048 + wave * 256);
+        dma4(which ? rsb : rsa, dst, has ? (uint32_t)lane * 4u : 0xFFFFFFF0u, has ? (uint32_t)(KIND == KIND_MXFP8 ? (kt >> 1) : kt) * 256u : 0u);
+    };
+    auto read_sc = [&](int slot, int q, int* sa_dst, int* sb_dst) {
+        if (q < MP) sa_dst[q] = *reinterpret_cast<const int*>(lds_x + slot * SC_SLOT + q * 256 + lane * 4);
+        else sb_dst[0] = *reinterpret_cast<const int*>(lds_x + slot * SC_SLOT + 2048 + wave * 256 + lane * 4);
+    };
+    const uint32_t b_lane_off = p.b_rowmajor ? (uint32_t)li * (uint32_t)K + (uint32_t)lg * 16u : (uint32_t)lane * 16u;
+    const uint32_t b_step = p.b_rowmajor ? 128u : 2048u, b_half = p.b_rowmajor ? 64u : 1024u;
+    auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi, auto CHK) {
+        const int ni = idx >> 1;
+        const bool has = !decltype(CHK)::value || (kt < kt_end && (kt * TK + (idx & 1) * 64) < K);
+        const uint32_t voff = b_lane_off + (uint32_t)ni * 16u * (uint32_t)K;
+        v4i v;
+        if constexpr ((T8_DBG & 128) != 0) {  // timing experiment: the same registers filled from LDS instead of memory
+            v = *reinterpret_cast<const v4i*>(&lds[((kt & 3) * 8 + idx) * 1024 + lane * 16]);
+        } else {
+            v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, (has && !(T8_DBG & 64)) ? (uint32_t)kt * b_step + (uint32_t)(idx & 1) * b_half : 0u);
+        }
+        if (idx & 1) hi[ni] = v; else lo[ni] = v;
+    };
+    // fragment (16 rows x 2 x 16 bytes of K) of m-block mi from a stage: row mi*16 + li, chunks lg and 4 + lg; the swizzle
+    // term (row/2)%8 = (li/2)%8 does not depend on mi
+    const int f_lo = li * TK + ((lg ^ ((li >> 1) & 7)) << 4);
+    const int f_hi = li * TK + (((4 + lg) ^ ((li >> 1) & 7)) << 4);
+    auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {
+        flo = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_lo]);
+        fhi = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_hi]);
+    };
+
+    constexpr int FRAG_AHEAD = (T8_DBG & 16) ? 3 : 2, FRAG_BUFS = 4;  // 16 m-blocks per step: buffer mi % 4 lines up across steps
+    v4i flo[FRAG_BUFS], fhi[FRAG_BUFS];
+
+    // One K step: MFMAs on LDS stage S and W set SB.  m-block 0 only multiplies (the compiler waits for this step's W
+    // fragments there); m-blocks 1..4 each issue one DMA of the A tile of step kt+3, m-blocks 5.. the W loads (and MX scale
+    // dwords) of step kt+PFW; every m-block reads the A fragment two m-blocks ahead, the last two those of step kt+1.
+    auto step = [&](int kt, auto SP, auto CHK) {
+        constexpr int S = decltype(SP)::value;   // LDS stage of this step (kt % 4)
+        constexpr int SB = S % NB;               // W register set of this step
+        constexpr int SN = (SB + PFW) % NB;      // W register set the loads of this step fill
+        constexpr int SS = S & 1;                // MX scale set of this step
+        constexpr int N_DMA = 4 + (MX ? 2 : 0);  // DMAs per wavefront per step: four 1 KB blocks of A (+ two chunks of MX scales)
+        constexpr int N_W = 2 * NR;              // W fragment loads per wavefront per step
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            if constexpr ((T8_DBG & 2) != 0) {
+            } else if constexpr (mi + FRAG_AHEAD < MR)
+                read_frag(S, mi + FRAG_AHEAD, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
+            else
+                read_frag((S + 1) % T8_NS, mi + FRAG_AHEAD - MR, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
+            // memory instructions, one m-block each from m-block 1 on: the DMAs of step kt+3, then the W loads of step kt+PFW
+            if constexpr (mi >= 1 && mi <= 4) {
+                if constexpr ((T8_DBG & 4) == 0) dma_a1(kt + 3, (S + 3) % T8_NS, mi - 1, CHK);
+            } else if constexpr (MX && mi == 5) {
+                dma_sc(kt + 3, (S + 3) % T8_NS, 0);
+                dma_sc(kt + 3, (S + 3) % T8_NS, 1);
+            } else if constexpr (mi >= (MX ? 6 : 5) && mi < (MX ? 6 : 5) + N_W) {
+                if constexpr ((T8_DBG & 8) == 0) load_b1(kt + PFW, mi - (MX ? 6 : 5), blo[SN], bhi[SN], CHK);
+            }
+            // MX: the scale dwords of step kt+1 leave their slot for the other register set, one per m-block
+            if constexpr (MX && mi >= MR - (MP + NP)) read_sc((S + 1) % T8_NS, mi - (MR - (MP + NP)), sav[SS ^ 1], sbv[SS ^ 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            const v4i alo = flo[mi % FRAG_BUFS], ahi = fhi[mi % FRAG_BUFS];
+            if constexpr (KIND == KIND_INT8) {
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], blo[SB][ni], alo);
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) mfma_i8(acc[mi][ni], bhi[SB][ni], ahi);
+            } else if constexpr (IS16) {
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], blo[SB][ni], alo); else mfma_f16(acc[mi][ni], blo[SB][ni], alo);
+                }
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    if constexpr (KIND == KIND_BF16) mfma_bf16(acc[mi][ni], bhi[SB][ni], ahi); else mfma_f16(acc[mi][ni], bhi[SB][ni], ahi);
+                }
+            } else if constexpr (KIND == KIND_MXFP4) {
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    mfma_mx<0, ni & 1, mi & 1>(acc[mi][ni], blo[SB][ni], alo, sbv[SS][ni / 2], sav[SS][mi / 2]);
+                });
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    mfma_mx<1, ni & 1, mi & 1>(acc[mi][ni], bhi[SB][ni], ahi, sbv[SS][ni / 2], sav[SS][mi / 2]);
+                });
+            } else if constexpr (KIND == KIND_MXFP8) {
+                const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    const v8i bf = {blo[SB][ni][0], blo[SB][ni][1], blo[SB][ni][2], blo[SB][ni][3],
+                                    bhi[SB][ni][0], bhi[SB][ni][1], bhi[SB][ni][2], bhi[SB][ni][3]};
+                    mfma_mx8<SS, ni & 1, mi & 1>(acc[mi][ni], bf, af, sbv[SS][ni / 2], sav[SS][mi / 2]);
+                });
+            } else {
+                const v8i af = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+#pragma unroll
+                for (int ni = 0; ni < NR; ni++) {
+                    const v8i bf = {blo[SB][ni][0], blo[SB][ni][1], blo[SB][ni][2], blo[SB][ni][3],
+                                    bhi[SB][ni][0], bhi[SB][ni][1], bhi[SB][ni][2], bhi[SB][ni][3]};
+                    mfma_f8(acc[mi][ni], bf, af);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // The DMAs this wavefront issued one step ago (A tile of step kt+2) must have landed before the barrier: behind them
+        // it has issued the W loads of that step and everything of this step.
+        if constexpr ((T8_DBG & 1) == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N_W + N_DMA + N_W) : "memory");
+    };
+
+    // prologue: the epilogue's scales into LDS, A(0), A(1), A(2) (and their MX scales) by DMA, W(0..PFW-1) into registers
+    float ep_sa = 0.f, ep_sb = 0.f;
+    if constexpr (SCALED && STORE != STORE_ACC) {
+        if (tid < 256) {
+            const int m = m0 + tid, n = n0 + tid;
+            ep_sa = p.sa[m < p.M ? m : p.M - 1];
+            ep_sb = p.sb[n < p.N ? n : p.N - 1];
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) dma_a1(kt_begin + s, s, j, std::true_type{});
+        if constexpr (MX) {
+            dma_sc(kt_begin + s, s, 0);
+            dma_sc(kt_begin + s, s, 1);
+        }
+    }
+    static_for<PFW>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+#pragma unroll
+        for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin + i, idx, blo[i], bhi[i], std::true_type{});
+    });
+    if constexpr (SCALED && STORE != STORE_ACC) {
+        if (tid < 256) {
+            reinterpret_cast<float*>(lds_x)[tid] = ep_sa;
+            reinterpret_cast<float*>(lds_x)[256 + tid] = ep_sb;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PFW * 2 * NR) : "memory");
+    static_for<FRAG_AHEAD>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        read_frag(0, i, flo[i], fhi[i]);
+    });
+    if constexpr (MX) {
+#pragma unroll
+        for (int q = 0; q < MP + NP; q++) read_sc(0, q, sav[0], sbv[0]);
+    }
+
+    T8_STAMP(1);
+    // Four K steps per iteration (LDS stages and register sets are compile-time).  The loop bodies have no branches: the
+    // compiler's count of outstanding loads at the loop head is then the same on every path and its waits for W stay exact
+    // (with skipped steps inside the loop it assumed the worst case and waited for every load on every fourth step).
+    // The first loop runs while every load it issues (three steps ahead at most) lies inside the K range and before the
+    // K tail, so it issues them unchecked; the second one finishes the range with checked loads; the one to three steps
+    // that are left run behind it.
+    int kt = kt_begin;
+    const int kt_full = (K % TK) ? kt_end - 1 : kt_end;  // steps before this one have all 128 bytes
+    for (; kt + 7 <= kt_full; kt += 4) {
+        step(kt, std::integral_constant<int, 0>{}, std::false_type{});
+        step(kt + 1, std::integral_constant<int, 1>{}, std::false_type{});
+        step(kt + 2, std::integral_constant<int, 2>{}, std::false_type{});
+        step(kt + 3, std::integral_constant<int, 3>{}, std::false_type{});
+    }
+    for (; kt + 4 <= kt_end; kt += 4) {
+        step(kt, std::integral_constant<int, 0>{}, std::true_type{});
+        step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{});
+        step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{});
+        step(kt + 3, std::integral_constant<int, 3>{}, std::true_type{});
+    }
+    if (kt < kt_end) {
+        step(kt, std::integral_constant<int, 0>{}, std::true_type{});
+        if (kt + 1 < kt_end) step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{});
+        if (kt + 2 < kt_end) step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{});
+    }
+    // wait states between the last MFMA and the first ordinary read of an accumulator (the compiler does not know that the
+    // asm statements are MFMAs), and every DMA still on its way (redirected past the bounds) must be done before the
+    // stages are reused for C
+    asm volatile("s_nop 15\n\ts_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    T8_STAMP(2);
+
+    float sa_v[MR];
+    v4f sb_v[NR];
+    if constexpr (STORE != STORE_ACC && SCALED) {
+#pragma unroll
+        for (int mi = 0; mi < MR; mi++) sa_v[mi] = reinterpret_cast<const float*>(lds_x)[mi * 16 + li];
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) sb_v[ni] = *reinterpret_cast<const v4f*>(lds_x + 1024 + ((wave * NR + ni) * 16 + lg * 4) * 4);
+    }
+
+    if constexpr (STORE == STORE_ACC) {
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            const int m = m0 + mi * 16 + li;
+            if (m < p.M) {
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                    if (n < p.N) {
+                        const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
+                        const size_t slice = (size_t)blockIdx.y * (size_t)p.M * (size_t)p.N;
+                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + (slice + idx) * 4) = acc[mi][ni];
+                    }
+                });
+            }
+        });
+    } else {
+        // The whole 16-bit C tile (256 rows x 512 bytes = 128 KB) is staged in the four A stages and written as whole rows.
+        // Nothing here is conditional: columns past N are staged like the others (their scales were clamped) and dropped by the
+        // store pass.  Row mi*16 + li keeps the swizzle term li for every mi, so a lane's 32 staging addresses are two bases
+        // (one per n-block) plus compile-time offsets.
+        constexpr int ROWB = TN * 2, GR = ROWB / 16, XM = 15, NT = WAVES * 64;
+        uint8_t* st_base[NR];
+#pragma unroll
+        for (int ni = 0; ni < NR; ni++) st_base[ni] = lds + li * ROWB + (((((wave * NR + ni) * 2 + (lg >> 1)) ^ li) & (GR - 1)) << 4) + (lg & 1) * 8;
+        static_for<MR>([&](auto MI) {
+            constexpr int mi = decltype(MI)::value;
+            float sa = 0.f;
+            if constexpr (SCALED) sa = sa_v[mi];
+            static_for<NR>([&](auto NI) {
+                constexpr int ni = decltype(NI)::value;
+                const acc_t r = acc[mi][ni];
+                v4f x;
+                if constexpr (!SCALED) {
+                    x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+                } else {
+                    const v4f sb = sb_v[ni];
+                    x = (v4f){((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2], ((float)r[3] * sa) * sb[3]};
+                }
+                v2i out;
+                if constexpr (STORE == STORE_C) {
+                    out = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
+                } else {
+                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                    const uint16_t* bias_n = p.bias + (n < p.N ? n : 0);
+                    out = p.out == OUT_BF16 ? finish4_rt<OUT_BF16>(x, bias_n, p.epi) : finish4_rt<OUT_FP16>(x, bias_n, p.epi);
+                }
+                *reinterpret_cast<v2i*>(st_base[ni] + mi * 16 * ROWB) = out;
+            });
+        });
+        T8_STAMP(4);
+        __syncthreads();
+        T8_STAMP(5);
+        // thread -> granule tid % 32 of rows tid / 32 + 16 i.  Stores go through a descriptor over the rows of C from m0 on:
+        // rows >= M fall behind its bound and are dropped; a granule past N is redirected there.
+        {
+            const int g = tid & (GR - 1), r0 = tid / GR;
+            const int n = n0 + g * 8;
+            __amdgpu_buffer_rsrc_t rc = make_rsrc(reinterpret_cast<uint16_t*>(p.c) + (size_t)m0 * (size_t)p.N, (uint64_t)(p.M - m0) * (uint64_t)p.N * 2ull);
+            const uint32_t c_off = n < p.N ? ((uint32_t)r0 * (uint32_t)p.N + (uint32_t)n) * 2u : 0xFFFFFFF0u;
+            const uint32_t c_step = (uint32_t)(NT / GR) * (uint32_t)p.N * 2u;
+            const uint8_t* src = lds + r0 * ROWB + ((g ^ (r0 & XM)) << 4);
+            static_assert(NT / GR == 16, "the row swizzle term must not change from pass to pass");
+#pragma unroll
+            for (int i = 0; i < TM / (NT / GR); i++) {
+                const v4i v = *reinterpret_cast<const v4i*>(src + i * (NT / GR) * ROWB);
+                __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rc, (int)(n < p.N ? c_off + (uint32_t)i * c_step : 0xFFFFFFF0u), 0, 0);
+            }
+        }
+    }
+#ifdef T8_TIMING
+    T8_STAMP(6);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    T8_STAMP(3);
+#endif
+}
+
+template <int KIND, int STORE, int PFW>
+hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream) {
+    const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 255) / 256;
+    const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
+    A8W8Params q = p;
+    q.splits = splits;
+    hipLaunchKernelGGL((k_tiled8<KIND, STORE, PFW>), dim3(tiles_m * tiles_n, splits), dim3(512), 0, stream, q);
+    return hipGetLastError();
+}
+
+}  // namespace

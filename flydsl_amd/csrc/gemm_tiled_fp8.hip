@@ -1,6 +1,6 @@
-// Instantiations of the tiled MFMA mainloop (gemm_tiled.h) for fp8 operands; one translation unit per operand
+// Instantiations of the tiled MFMA mainloop (gemm_tiled.h, gemm_tiled8.h) for fp8 operands; one translation unit per operand
 // type so that the instantiations compile in parallel.
-#include "gemm_tiled.h"
+#include "gemm_tiled8.h"
 
 hipError_t psg_launch_tiled_fp8(const A8W8Params& p, int store, int tile_m, int tile_n, hipStream_t stream) {
     if (store == STORE_ACC) return launch_shape<KIND_FP8, STORE_ACC>(p, tile_m, tile_n, stream);

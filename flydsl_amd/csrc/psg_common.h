@@ -90,12 +90,24 @@ __device__ __forceinline__ float from_out16(uint16_t b) {
     }
 }
 
-// four fp32 -> four 16-bit outputs packed into 8 bytes
+// four fp32 -> four 16-bit outputs packed into 8 bytes; two values per conversion instruction (v_cvt_pk_bf16_f32 /
+// v_cvt_pk_f16_f32, round to nearest even like the scalar conversions)
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+template <int OUT>
+__device__ __forceinline__ int pack2_out16(float a, float b) {
+    const v2f x = {a, b};
+    if constexpr (OUT == OUT_BF16) {
+        return __builtin_bit_cast(int, __builtin_convertvector(x, v2bf));
+    } else {
+        return __builtin_bit_cast(int, __builtin_convertvector(x, v2h));
+    }
+}
 template <int OUT>
 __device__ __forceinline__ v2i pack4_out16(float a, float b, float c, float d) {
     v2i r;
-    r[0] = (int)((uint32_t)to_out16<OUT>(a) | ((uint32_t)to_out16<OUT>(b) << 16));
-    r[1] = (int)((uint32_t)to_out16<OUT>(c) | ((uint32_t)to_out16<OUT>(d) << 16));
+    r[0] = pack2_out16<OUT>(a, b);
+    r[1] = pack2_out16<OUT>(c, d);
     return r;
 }
 

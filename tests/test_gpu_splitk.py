@@ -144,7 +144,7 @@ def test_two_streams_take_the_split_plan_without_sharing_a_workspace():
         for t, ref, c, s, fn in work:
             fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s)
     torch.cuda.synchronize()
-    bufs = [_lib._pool._live[(id(w[4]), torch.cuda.current_device(), _lib.stream_handle(w[3]))] for w in work]
+    bufs = [_lib._pool._live[(w[4]._ws_owner, torch.cuda.current_device(), _lib.stream_handle(w[3]))] for w in work]
     assert bufs[0] is not bufs[1]
     # one launcher on two streams: separate buffers as well
     t, ref, c, s, fn = work[0]
@@ -153,7 +153,7 @@ def test_two_streams_take_the_split_plan_without_sharing_a_workspace():
     fn(c, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s)
     fn(c2, t["a_q"], t["b_shuf"], t["sa"], t["sb"], bias, M, N, s2)
     torch.cuda.synchronize()
-    assert _lib._pool._live[(id(fn), torch.cuda.current_device(), _lib.stream_handle(s2))] is not bufs[0]
+    assert _lib._pool._live[(fn._ws_owner, torch.cuda.current_device(), _lib.stream_handle(s2))] is not bufs[0]
     assert np.array_equal(bf16_bits(c2), ref)
     for t, ref, c, s, fn in work:
         assert np.array_equal(bf16_bits(c), ref)
