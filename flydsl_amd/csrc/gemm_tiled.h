@@ -489,7 +489,7 @@ hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
 }
 
 // the 256x256 tile of eight wavefronts has a kernel of its own (gemm_tiled8.h, which includes this file)
-template <int KIND, int STORE, int PFW>
+template <int KIND, int STORE, int OPT>
 hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream);
 
 // p.wave_layout selects the wavefront layout of the 256x256 tile: 2 = 2x2 wavefronts, 8 = eight wavefronts along N, anything
@@ -502,7 +502,7 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
         PSG_CASE(8, 8, 2)
     }
     if (p.wave_layout == 8) {  // eight wavefronts side by side along N: 256x256 tile, every W fragment loaded once
-        if (tile_m == 256 && tile_n == 256) return launch_tiled8<KIND, STORE, 1>(p, stream);
+        if (tile_m == 256 && tile_n == 256) return launch_tiled8<KIND, STORE, 0>(p, stream);
     }
     if constexpr (KIND != KIND_MXFP4 && KIND != KIND_MXFP8) {
         // few tiles (p.ksplit = 3: the planner's mark for launches of at most two workgroups per CU): W fetched three steps ahead

@@ -18,6 +18,15 @@
 //     return in order, and the compiler counts only the W loads it knows about, so within a step the DMAs are issued
 //     before the W loads and only behind the first MFMAs (where the compiler waits for this step's W fragments): a
 //     compiler-made vmcnt then never covers a DMA that was issued a moment ago.
+//   * MX scale dwords take the same road (4-byte DMAs into a slot per stage, read back one step ahead): as register
+//     loads the compiler had to wait for all of them, i.e. for every load in flight, at the top of every step.
+//   * Every descriptor an instruction of the loop uses is built from values forced into scalar registers
+//     (make_rsrc_uniform): left to the compiler, the W descriptor of some builds lived in vector registers and every W load
+//     paid four v_readfirstlane (350 core cycles per fp8 K step).
+//   * In steady state no load is predicated: the selects and compares that redirect loads past the K range run only in
+//     the last steps (a second copy of the loop), not in front of the MFMAs of every step.
+//   * C leaves through LDS as whole rows, in two halves: the stores of rows 0..127 are under way while rows 128..255 are
+//     converted.  Epilogue scales wait in LDS since the prologue.
 #pragma once
 #include "gemm_tiled.h"
 
@@ -41,11 +50,10 @@ __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, uint32_t lds_add
                  : "memory");
 }
 
-#ifndef T8_DBG
-#define T8_DBG 0
-#endif
+// Built with -DT8_TIMING (a measuring harness, never the library) thread 0 of every workgroup records the core clock and the
+// 10 ns wall clock at: 0 start, 1 loop begin, 2 loop end, 4 C staged, 5 behind the barrier, 6 stores issued, 3 stores done.
 #ifdef T8_TIMING
-__device__ unsigned long long* t8_dbg;  // per workgroup: 8 x (core clock, 10 ns wall clock) at start / loop begin / loop end / kernel end
+__device__ unsigned long long* t8_dbg;
 #define T8_STAMP(i) do { if (threadIdx.x == 0) { t8_dbg[blockIdx.x * 16 + 2 * (i)] = clock64(); t8_dbg[blockIdx.x * 16 + 2 * (i) + 1] = wall_clock64(); } } while (0)
 #else
 #define T8_STAMP(i) do { } while (0)
@@ -57,14 +65,19 @@ __device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr
                  : "memory");
 }
 
-// PFW = K steps the W fragments are fetched ahead of their MFMAs (1 or 3; PFW + 1 register sets)
-template <int KIND, int STORE, int PFW>
+// OPT (0 in the library; the other builds exist to be measured against it): bit 0 staggers the memory instructions of the two
+// wavefronts that share a SIMD (w and w + 4) by two m-blocks, bit 1 raises the wave priority around the MFMAs.  fp8
+// 8192x4096x4096, core cycles per K step / us per launch: plain 2,311 / 114.5, staggered 2,354 / 115.5, staggered with
+// priority 2,425 / 115.4 (2,048 cycles is the issue limit of the 64 MFMAs per SIMD).  W fragments are fetched one K step
+// ahead (two register sets): three steps ahead (four sets) measured the same and leaves the allocator no room.
+constexpr int T8_STAGGER = 1, T8_SETPRIO = 2;
+template <int KIND, int STORE, int OPT = 0>
 __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
+    constexpr int PFW = 1;
     using acc_t = typename Acc<KIND>::type;
     constexpr int MR = 16, NR = 2, WAVES = 8;
     constexpr int TM = 256, TN = 256;
     constexpr int NB = PFW + 1;
-    static_assert(NB == 2 || NB == 4, "W register sets");
     constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
     constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;
     constexpr bool MX = KIND == KIND_MXFP4 || KIND == KIND_MXFP8;
@@ -100,7 +113,7 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     const int nb0 = (n0 >> 4) + wave * NR;
     const uint64_t b_off = (uint64_t)nb0 * 16ull * (uint64_t)K;
     const uint64_t b_total = (uint64_t)p.N * (uint64_t)K;
-    __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
+    __amdgpu_buffer_rsrc_t rb = make_rsrc_uniform(p.b + (b_off < b_total ? b_off : b_total), b_off < b_total ? b_total - b_off : 0);
 
     // MX scales: per (32-row chunk, 256-element K chunk) 64 dwords, one per lane.  Wavefront w brings A-side chunk w of the
     // tile and its own W-side chunk (32 columns) into the slot of the step by two 4-byte DMAs; chunks past the end read
@@ -137,56 +150,54 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     }
     // CHK = false: the step is known to lie inside [kt_begin, kt_end) and not to be the K tail, so nothing is redirected (the
     // selects and compares of the checked form are ten instructions per load in front of the MFMAs of both wavefronts of a SIMD)
-    auto dma_a1 = [&](int kt, int stage, int j, auto CHK) {
+    auto dma_a1 = [&](int kt, int stage, int j, auto CHK) __attribute__((always_inline)) {
         const uint32_t dst = lds_base + (uint32_t)(stage * T8_STAGE + (wave * 4 + j) * 1024);
         if constexpr (decltype(CHK)::value) {
             const bool in_k = kt < kt_end && (uint32_t)(kt * TK + a_kc[j & 1] * 16) < (uint32_t)K;
-            dma16(ra, dst, in_k ? a_voff[j] : 0xFFFFFFF0u, (kt < kt_end && !(T8_DBG & 64)) ? (uint32_t)kt * TK : 0u);
+            dma16(ra, dst, in_k ? a_voff[j] : 0xFFFFFFF0u, kt < kt_end ? (uint32_t)kt * TK : 0u);
         } else {
-            dma16(ra, dst, a_voff[j], (T8_DBG & 64) ? 0u : (uint32_t)kt * TK);
+            dma16(ra, dst, a_voff[j], (uint32_t)kt * TK);
         }
     };
 
     // scale dwords of step kt -> slot (two DMAs per wavefront), and slot -> registers
-    auto dma_sc = [&](int kt, int slot, int which) {
+    auto dma_sc = [&](int kt, int slot, int which) __attribute__((always_inline)) {
         const bool has = kt < kt_end;
         const uint32_t dst = lds_base + (uint32_t)(T8_NS * T8_STAGE + slot * SC_SLOT + which * 2048 + wave * 256);
         dma4(which ? rsb : rsa, dst, has ? (uint32_t)lane * 4u : 0xFFFFFFF0u, has ? (uint32_t)(KIND == KIND_MXFP8 ? (kt >> 1) : kt) * 256u : 0u);
     };
-    auto read_sc = [&](int slot, int q, int* sa_dst, int* sb_dst) {
+    auto read_sc = [&](int slot, int q, int* sa_dst, int* sb_dst) __attribute__((always_inline)) {
         if (q < MP) sa_dst[q] = *reinterpret_cast<const int*>(lds_x + slot * SC_SLOT + q * 256 + lane * 4);
         else sb_dst[0] = *reinterpret_cast<const int*>(lds_x + slot * SC_SLOT + 2048 + wave * 256 + lane * 4);
     };
     const uint32_t b_lane_off = p.b_rowmajor ? (uint32_t)li * (uint32_t)K + (uint32_t)lg * 16u : (uint32_t)lane * 16u;
     const uint32_t b_step = p.b_rowmajor ? 128u : 2048u, b_half = p.b_rowmajor ? 64u : 1024u;
-    auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi, auto CHK) {
+    auto load_b1 = [&](int kt, int idx, v4i* lo, v4i* hi, auto CHK) __attribute__((always_inline)) {
         const int ni = idx >> 1;
         const bool has = !decltype(CHK)::value || (kt < kt_end && (kt * TK + (idx & 1) * 64) < K);
         const uint32_t voff = b_lane_off + (uint32_t)ni * 16u * (uint32_t)K;
-        v4i v;
-        if constexpr ((T8_DBG & 128) != 0) {  // timing experiment: the same registers filled from LDS instead of memory
-            v = *reinterpret_cast<const v4i*>(&lds[((kt & 3) * 8 + idx) * 1024 + lane * 16]);
-        } else {
-            v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, (has && !(T8_DBG & 64)) ? (uint32_t)kt * b_step + (uint32_t)(idx & 1) * b_half : 0u);
-        }
+        const v4i v = buf_load16(rb, has ? voff : 0xFFFFFFF0u, has ? (uint32_t)kt * b_step + (uint32_t)(idx & 1) * b_half : 0u);
         if (idx & 1) hi[ni] = v; else lo[ni] = v;
     };
     // fragment (16 rows x 2 x 16 bytes of K) of m-block mi from a stage: row mi*16 + li, chunks lg and 4 + lg; the swizzle
     // term (row/2)%8 = (li/2)%8 does not depend on mi
     const int f_lo = li * TK + ((lg ^ ((li >> 1) & 7)) << 4);
     const int f_hi = li * TK + (((4 + lg) ^ ((li >> 1) & 7)) << 4);
-    auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) {
+    auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) __attribute__((always_inline)) {
         flo = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_lo]);
         fhi = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_hi]);
     };
 
-    constexpr int FRAG_AHEAD = (T8_DBG & 16) ? 3 : 2, FRAG_BUFS = 4;  // 16 m-blocks per step: buffer mi % 4 lines up across steps
+    constexpr int FRAG_AHEAD = 2, FRAG_BUFS = 4;  // 16 m-blocks per step: buffer mi % 4 lines up across steps
     v4i flo[FRAG_BUFS], fhi[FRAG_BUFS];
 
     // One K step: MFMAs on LDS stage S and W set SB.  m-block 0 only multiplies (the compiler waits for this step's W
-    // fragments there); m-blocks 1..4 each issue one DMA of the A tile of step kt+3, m-blocks 5.. the W loads (and MX scale
-    // dwords) of step kt+PFW; every m-block reads the A fragment two m-blocks ahead, the last two those of step kt+1.
-    auto step = [&](int kt, auto SP, auto CHK) {
+    // fragments there); from m-block 1 on one memory instruction per m-block: four DMAs of the A tile of step kt+3 (MX: and
+    // two of its scale chunks), then the four W loads of step kt+1; every m-block reads the A fragment two m-blocks ahead,
+    // the last two those of step kt+1.
+    // (always_inline: with 22 call sites the inliner would otherwise leave this lambda a function of its own, with the
+    // accumulators and descriptors passed through memory)
+    auto step = [&](int kt, auto SP, auto CHK, auto GRP) __attribute__((always_inline)) {
         constexpr int S = decltype(SP)::value;   // LDS stage of this step (kt % 4)
         constexpr int SB = S % NB;               // W register set of this step
         constexpr int SN = (SB + PFW) % NB;      // W register set the loads of this step fill
@@ -195,23 +206,26 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
         constexpr int N_W = 2 * NR;              // W fragment loads per wavefront per step
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
-            if constexpr ((T8_DBG & 2) != 0) {
-            } else if constexpr (mi + FRAG_AHEAD < MR)
+            if constexpr (mi + FRAG_AHEAD < MR)
                 read_frag(S, mi + FRAG_AHEAD, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
             else
                 read_frag((S + 1) % T8_NS, mi + FRAG_AHEAD - MR, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
-            // memory instructions, one m-block each from m-block 1 on: the DMAs of step kt+3, then the W loads of step kt+PFW
-            if constexpr (mi >= 1 && mi <= 4) {
-                if constexpr ((T8_DBG & 4) == 0) dma_a1(kt + 3, (S + 3) % T8_NS, mi - 1, CHK);
-            } else if constexpr (MX && mi == 5) {
+            // memory instructions, one m-block each: the DMAs of step kt+3, then the W loads of step kt+1.  The first four
+            // wavefronts (one per SIMD) start at m-block 1, their SIMD partners two m-blocks later (GRP)
+            constexpr int OFF = decltype(GRP)::value ? 2 : 0;
+            constexpr int W0 = (MX ? 6 : 5) + OFF;
+            if constexpr (mi >= 1 + OFF && mi <= 4 + OFF) {
+                dma_a1(kt + 3, (S + 3) % T8_NS, mi - 1 - OFF, CHK);
+            } else if constexpr (MX && mi == 5 + OFF) {
                 dma_sc(kt + 3, (S + 3) % T8_NS, 0);
                 dma_sc(kt + 3, (S + 3) % T8_NS, 1);
-            } else if constexpr (mi >= (MX ? 6 : 5) && mi < (MX ? 6 : 5) + N_W) {
-                if constexpr ((T8_DBG & 8) == 0) load_b1(kt + PFW, mi - (MX ? 6 : 5), blo[SN], bhi[SN], CHK);
+            } else if constexpr (mi >= W0 && mi < W0 + N_W) {
+                load_b1(kt + PFW, mi - W0, blo[SN], bhi[SN], CHK);
             }
             // MX: the scale dwords of step kt+1 leave their slot for the other register set, one per m-block
             if constexpr (MX && mi >= MR - (MP + NP)) read_sc((S + 1) % T8_NS, mi - (MR - (MP + NP)), sav[SS ^ 1], sbv[SS ^ 1]);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr ((OPT & T8_SETPRIO) != 0) asm volatile("s_setprio 1" ::: "memory");
             const v4i alo = flo[mi % FRAG_BUFS], ahi = fhi[mi % FRAG_BUFS];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
@@ -253,11 +267,12 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
                     mfma_f8(acc[mi][ni], bf, af);
                 }
             }
+            if constexpr ((OPT & T8_SETPRIO) != 0) asm volatile("s_setprio 0" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
         });
         // The DMAs this wavefront issued one step ago (A tile of step kt+2) must have landed before the barrier: behind them
         // it has issued the W loads of that step and everything of this step.
-        if constexpr ((T8_DBG & 1) == 0) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N_W + N_DMA + N_W) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N_W + N_DMA + N_W) : "memory");
     };
 
     // prologue: the epilogue's scales into LDS, A(0), A(1), A(2) (and their MX scales) by DMA, W(0..PFW-1) into registers
@@ -306,24 +321,32 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     // The first loop runs while every load it issues (three steps ahead at most) lies inside the K range and before the
     // K tail, so it issues them unchecked; the second one finishes the range with checked loads; the one to three steps
     // that are left run behind it.
-    int kt = kt_begin;
     const int kt_full = (K % TK) ? kt_end - 1 : kt_end;  // steps before this one have all 128 bytes
-    for (; kt + 7 <= kt_full; kt += 4) {
-        step(kt, std::integral_constant<int, 0>{}, std::false_type{});
-        step(kt + 1, std::integral_constant<int, 1>{}, std::false_type{});
-        step(kt + 2, std::integral_constant<int, 2>{}, std::false_type{});
-        step(kt + 3, std::integral_constant<int, 3>{}, std::false_type{});
-    }
-    for (; kt + 4 <= kt_end; kt += 4) {
-        step(kt, std::integral_constant<int, 0>{}, std::true_type{});
-        step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{});
-        step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{});
-        step(kt + 3, std::integral_constant<int, 3>{}, std::true_type{});
-    }
-    if (kt < kt_end) {
-        step(kt, std::integral_constant<int, 0>{}, std::true_type{});
-        if (kt + 1 < kt_end) step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{});
-        if (kt + 2 < kt_end) step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{});
+    auto run_steps = [&](auto GRP) __attribute__((always_inline)) {
+        int kt = kt_begin;
+        for (; kt + 7 <= kt_full; kt += 4) {
+            step(kt, std::integral_constant<int, 0>{}, std::false_type{}, GRP);
+            step(kt + 1, std::integral_constant<int, 1>{}, std::false_type{}, GRP);
+            step(kt + 2, std::integral_constant<int, 2>{}, std::false_type{}, GRP);
+            step(kt + 3, std::integral_constant<int, 3>{}, std::false_type{}, GRP);
+        }
+        for (; kt + 4 <= kt_end; kt += 4) {
+            step(kt, std::integral_constant<int, 0>{}, std::true_type{}, GRP);
+            step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{}, GRP);
+            step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{}, GRP);
+            step(kt + 3, std::integral_constant<int, 3>{}, std::true_type{}, GRP);
+        }
+        if (kt < kt_end) {
+            step(kt, std::integral_constant<int, 0>{}, std::true_type{}, GRP);
+            if (kt + 1 < kt_end) step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{}, GRP);
+            if (kt + 2 < kt_end) step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{}, GRP);
+        }
+    };
+    if constexpr ((OPT & T8_STAGGER) != 0) {
+        // two copies of the loops whose memory instructions sit in different m-blocks; the barriers pair up all the same
+        if (wave < 4) run_steps(std::false_type{}); else run_steps(std::true_type{});
+    } else {
+        run_steps(std::false_type{});
     }
     // wait states between the last MFMA and the first ordinary read of an accumulator (the compiler does not know that the
     // asm statements are MFMAs), and every DMA still on its way (redirected past the bounds) must be done before the
@@ -365,50 +388,51 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
         uint8_t* st_base[NR];
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) st_base[ni] = lds + li * ROWB + (((((wave * NR + ni) * 2 + (lg >> 1)) ^ li) & (GR - 1)) << 4) + (lg & 1) * 8;
-        static_for<MR>([&](auto MI) {
-            constexpr int mi = decltype(MI)::value;
-            float sa = 0.f;
-            if constexpr (SCALED) sa = sa_v[mi];
-            static_for<NR>([&](auto NI) {
-                constexpr int ni = decltype(NI)::value;
-                const acc_t r = acc[mi][ni];
-                v4f x;
-                if constexpr (!SCALED) {
-                    x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
-                } else {
-                    const v4f sb = sb_v[ni];
-                    x = (v4f){((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2], ((float)r[3] * sa) * sb[3]};
-                }
-                v2i out;
-                if constexpr (STORE == STORE_C) {
-                    out = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
-                } else {
-                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
-                    const uint16_t* bias_n = p.bias + (n < p.N ? n : 0);
-                    out = p.out == OUT_BF16 ? finish4_rt<OUT_BF16>(x, bias_n, p.epi) : finish4_rt<OUT_FP16>(x, bias_n, p.epi);
-                }
-                *reinterpret_cast<v2i*>(st_base[ni] + mi * 16 * ROWB) = out;
+        const int g = tid & (GR - 1), r0 = tid / GR;  // store pass: thread -> granule tid % 32 of rows tid / 32 + 16 i
+        const int n_st = n0 + g * 8;
+        // stores go through a descriptor over the rows of C from m0 on: rows >= M fall behind its bound and are dropped; a
+        // granule past N is redirected there
+        __amdgpu_buffer_rsrc_t rc = make_rsrc(reinterpret_cast<uint16_t*>(p.c) + (size_t)m0 * (size_t)p.N, (uint64_t)(p.M - m0) * (uint64_t)p.N * 2ull);
+        const uint32_t c_off = ((uint32_t)r0 * (uint32_t)p.N + (uint32_t)n_st) * 2u;
+        const uint32_t c_step = (uint32_t)(NT / GR) * (uint32_t)p.N * 2u;
+        const uint8_t* src = lds + r0 * ROWB + ((g ^ (r0 & XM)) << 4);
+        static_assert(NT / GR == 16, "the row swizzle term must not change from pass to pass");
+        static_for<2>([&](auto HALF) {
+            constexpr int half = decltype(HALF)::value;
+            static_for<MR / 2>([&](auto MI) {
+                constexpr int mi = half * (MR / 2) + decltype(MI)::value;
+                float sa = 0.f;
+                if constexpr (SCALED) sa = sa_v[mi];
+                static_for<NR>([&](auto NI) {
+                    constexpr int ni = decltype(NI)::value;
+                    const acc_t r = acc[mi][ni];
+                    v4f x;
+                    if constexpr (!SCALED) {
+                        x = (v4f){(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+                    } else {
+                        const v4f sb = sb_v[ni];
+                        x = (v4f){((float)r[0] * sa) * sb[0], ((float)r[1] * sa) * sb[1], ((float)r[2] * sa) * sb[2], ((float)r[3] * sa) * sb[3]};
+                    }
+                    v2i out;
+                    if constexpr (STORE == STORE_C) {
+                        out = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
+                    } else {
+                        const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                        const uint16_t* bias_n = p.bias + (n < p.N ? n : 0);
+                        out = p.out == OUT_BF16 ? finish4_rt<OUT_BF16>(x, bias_n, p.epi) : finish4_rt<OUT_FP16>(x, bias_n, p.epi);
+                    }
+                    *reinterpret_cast<v2i*>(st_base[ni] + mi * 16 * ROWB) = out;
+                });
             });
-        });
-        T8_STAMP(4);
-        __syncthreads();
-        T8_STAMP(5);
-        // thread -> granule tid % 32 of rows tid / 32 + 16 i.  Stores go through a descriptor over the rows of C from m0 on:
-        // rows >= M fall behind its bound and are dropped; a granule past N is redirected there.
-        {
-            const int g = tid & (GR - 1), r0 = tid / GR;
-            const int n = n0 + g * 8;
-            __amdgpu_buffer_rsrc_t rc = make_rsrc(reinterpret_cast<uint16_t*>(p.c) + (size_t)m0 * (size_t)p.N, (uint64_t)(p.M - m0) * (uint64_t)p.N * 2ull);
-            const uint32_t c_off = n < p.N ? ((uint32_t)r0 * (uint32_t)p.N + (uint32_t)n) * 2u : 0xFFFFFFF0u;
-            const uint32_t c_step = (uint32_t)(NT / GR) * (uint32_t)p.N * 2u;
-            const uint8_t* src = lds + r0 * ROWB + ((g ^ (r0 & XM)) << 4);
-            static_assert(NT / GR == 16, "the row swizzle term must not change from pass to pass");
+            if constexpr (half == 1) T8_STAMP(4);
+            __syncthreads();
+            if constexpr (half == 1) T8_STAMP(5);
 #pragma unroll
-            for (int i = 0; i < TM / (NT / GR); i++) {
+            for (int i = half * (TM / 32); i < (half + 1) * (TM / 32); i++) {
                 const v4i v = *reinterpret_cast<const v4i*>(src + i * (NT / GR) * ROWB);
-                __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rc, (int)(n < p.N ? c_off + (uint32_t)i * c_step : 0xFFFFFFF0u), 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rc, (int)(n_st < p.N ? c_off + (uint32_t)i * c_step : 0xFFFFFFF0u), 0, 0);
             }
-        }
+        });
     }
 #ifdef T8_TIMING
     T8_STAMP(6);
@@ -417,13 +441,13 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
 #endif
 }
 
-template <int KIND, int STORE, int PFW>
+template <int KIND, int STORE, int OPT>
 hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream) {
     const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 255) / 256;
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     A8W8Params q = p;
     q.splits = splits;
-    hipLaunchKernelGGL((k_tiled8<KIND, STORE, PFW>), dim3(tiles_m * tiles_n, splits), dim3(512), 0, stream, q);
+    hipLaunchKernelGGL((k_tiled8<KIND, STORE, OPT>), dim3(tiles_m * tiles_n, splits), dim3(512), 0, stream, q);
     return hipGetLastError();
 }
 
