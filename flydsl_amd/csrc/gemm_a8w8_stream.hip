@@ -321,7 +321,7 @@ hipError_t launch_planned(const A8W8Params& p0, int kbytes, hipStream_t stream) 
     while (ks > 1 && ks * 2 > steps) ks >>= 1;
     const int gpw = nwaves / ks;
     const long units = p.N / 8;
-    const long cus = 256;
+    const long cus = psg_cu_count();
     const long rounds = (units + 4 * cus * gpw - 1) / (4 * cus * gpw);
     long tg = cus * gpw * rounds;  // column groups: a whole number of workgroups per CU ...
     if (tg > units) tg = units;    // ... but never less than one 8-column unit per group

@@ -119,7 +119,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
         blk = (int)blockIdx.x / p.n_tiles;  // block of TM sorted rows; the sorter's blocks hold TM << eshift rows
         n_tile = (int)blockIdx.x % p.n_tiles;
     }
-    if (blk * TM >= p.num_valid[0]) return;
+    // the quad order rounds the row blocks up to an even number: the odd one out has no entry in expert_ids
+    if ((blk >> p.eshift) >= p.blocks || blk * TM >= p.num_valid[0]) return;
     const int e = p.expert_ids[blk >> p.eshift];
     if ((unsigned)e >= (unsigned)p.experts) return;
     if (p.by_expert) n_tile += ((int)blockIdx.x - e * p.n_tiles) & 7;
@@ -350,6 +351,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR <= 
 template <int AF, int STAGE>
 hipError_t launch_rows(MoeMxParams p, int block_m, int blocks, hipStream_t stream) {
     p.eshift = block_m == 128 ? 1 : 0;
+    p.blocks = blocks;
     p.n_tiles = p.n_out / (STAGE == 1 ? 128 : 256);
     p.n_groups = (p.n_tiles + 7) / 8;
     // Keyed by expert while an expert has few rows (then sharing an L2 is what saves re-reads: 256 tokens x top-8 on 32 experts,

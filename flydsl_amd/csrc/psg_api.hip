@@ -124,11 +124,12 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
         const int tm = shapes[i].m, tn = shapes[i].n;
         const long tiles_m = (M + tm - 1) / tm, tiles_n = (N + tn - 1) / tn;
         const long tiles = tiles_m * tiles_n;
-        const long slots = 256L * shapes[i].per_cu;
+        const long cus = psg_cu_count();
+        const long slots = cus * shapes[i].per_cu;
         const long rounds = (tiles + slots - 1) / slots;
         // a partly filled last round still costs a full tile time on the CUs it touches
         const double fill = (double)tiles / (double)(rounds * slots);
-        const double busy = tiles >= slots ? fill : (double)(tiles < 256 ? tiles : 256) / 256.0;
+        const double busy = tiles >= slots ? fill : (double)(tiles < cus ? tiles : cus) / (double)cus;
         const double pad = ((double)M / (double)(tiles_m * tm)) * ((double)N / (double)(tiles_n * tn));
         const double score = busy * pad * shapes[i].eff;
         if (score > best) {
@@ -147,14 +148,15 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
 int pick_splits(int M, int N, int kbytes, Tile t) {
     const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
     const int steps = (kbytes + 127) / 128;
-    if (tiles >= 192 || steps < 32) return 1;
+    const long cus = psg_cu_count();
+    if (tiles >= cus * 3 / 4 || steps < 32) return 1;
     // measured on operands that do not fit the last-level cache: at least 12 K steps per workgroup, at most one workgroup per
-    // CU (256) in total, partial traffic bounded: a quarter of W once half the CUs have a workgroup; while more than half would
+    // CU in total, partial traffic bounded: a quarter of W once half the CUs have a workgroup; while more than half would
     // stay idle the bound is five times looser, because an idle CU costs more than the partial sums (fp8, us for 1/2/4/8 splits
     // of 128x128 tiles: 96x4096x14336 68/41/28/24, 512x4096x14336 71/48/49/60, 96x8192x8192 43/31/25/28, 384x5120x13824
     // 67/46/47/58, 512x5120x5120, 160 tiles, 30/37)
     int s = 1;
-    while (s < 8 && steps / (s * 2) >= 12 && tiles * (s * 2) <= 256 && (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s <= 128 ? 5 : 1))
+    while (s < 8 && steps / (s * 2) >= 12 && tiles * (s * 2) <= cus && (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s <= cus / 2 ? 5 : 1))
         s *= 2;
     return s;
 }
@@ -167,7 +169,7 @@ int mx_general_splits(int M, int N, int K) {
     const long tiles = (long)((M + (M <= 32 ? 31 : 63)) / (M <= 32 ? 32 : 64)) * (long)((N + 127) / 128);
     const int steps = K / 128;
     int s = 1;
-    while (s < 8 && tiles * (s * 2) <= 512 && steps / (s * 2) >= 8 && (uint64_t)(s * 2) * (uint64_t)M * (uint64_t)N * 8ull <= w_bytes / 4) s *= 2;
+    while (s < 8 && tiles * (s * 2) <= 2L * psg_cu_count() && steps / (s * 2) >= 8 && (uint64_t)(s * 2) * (uint64_t)M * (uint64_t)N * 8ull <= w_bytes / 4) s *= 2;
     return s;
 }
 
@@ -181,7 +183,7 @@ Plan plan_tiled(int M, int N, int kbytes, bool mx) {
     Tile t = pick_tile(M, N, mx, 0, 0);
     const long tiles_big = (long)((M + 127) / 128) * (long)((N + 255) / 256);
     const int steps = (kbytes + 127) / 128;
-    if (!mx && tiles_big < 192 && steps >= 48) t = M <= 64 ? Tile{64, 64, 4} : Tile{128, 128, 4};
+    if (!mx && tiles_big < psg_cu_count() * 3L / 4 && steps >= 48) t = M <= 64 ? Tile{64, 64, 4} : Tile{128, 128, 4};
     // Shorter rows (8..47 steps; K = 4096 one-byte elements is 32): while at most about 600 of them exist, 64x64 tiles beat
     // every larger shape, with or without split-K: many small workgroups keep more bytes of W in flight than a few large ones
     // (fp8, weights not cache-resident: M=128, N=K=4096 14.0 us against 19.4 with 128x128 tiles and two K splits; M=256,
@@ -255,6 +257,9 @@ int check_moe_sort(const psg_moe_sort_args* a, bool need_routing, MoeSortParams*
     if (a->topk < 1 || a->topk > 255) return fail(PSG_E_SHAPE, "topk=%d outside [1, 255]", a->topk);
     if (a->experts < 1 || a->experts > psg_moe_sort_max_experts()) return fail(PSG_E_SHAPE, "experts=%d outside [1, %d]", a->experts, psg_moe_sort_max_experts());
     if (a->block_m < 1 || a->block_m > 4096) return fail(PSG_E_SHAPE, "block_m=%d outside [1, 4096]", a->block_m);
+    // the bound below (the reference's) counts at most one partly filled block per expert and at least topk rows routed: with
+    // more slots than experts a token repeats an expert and the padded total can exceed it
+    if (a->topk > a->experts) return fail(PSG_E_SHAPE, "topk=%d exceeds experts=%d", a->topk, a->experts);
     const int64_t pairs = (int64_t)a->tokens * a->topk;
     const int64_t need = pairs + (int64_t)a->experts * a->block_m - a->topk;
     if (need > 0x7FFFFFFF) return fail(PSG_E_SHAPE, "tokens*topk + experts*block_m must stay below 2^31");
@@ -393,7 +398,22 @@ int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
     return run_a8w8(args, args->c, STORE_C, stream);
 }
 
+// Compute units of the current device, read once (the planners deal workgroups out per CU).  Without a device (host-only use of
+// the planning entry points) the MI355X's 256.
+int psg_cu_count() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        return cus;
+    }();
+    return n;
+}
+
 int psg_init(void) {
+    (void)psg_cu_count();
     void* ptr = nullptr;
     if (int rc = static_scratch(&ptr)) return rc;
     g_err[0] = 0;
@@ -584,7 +604,7 @@ static int mx_common(const psg_mxfp4_args* a, void* out, int store, void* stream
         const Plan plan = plan_tiled(a->M, a->N, a->K / 2, true);
         const Tile t = forced ? Tile{a->tile_m, a->tile_n, 4} : plan.t;
         int splits = forced ? (a->tile_k >= 1 && a->tile_k <= 16 ? a->tile_k : 1) : plan.splits;
-        if (store != STORE_C || !a->workspace || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
+        if (store != STORE_C || !a->workspace || !aligned(a->workspace, 16) || a->workspace_bytes < splitk_bytes(a->M, a->N, splits)) splits = 1;
         A8W8Params q{};
         q.c = p.c;
         q.a = p.a;

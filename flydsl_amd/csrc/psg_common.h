@@ -111,6 +111,9 @@ __device__ __forceinline__ v2i pack4_out16(float a, float b, float c, float d) {
     return r;
 }
 
+// compute units of the current device (host; defined next to psg_init, read once)
+int psg_cu_count();
+
 // Arguments shared by the 8-bit kernels.  Plain data, passed by value.
 struct A8W8Params {
     void* c;             // [M,N] out16, or raw accumulators when STORE_ACC
@@ -208,6 +211,7 @@ struct MoeMxParams {
     int n_tiles, n_groups;      // set by the launcher: column tiles of the output, and groups of 8 of them
     int by_expert;              // set by the launcher: workgroup ids are mapped to XCDs by (expert, column tile)
     int quad_tiles;             // set by the launcher: workgroup ids are mapped to XCDs by (row block parity, column tile % 4)
+    int blocks;                 // set by the launcher: entries of expert_ids (a workgroup id past the last block leaves at once)
 };
 
 // Arguments of the device-side expert sorter (the step in front of the MoE grouped GEMMs).

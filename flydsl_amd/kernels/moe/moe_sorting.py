@@ -30,8 +30,12 @@ def moe_sorting_get_workspace_size(M, num_experts, topk, unit_size=UNIT_SIZE):
 
 
 def _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size, expert_mask,
-               workspace, device, routing=()):
-    """Checks the sorter's tensors and fills a ``psg_moe_sort_args`` (``routing`` = (topk_ids, topk_weights) when they are read)."""
+               workspace, device, routing=(), stream_h=0):
+    """Checks the sorter's tensors and fills a ``psg_moe_sort_args`` (``routing`` = (topk_ids, topk_weights) when they are read).
+    A workspace the caller did not bring comes from the library's pool for (device, stream ``stream_h``): those buffers are never
+    released, so the up to three queued launches can still read it after this call has returned, whatever stream they run on
+    (a tensor from the caching allocator would be handed to other work as soon as it is dropped here); the pool refuses to grow
+    during graph capture."""
     E, B = int(num_experts), int(unit_size)
     need_rows, _ = sorted_sizes(tokens, topk, E, B)
     checks = [("sorted_ids", sorted_ids, torch.int32, need_rows), ("sorted_weights", sorted_weights, torch.float32, need_rows),
@@ -59,7 +63,7 @@ def _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_
         args.zero_buf, args.zero_bytes = moe_buf.data_ptr(), moe_buf.numel() * moe_buf.element_size()
     want = int(_lib.lib().psg_moe_sorting_workspace_bytes(tokens, topk, E))
     if workspace is None and want:
-        workspace = torch.empty(want, dtype=torch.uint8, device=device)
+        workspace = _lib.workspace(device, want, stream_h, owner="moe_sort")
     if workspace is not None and workspace is not False:
         if not workspace.is_cuda or not workspace.is_contiguous():
             raise ValueError("workspace must be a contiguous device tensor")
@@ -95,10 +99,11 @@ def moe_sorting_flydsl(topk_ids, topk_weights, sorted_ids, sorted_weights, sorte
         raise ValueError("topk_ids and topk_weights must both be [tokens, topk]")
     tokens, topk = topk_ids.shape
     tokens = _local_tokens(num_local_tokens, tokens)
+    stream_h = _lib.stream_handle(stream)
     args, _ws = _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size,
-                           expert_mask, workspace, topk_ids.device, routing=(topk_ids, topk_weights))
+                           expert_mask, workspace, topk_ids.device, routing=(topk_ids, topk_weights), stream_h=stream_h)
     handle = _lib.lib()
-    rc = handle.psg_moe_sorting(ctypes.byref(args), _lib.stream_handle(stream))
+    rc = handle.psg_moe_sorting(ctypes.byref(args), stream_h)
     if rc != 0:
         raise (ValueError if rc < 0 else RuntimeError)(handle.psg_last_error().decode())
     return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf
@@ -111,7 +116,9 @@ def moe_softmax_sort_flydsl(gating_logits, sorted_ids, sorted_weights, sorted_ex
     same positional arguments and the same outputs as ``moe_sorting_flydsl``.  For decode-sized batches (16 tokens with 256
     experts, 32 with up to 128) this is ONE launch (every sorting workgroup repeats the gating of all tokens in LDS; ``topk_ids`` / ``topk_weights`` are then optional extra
     outputs); beyond that the gating kernel and the sorter run back to back, through ``topk_ids`` / ``topk_weights`` when the
-    caller gives them (``[tokens, topk]`` int32 / fp32; needed under graph capture) and through fresh tensors otherwise."""
+    caller gives them (``[tokens, topk]`` int32 / fp32) and through a buffer of the library's pool for this device and stream
+    otherwise (never released, so the queued launches may outlive this call on any stream; the pool does not grow during
+    graph capture: run the call once before capturing, or bring the tensors)."""
     from .topk_gating_softmax import gating_args
 
     if gating_logits.dim() != 2 or gating_logits.shape[1] != int(num_experts):
@@ -119,15 +126,18 @@ def moe_softmax_sort_flydsl(gating_logits, sorted_ids, sorted_weights, sorted_ex
     tokens, topk = _local_tokens(num_local_tokens, int(gating_logits.shape[0])), int(topk)
     handle = _lib.lib()
     fused = bool(handle.psg_moe_softmax_sorting_fused(tokens, topk, int(num_experts)))
-    if not fused:
+    stream_h = _lib.stream_handle(stream)
+    if not fused and (topk_ids is None or topk_weights is None):
+        n = tokens * topk
+        tmp = _lib.workspace(gating_logits.device, 8 * n, stream_h, owner="moe_softmax_sort")
         if topk_ids is None:
-            topk_ids = torch.empty((tokens, topk), dtype=torch.int32, device=gating_logits.device)
+            topk_ids = tmp[: 4 * n].view(torch.int32).view(tokens, topk)
         if topk_weights is None:
-            topk_weights = torch.empty((tokens, topk), dtype=torch.float32, device=gating_logits.device)
+            topk_weights = tmp[4 * n: 8 * n].view(torch.float32).view(tokens, topk)
     gargs = gating_args(gating_logits, topk_weights, topk_ids, None, tokens, int(num_experts), topk, dtype_str, renormalize)
     sargs, _ws = _sort_args(tokens, topk, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf, num_experts, unit_size,
-                            expert_mask, workspace, gating_logits.device, routing=() if fused else (topk_ids, topk_weights))
-    rc = handle.psg_moe_softmax_sorting(ctypes.byref(gargs), ctypes.byref(sargs), _lib.stream_handle(stream))
+                            expert_mask, workspace, gating_logits.device, routing=() if fused else (topk_ids, topk_weights), stream_h=stream_h)
+    rc = handle.psg_moe_softmax_sorting(ctypes.byref(gargs), ctypes.byref(sargs), stream_h)
     if rc != 0:
         raise (ValueError if rc < 0 else RuntimeError)(handle.psg_last_error().decode())
     return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf

@@ -90,6 +90,11 @@ def flydsl_mxfp4_gemm1(*, a_quant, a_scale_sorted_shuffled, w1_u8, w1_scale_u8, 
         a_row = int(D_HIDDEN) // 2 if a_dtype == "fp4" else int(D_HIDDEN)
         if _rows(a_quant, a_row) < int(n_tokens):
             raise ValueError(f"a_quant holds {_rows(a_quant, a_row)} rows of {a_row} bytes, n_tokens={n_tokens}")
+        # the kernel's descriptor for these scales is sized from the sorted list, not from the tensor
+        need_scale = (int(m_indices.numel()) + 31) // 32 * 32 * (int(D_HIDDEN) // 32)
+        if a_scale_sorted_shuffled.numel() < need_scale:
+            raise ValueError(f"a_scale_sorted_shuffled holds {a_scale_sorted_shuffled.numel()} bytes, the sorted list of "
+                             f"{m_indices.numel()} rows needs ceil(rows / 32) * 32 * D_HIDDEN/32 = {need_scale}")
     if w1_u8.numel() < int(NE) * 2 * int(D_INTER) * (int(D_HIDDEN) // 2) or w1_scale_u8.numel() < int(NE) * 2 * int(D_INTER) * (int(D_HIDDEN) // 32):
         raise ValueError("w1_u8 / w1_scale_u8 are smaller than NE * 2*D_INTER rows of D_HIDDEN/2 code bytes and D_HIDDEN/32 scale bytes")
     sorted_size = int(m_indices.numel())

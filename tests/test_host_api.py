@@ -163,6 +163,64 @@ def test_moe_c_abi_validation_codes():
     assert handle.psg_moe_reduce(0x1008, 0x1000, 4, 2, 8, 2, None) == -6  # fp32 rows are moved 16 bytes at a time
 
 
+def test_sorter_refuses_more_slots_than_experts():
+    """tokens*topk + experts*block_m - topk rows only bound the padded total while a token cannot repeat an expert: experts=2,
+    topk=4, block_m=2 with ids [0, 0, 0, 1] pads to 6 rows against a bound of 4."""
+    handle = _lib.lib()
+    a = _lib.MoeSortArgs()
+    for f in ("topk_ids", "topk_weights", "sorted_ids", "sorted_weights", "sorted_expert_ids", "num_valid_ids"):
+        setattr(a, f, 0x1000)
+    a.tokens, a.topk, a.experts, a.block_m, a.sorted_size, a.blocks = 1, 4, 2, 2, 4, 2
+    assert handle.psg_moe_sorting(ctypes.byref(a), None) == -2
+    assert b"topk=4 exceeds experts=2" in handle.psg_last_error()
+
+
+def test_sorter_workspace_comes_from_the_pool_of_the_launch_stream(monkeypatch):
+    """A workspace the caller does not bring must outlive the queued launches on whatever stream they run: it is taken from the
+    never-released pool keyed by (device, stream), not from the caching allocator, and is refused during graph capture."""
+    from flydsl_amd.kernels.moe import moe_sorting as S
+
+    class Fake:
+        def __init__(self, numel, dtype, esize=4):
+            self._n, self.dtype, self._e, self.is_cuda, self.device = numel, dtype, esize, True, "cuda:0"
+
+        def numel(self):
+            return self._n
+
+        def element_size(self):
+            return self._e
+
+        def is_contiguous(self):
+            return True
+
+        def data_ptr(self):
+            return 0x10000
+
+    made = []
+    capturing = [False]
+    pool = _lib.WorkspacePool(alloc=lambda n, dev: made.append(Fake(n, torch.uint8, 1)) or made[-1], capturing=lambda: capturing[0])
+    monkeypatch.setattr(_lib, "_pool", pool)
+    monkeypatch.setattr(_lib, "workspace", lambda device, nbytes, stream=0, owner="shared": pool.get(owner, 0, int(stream), int(nbytes)))
+    tokens, topk, E, B = 5000, 8, 64, 32
+    want = S.moe_sorting_get_workspace_size(tokens, E, topk, B)
+    assert want > 0
+    rows, blocks = S.sorted_sizes(tokens, topk, E, B)
+    outs = (Fake(rows, torch.int32), Fake(rows, torch.float32), Fake(blocks, torch.int32), Fake(2, torch.int32))
+    routing = (Fake(tokens * topk, torch.int32), Fake(tokens * topk, torch.float32))
+    args, ws = S._sort_args(tokens, topk, *outs, None, E, B, None, None, "cuda:0", routing=routing, stream_h=0x77)
+    assert ws is made[0] and ws.numel() >= want and args.workspace_bytes == ws.numel()
+    assert pool._live[("moe_sort", 0, 0x77)] is ws  # parked under the launch stream, never dropped
+    _, ws2 = S._sort_args(tokens, topk, *outs, None, E, B, None, None, "cuda:0", routing=routing, stream_h=0x77)
+    assert ws2 is ws and len(made) == 1
+    _, ws3 = S._sort_args(tokens, topk, *outs, None, E, B, None, None, "cuda:0", routing=routing, stream_h=0x88)
+    assert ws3 is not ws  # another stream never shares
+    capturing[0] = True
+    pool2 = _lib.WorkspacePool(alloc=lambda n, dev: made.append(Fake(n, torch.uint8, 1)) or made[-1], capturing=lambda: True)
+    monkeypatch.setattr(_lib, "workspace", lambda device, nbytes, stream=0, owner="shared": pool2.get(owner, 0, int(stream), int(nbytes)))
+    with pytest.raises(RuntimeError, match="graph capture"):
+        S._sort_args(tokens, topk, *outs, None, E, B, None, None, "cuda:0", routing=routing, stream_h=0x99)
+
+
 def test_mx_quantisers_match_the_oracle_byte_for_byte():
     from flydsl_amd import quant
     from oracle import psg_oracle as O
