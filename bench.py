@@ -249,7 +249,7 @@ def run_quant_workload(name, steps=50, warmup=5):
     return {"workload": name, "dtype": kind, "M": M, "K": K, "gb_per_s": achieved, "us_per_launch_events": sec * 1e6,
             "operand_sets": n_sets, "graph_replays_per_timing": replays, "parity_ok": ok, "timing": "graph replay, caller-owned outputs, HIP events",
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK["hbm"], "unit": "GB/s", "frac": achieved / PEAK["hbm"],
-                         "traffic": None, "algorithmic_bytes": nbytes}}
+                         "traffic": load_traffic(name), "algorithmic_bytes": nbytes}}
 
 
 def run_next_row_workloads(only=None):
@@ -472,31 +472,7 @@ def run_reference_test_shapes():
     dev = torch.device("cuda:0")
     out = []
 
-    def graph_time(launch, sets, steps=20):
-        for i in range(3):
-            launch(sets[i % len(sets)])
-        torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=side):
-            for i in range(steps):
-                launch(sets[i % len(sets)])
-        torch.cuda.synchronize()
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        replays = max(1, math.ceil(MIN_TIMED_S / max(e0.elapsed_time(e1) * 1e-3, 1e-7)))
-        e0.record()
-        for _ in range(replays):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / (steps * replays)
+    graph_time = _graph_time
 
     def tile(t, rows, unit):  # rows of a host tensor repeated to `rows` (weights of the large shapes are built from a slab)
         return t.repeat((rows + unit - 1) // unit, *([1] * (t.dim() - 1)))[:rows].contiguous()
@@ -539,6 +515,121 @@ def run_reference_test_shapes():
         del sets
         torch.cuda.empty_cache()
     return out
+
+
+# the reference's own benchmark list for this path (scripts/run_benchmark.sh:120-142, GEMM_SHAPES): dtype, M, N, K
+REFERENCE_BENCHMARK_SHAPES = [("fp8", 16, 40960, 5120), ("fp8", 16, 77824, 5120), ("fp8", 256, 2112, 7168), ("fp8", 512, 2112, 7168),
+                              ("fp8", 5120, 5120, 8320), ("fp8", 9728, 8192, 8320), ("fp8", 8192, 8192, 8192),
+                              ("int8", 9728, 8192, 8320), ("bf16", 5120, 5120, 8320)]
+
+
+def run_reference_benchmark_shapes():
+    """The nine shapes the reference benchmarks this path on (its results are not recorded anywhere), through the automatic
+    dispatcher, each with the roofline that bounds it: HBM when the algorithmic flops per byte lie below peak flops / peak
+    bytes, MFMA otherwise.  Same timing as the main workloads: 20 launches per HIP graph over rotating operand sets (more
+    than twice the Infinity Cache per pass), replayed until 50 ms are timed."""
+    import torch
+
+    from flydsl_amd.synthetic import make_a8w8, make_a16w16
+
+    dev = torch.device("cuda:0")
+    out = []
+
+    def tile(t, rows, unit):
+        return t.repeat((rows + unit - 1) // unit, *([1] * (t.dim() - 1)))[:rows].contiguous()
+
+    for kind, M, N, K in REFERENCE_BENCHMARK_SHAPES:
+        family = "a16w16" if kind == "bf16" else "a8w8"
+        mh, nh = min(M, 512), min(N, 512)
+        host = make_a16w16(mh, nh, K, kind, seed=0, w_std=0.02) if kind == "bf16" else make_a8w8(mh, nh, K, kind, seed=0)
+        nbytes = algorithmic_bytes(family, M, N, K)
+        flops = 2.0 * M * N * K
+        n_sets = max(2, min(16, math.ceil(2 * MALL_BYTES / nbytes)))
+        none = torch.empty(0, dtype=torch.float32, device=dev)
+        sets = [{"a": tile(host["a_q"], M, mh).to(dev), "b": tile(host["b_shuf"].view(nh, -1), N, nh).to(dev),
+                 "sa": none if kind == "bf16" else tile(host["sa"].view(-1), M, mh).to(dev),
+                 "sb": none if kind == "bf16" else tile(host["sb"].view(-1), N, nh).to(dev),
+                 "c": torch.zeros(M, N, dtype=torch.bfloat16, device=dev)} for _ in range(n_sets)]
+        sec = _graph_time(make_launcher(family, kind, M, N, K), sets)
+        bound = "hbm" if flops / nbytes < PEAK[kind] * 1e12 / (PEAK["hbm"] * 1e9) else "mfma"
+        achieved = nbytes / sec / 1e9 if bound == "hbm" else flops / sec / 1e12
+        peak = PEAK["hbm"] if bound == "hbm" else PEAK[kind]
+        out.append({"workload": f"{kind}_m{M}_n{N}_k{K}", "us_per_launch_events": sec * 1e6, "tflops": flops / sec / 1e12,
+                    "gb_per_s": nbytes / sec / 1e9, "operand_sets": n_sets,
+                    "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+                                 "frac": achieved / peak, "algorithmic_bytes": nbytes, "flops": flops}})
+        del sets
+        torch.cuda.empty_cache()
+    return out
+
+
+def _graph_time(launch, sets, steps=20):
+    """Seconds per launch: `steps` launches recorded into one HIP graph over rotating operand sets, replayed until
+    MIN_TIMED_S of work is timed with events on the launch stream."""
+    import torch
+
+    for i in range(3):
+        launch(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        for i in range(steps):
+            launch(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    replays = max(1, math.ceil(MIN_TIMED_S / max(e0.elapsed_time(e1) * 1e-3, 1e-7)))
+    best = float("inf")
+    for _ in range(2):
+        e0.record()
+        for _r in range(replays):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e-3 / (steps * replays))
+    return best
+
+
+def host_cost_per_call(name="fp8_decode_m16", calls=2000):
+    """Host time of one eager launch (no graph): wall clock of a loop of `calls` launches on one stream divided by the
+    calls, for the launcher's default path (operands validated once, then looked up) and for the path that validates every
+    call.  The GPU work of the loop is far shorter than the loop, so this is the cost of getting a launch into the queue."""
+    import torch
+
+    from flydsl_amd.synthetic import make_a8w8
+    from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
+
+    family, kind, M, N, K, _ = WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    host = make_a8w8(M, N, K, kind, seed=0)
+    a, b, sa, sb = host["a_q"].to(dev), host["b_shuf"].to(dev), host["sa"].to(dev), host["sb"].to(dev)
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    bias = torch.empty(0, dtype=torch.bfloat16, device=dev)
+    fn = compile_preshuffle_gemm(N=N, K=K, tile_m=128, tile_n=256, tile_k=64, in_dtype=kind)
+    stream = torch.cuda.current_stream()
+    out = {}
+    for label, call in (("fast_path", fn), ("checked_path", fn.launch_checked)):
+        for _ in range(50):
+            call(c, a, b, sa, sb, bias, M, N, stream)
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _i in range(calls):
+                call(c, a, b, sa, sb, bias, M, N, stream)
+            dt = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            best = min(best, dt / calls)
+        out[label] = best * 1e6
+    return {"workload": name, "calls": calls, "fast_path": out["fast_path"], "checked_path": out["checked_path"],
+            "unit": "us per call, host wall clock of an eager launch loop"}
 
 
 def cpu_baseline(name, host, budget_s=12.0):  # budget_s bounds the CPU work of one workload
@@ -601,11 +692,15 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--reference-shapes", action="store_true",
-                    help="also time the shapes of the reference's own tests for this path; adds a reference_test_shapes list")
+                    help="also time the reference's own benchmark list (scripts/run_benchmark.sh) and the shapes of its tests for "
+                         "this path; adds reference_benchmark_shapes and reference_test_shapes lists")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the general MX kernel and the MoE stages (rows next to the hot path); adds a next_rows list")
     ap.add_argument("--next-rows-only", default=None, choices=("mx", "moe_fp8", "moe_mxfp4", "moe_sorting", "moe_gating"),
                     help="with --next-rows: run one section of them only (for profiler runs)")
+    ap.add_argument("--quant-only", default=None, choices=("quant_pertoken_fp8_m8192", "quant_mxfp4_m4096"),
+                    help="only run one of the on-device quantiser workloads (for profiler runs)")
+    ap.add_argument("--host-cost", action="store_true", help="measure host_us_per_call even with --no-others")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy a few times (the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against)")
@@ -631,6 +726,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": 5}))
+        return
+
+    if args.quant_only:
+        print(json.dumps(run_quant_workload(args.quant_only)))
         return
 
     family, kind, M, N, K, bound = WORKLOADS[args.workload]
@@ -660,6 +759,8 @@ def main():
             others.append(run_quant_workload(name))
     next_rows = run_next_row_workloads(args.next_rows_only) if args.next_rows else None
     ref_shapes = run_reference_test_shapes() if args.reference_shapes else None
+    ref_bench = run_reference_benchmark_shapes() if args.reference_shapes else None
+    host_cost = host_cost_per_call() if not args.no_others or args.host_cost else None
 
     line = {
         "metric": "TFLOPS + % roofline (HBM GB/s at M=16, MFMA util at M=8192), 1 MI355X",
@@ -693,6 +794,10 @@ def main():
         line["next_rows"] = next_rows
     if ref_shapes is not None:
         line["reference_test_shapes"] = ref_shapes
+    if ref_bench is not None:
+        line["reference_benchmark_shapes"] = ref_bench
+    if host_cost is not None:
+        line["host_us_per_call"] = host_cost
     # the metric names two operating points; the second one (MFMA-bound prefill) is lifted out of the table for convenience
     for r in others:
         if r["workload"] == "fp8_prefill_m8192":

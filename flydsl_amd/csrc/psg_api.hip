@@ -40,6 +40,20 @@ hipError_t psg_launch_quant_mxfp4(const void* x, int x_dtype, void* packed, void
 #define PSG_STATIC_SCRATCH_BYTES (32u << 20)
 static __device__ __align__(256) unsigned char scratch[PSG_STATIC_SCRATCH_BYTES];
 
+// Compute units of the current device, read once (the planners deal workgroups out per CU).  Without a device (host-only use of
+// the planning entry points) the MI355X's 256.
+int psg_cu_count() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        return cus;
+    }();
+    return n;
+}
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -396,20 +410,6 @@ uint64_t psg_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t in_dtype) 
 int psg_gemm_a8w8(const psg_a8w8_args* args, void* stream) {
     if (int rc = validate_a8w8(args, false, nullptr)) return rc;
     return run_a8w8(args, args->c, STORE_C, stream);
-}
-
-// Compute units of the current device, read once (the planners deal workgroups out per CU).  Without a device (host-only use of
-// the planning entry points) the MI355X's 256.
-int psg_cu_count() {
-    static const int n = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
-            (void)hipGetLastError();
-            cus = 256;
-        }
-        return cus;
-    }();
-    return n;
 }
 
 int psg_init(void) {
