@@ -12,11 +12,13 @@
 //     blocks of both windows) is issued before anything waits.  Chunks are NOT prefetched across: with all 256 CUs
 //     streaming, more than about 100 KB of requests per CU only deepens the queues of the memory system (measured:
 //     keeping two chunks in flight per wavefront is 4 % slower than one), so the chunk size sets the depth.
-//   * A (at most 32 rows, L2 resident after first touch) is needed in fragment order (16 different rows per load
-//     instruction, which costs the texture addresser more than the whole W stream), so each wavefront reads its K
-//     slice of A with row-contiguous loads into a private LDS patch (XOR-swizzled 16-byte chunks, no barrier) and
-//     picks the fragments up from there.  A is loaded before W in every chunk: loads return in order and A comes
-//     from L2.
+//   * A (at most 64 rows, L2 resident after first touch) is needed in fragment order (16 different rows per load
+//     instruction, which costs the texture addresser more than the whole W stream), so each wavefront brings its K
+//     slice of A row-contiguously into a private LDS patch (XOR-swizzled 16-byte chunks, no barrier) and picks the
+//     fragments up from there.  The rows travel global -> LDS by DMA (buffer_load_dwordx4 ... lds: 64 lanes x 16 bytes to
+//     consecutive LDS addresses, so the swizzle is applied to the source address of each lane): no staging registers, no
+//     ds_write.  A is requested before W in every chunk: loads return in order and A comes from L2, so one
+//     s_waitcnt vmcnt(number of W loads) is the wait for A.
 // Operands are swapped like in the tiled kernel (src0 = W fragment, src1 = A fragment): a lane holds
 // C[m = lane%16][n = window + (lane/16)*4 + 0..3].
 #include "psg_common.h"
@@ -34,19 +36,36 @@ struct Acc<KIND_INT8> {
     using type = v4i;
 };
 
+// descriptor built from values forced into scalar registers (an inline-asm "s" operand must not end up in vector registers)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_uniform(const void* base, uint64_t bytes) {
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint32_t n = (uint32_t)__builtin_amdgcn_readfirstlane((int)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>((uintptr_t)(((uint64_t)hi << 32) | lo)), 0, (int)n, 0x00020000);
+}
+
+// one DMA instruction: 64 lanes x 16 bytes from (descriptor, voff) to LDS [lds_addr, lds_addr + 1024).  Issued from inline
+// assembly: the compiler does not know that it writes LDS (it would put a full vmcnt wait in front of every LDS read that
+// follows), so the kernel waits for it itself.
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voff), "s"(r)
+                 : "memory");
+}
+
 // MB = 16-row blocks of A (1 to 4); NWIN = 16-column windows per wavefront group (1 or 2).
 // CH = 128-byte K steps per chunk; NWAVES = wavefronts per workgroup.
-// DIAG is 0 in the library.  The hardware-ceilings probe instantiates the kernel with parts switched off to price them
-// (results are then wrong on purpose): bit 0 = A loads redirected past the buffer bound, bit 1 = wavefronts end after
-// their MFMAs (no reduction, no store), bit 2 = reduction kept but nothing stored.
-template <int KIND, int MB, int NWIN, int NWAVES, int CH, int STORE, int DIAG = 0>
+template <int KIND, int MB, int NWIN, int NWAVES, int CH, int STORE>
 __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
     constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
     constexpr int ROWS = 16 * MB;
     constexpr int CPR = CH * 8;                 // 16-byte chunks per staged row (256 bytes)
-    constexpr int PASSES = ROWS * CPR / 64;     // staging loads per lane per chunk
+    constexpr int PASSES = ROWS * CPR / 64;     // staging loads (or DMA instructions) per chunk, 1 KB of the patch each
     constexpr int RPP = 64 / CPR;               // rows per staging pass
+    // A by DMA from two 16-row blocks on: fp8 N=6144 K=4096, us per launch, registers + ds_write against DMA: M=32 8.50 / 8.28,
+    // M=16 6.67 / 6.84, M=1 6.33 / 6.46 (one block moves too little for the DMA's extra wait and issue cost to pay)
+    constexpr bool ADMA = MB >= 2;
     __shared__ __attribute__((aligned(16))) v4i patch[NWAVES][ROWS * CPR];
     // the partial sums of the split-K reduction reuse the wavefront's own patch (it is done with it by then): with 64 rows
     // patch and a separate array would not fit the LDS together
@@ -120,8 +139,9 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
 
     if (nchunks > 0 && n_end > n_begin) {
         __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, (uint64_t)p.N * (uint64_t)K);
-        __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a, (uint64_t)p.M * (uint64_t)K);
+        __amdgpu_buffer_rsrc_t ra = ADMA ? make_rsrc_uniform(p.a, (uint64_t)p.M * (uint64_t)K) : make_rsrc(p.a, (uint64_t)p.M * (uint64_t)K);
         v4i* my_patch = patch[wave];
+        const uint32_t patch_lds = (uint32_t)(uintptr_t)my_patch;
         // per-window W offset of this lane: row n of the window, 16-byte K group lg of a 1 KB block
         uint32_t wvoff[NWIN];
 #pragma unroll
@@ -133,19 +153,43 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
             wvoff[w] = n < n_end ? off : OOB;
         }
         const uint32_t w_step = p.b_rowmajor ? 128u : 2048u, w_half = p.b_rowmajor ? 64u : 1024u;
-        const int st_c = lane % CPR;
-        const int st_r0 = lane / CPR;
+        // DMA instruction ps fills patch chunks [64 ps, 64 ps + 64): lane l writes physical chunk (64 ps + l) % CPR of row
+        // (64 ps + l) / CPR and therefore fetches that row's logical chunk physical ^ (row & 15).  (row & 15) repeats every
+        // 16 / RPP instructions, so a lane needs that many source offsets; the others follow by adding whole rows.
+        constexpr int NVAR = 16 / RPP < PASSES ? 16 / RPP : PASSES;
+        uint32_t a_src[NVAR];
+#pragma unroll
+        for (int v = 0; v < NVAR; v++) {
+            const int r = v * RPP + lane / CPR;
+            a_src[v] = (uint32_t)r * (uint32_t)K + (uint32_t)(((lane % CPR) ^ (r & 15)) << 4);
+        }
         const uint32_t slice_end = (uint32_t)(s_end * 128 < K ? s_end * 128 : K);
 
         // chunk c of this wavefront's K slice: A rows first (they come from L2 and must not queue behind W), then W
-        auto load_chunk = [&](int c, v4i (&at)[PASSES], v4i (&wlo)[NWIN][CH], v4i (&whi)[NWIN][CH]) {
+        const int st_c = lane % CPR;
+        const int st_r0 = lane / CPR;
+        constexpr int NAT = ADMA ? 1 : PASSES;
+        auto load_chunk = [&](int c, v4i (&at)[NAT], v4i (&wlo)[NWIN][CH], v4i (&whi)[NWIN][CH]) __attribute__((always_inline)) {
             const int s0 = s_begin + c * CH;
-            const uint32_t kbyte = (uint32_t)s0 * 128u + (uint32_t)st_c * 16u;
-            const bool a_ok = !(DIAG & 1) && c < nchunks && kbyte < slice_end;
+            const uint32_t kbyte0 = (uint32_t)s0 * 128u;
+            if constexpr (ADMA) {
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ps++) {
-                const int r = st_r0 + ps * RPP;
-                at[ps] = buf_load16(ra, a_ok ? (uint32_t)r * (uint32_t)K + kbyte : OOB, 0);
+                for (int ps = 0; ps < PASSES; ps++) {
+                    const uint32_t src = a_src[ps % NVAR] + (uint32_t)((ps / NVAR) * 16) * (uint32_t)K;
+                    // rows >= M lie behind the descriptor's bound; a chunk past the K slice (or a chunk that does not exist) is
+                    // redirected there too: both write zeros
+                    const uint32_t kb = kbyte0 + ((((uint32_t)(lane % CPR)) ^ (uint32_t)(((ps % NVAR) * RPP + lane / CPR) & 15)) << 4);
+                    const bool a_ok = c < nchunks && kb < slice_end;
+                    dma16(ra, patch_lds + (uint32_t)ps * 1024u, a_ok ? src + kbyte0 : OOB);
+                }
+            } else {
+                const uint32_t kbyte = kbyte0 + (uint32_t)st_c * 16u;
+                const bool a_ok = c < nchunks && kbyte < slice_end;
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ps++) {
+                    const int r = st_r0 + ps * RPP;
+                    at[ps] = buf_load16(ra, a_ok ? (uint32_t)r * (uint32_t)K + kbyte : OOB, 0);
+                }
             }
 #pragma unroll
             for (int w = 0; w < NWIN; w++)
@@ -161,11 +205,18 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
             __builtin_amdgcn_sched_barrier(0);
         };
         // A through the private patch into fragment order, then the chunk's MFMAs as W arrives
-        auto compute_chunk = [&](const v4i (&at)[PASSES], const v4i (&wlo)[NWIN][CH], const v4i (&whi)[NWIN][CH]) {
+        auto compute_chunk = [&](const v4i (&at)[NAT], const v4i (&wlo)[NWIN][CH], const v4i (&whi)[NWIN][CH], auto FIRST) __attribute__((always_inline)) {
+            if constexpr (ADMA) {
+                // the chunk's A has landed once only what was requested behind its DMAs is still on its way: its W loads
+                // and, for the first chunk, the epilogue scales
+                constexpr int BEHIND = NWIN * CH * 2 + (decltype(FIRST)::value && STORE != STORE_ACC && !IS16 ? 2 * FIN : 0);
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(BEHIND) : "memory");
+            } else {
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ps++) {
-                const int r = st_r0 + ps * RPP;
-                my_patch[r * CPR + (st_c ^ (r & 15))] = at[ps];
+                for (int ps = 0; ps < PASSES; ps++) {
+                    const int r = st_r0 + ps * RPP;
+                    my_patch[r * CPR + (st_c ^ (r & 15))] = at[ps];
+                }
             }
             // one K step's MFMAs on fragments alo / ahi (per 16-row block) and W registers wlo / whi (per window) of step t
             auto mfma_step = [&](int t, const v4i (&alo_t)[MB], const v4i (&ahi_t)[MB], int w) {
@@ -223,28 +274,29 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
             }
         };
 
-        v4i at[PASSES];
+        v4i at[NAT];
         v4i wlo[NWIN][CH], whi[NWIN][CH];
         load_chunk(0, at, wlo, whi);
         fetch_scales();
         __builtin_amdgcn_sched_barrier(0);
-        for (int c = 0; c < nchunks; c++) {
-            compute_chunk(at, wlo, whi);
-            if (c + 1 < nchunks) load_chunk(c + 1, at, wlo, whi);
+        if constexpr (ADMA) {
+            // the first chunk apart: its wait for A counts the scale loads too
+            compute_chunk(at, wlo, whi, std::true_type{});
+            if (1 < nchunks) load_chunk(1, at, wlo, whi);
+            for (int c = 1; c < nchunks; c++) {
+                compute_chunk(at, wlo, whi, std::false_type{});
+                if (c + 1 < nchunks) load_chunk(c + 1, at, wlo, whi);
+            }
+        } else {
+            for (int c = 0; c < nchunks; c++) {
+                compute_chunk(at, wlo, whi, std::false_type{});
+                if (c + 1 < nchunks) load_chunk(c + 1, at, wlo, whi);
+            }
         }
     } else {
         fetch_scales();  // wavefronts without work still finish outputs
     }
 
-    if constexpr ((DIAG & 2) != 0) {  // keep the MFMAs alive without a reduction or a store
-        float t = 0.f;
-#pragma unroll
-        for (int w = 0; w < NWIN; w++)
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) t += (float)acc[w][mb][0] + (float)acc[w][mb][1] + (float)acc[w][mb][2] + (float)acc[w][mb][3];
-        if (t == 12345.678f) reinterpret_cast<float*>(p.c)[0] = t;
-        return;
-    }
     // split-K reduction through LDS, fixed order
 #pragma unroll
     for (int w = 0; w < NWIN; w++)
@@ -279,11 +331,7 @@ __global__ void __launch_bounds__(NWAVES * 64) k_a8w8_stream(A8W8Params p) {
                     x = (v4f){((float)sum[0] * sa) * sb[0], ((float)sum[1] * sa) * sb[1], ((float)sum[2] * sa) * sb[2],
                               ((float)sum[3] * sa) * sb[3]};
                 }
-                if constexpr ((DIAG & 4) != 0) {
-                    if (x[0] == 12345.678f) store_c4(p, idx, n, x);
-                } else {
-                    store_c4(p, idx, n, x);
-                }
+                store_c4(p, idx, n, x);
             }
         }
     }
