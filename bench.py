@@ -628,7 +628,21 @@ def host_cost_per_call(name="fp8_decode_m16", calls=2000):
             torch.cuda.synchronize()
             best = min(best, dt / calls)
         out[label] = best * 1e6
+    # what both paths share: the C ABI call itself (ctypes + the library's checks + hipLaunchKernel) on a filled struct
+    ref, handle = next(iter(fn._fast.values()))[:2]
+    gemm = fn._gemm
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _i in range(calls):
+            gemm(ref, handle)
+        dt = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        best = min(best, dt / calls)
+    c_call = best * 1e6
     return {"workload": name, "calls": calls, "fast_path": out["fast_path"], "checked_path": out["checked_path"],
+            "c_abi_call_alone": c_call, "launcher_overhead_fast": out["fast_path"] - c_call,
+            "launcher_overhead_checked": out["checked_path"] - c_call,
             "unit": "us per call, host wall clock of an eager launch loop"}
 
 
