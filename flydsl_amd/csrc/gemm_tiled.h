@@ -489,8 +489,10 @@ hipError_t launch_one(const A8W8Params& p, hipStream_t stream) {
 }
 
 // the 256x256 tile of eight wavefronts has a kernel of its own (gemm_tiled8.h, which includes this file)
-template <int KIND, int STORE, int OPT>
+template <int KIND, int STORE>
 hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream);
+template <int KIND, int STORE>
+hipError_t launch_tiled_deep(const A8W8Params& p, hipStream_t stream);
 
 // p.wave_layout selects the wavefront layout of the 256x256 tile: 2 = 2x2 wavefronts, 8 = eight wavefronts along N, anything
 // else = 1x4
@@ -502,12 +504,18 @@ hipError_t launch_shape(const A8W8Params& p, int tile_m, int tile_n, hipStream_t
         PSG_CASE(8, 8, 2)
     }
     if (p.wave_layout == 8) {  // eight wavefronts side by side along N: 256x256 tile, every W fragment loaded once
-        if (tile_m == 256 && tile_n == 256) return launch_tiled8<KIND, STORE, 0>(p, stream);
+        if (tile_m == 256 && tile_n == 256) return launch_tiled8<KIND, STORE>(p, stream);
     }
     if constexpr (KIND != KIND_MXFP4 && KIND != KIND_MXFP8) {
         // few tiles (p.ksplit = 3: the planner's mark for launches of at most two workgroups per CU): W fetched three steps ahead
         if (p.ksplit == 3) {
-            if (tile_m == 128 && tile_n == 128) return launch_one<KIND, 8, 2, 1, STORE, 4, 1, 3>(p, stream);
+            // 128x128 with a deep ring of stages (gemm_tiled8.h); wave_layout 4 keeps the older build with W three steps ahead
+            if (tile_m == 128 && tile_n == 128) {
+                // one workgroup per CU at most (its LDS ring fills the CU), and only above 256 rows (measured: no gain below);
+                // everything else keeps the register-ring build
+                const long wgs = (long)((p.M + 127) / 128) * (long)((p.N + 127) / 128) * (STORE == STORE_ACC && p.splits > 1 ? p.splits : 1);
+                return p.wave_layout == 4 || wgs > psg_cu_count() || p.M <= 256 ? launch_one<KIND, 8, 2, 1, STORE, 4, 1, 3>(p, stream) : launch_tiled_deep<KIND, STORE>(p, stream);
+            }
             if (tile_m == 64 && tile_n == 64) return launch_one<KIND, 4, 1, 1, STORE, 4, 0, 3>(p, stream);
         }
     }

@@ -1,4 +1,6 @@
-// 256x256 tile of the compute-bound mainloop, eight wavefronts side by side along N (gfx950).
+// Tiles of the compute-bound mainloop whose A operand travels global -> LDS by DMA (gfx950): the 256x256 tile of eight
+// wavefronts side by side along N, and a 128x128 tile of four wavefronts with a deep ring of stages for launches with few
+// tiles and a long K.
 //
 // Same operand paths as gemm_tiled.h (W fragments straight from memory into MFMA operand registers, every fragment read
 // from memory once per workgroup; the A tile shared through LDS and read by all eight wavefronts), with a different way
@@ -8,9 +10,9 @@
 //     swizzle of the 16-byte chunks is applied to the SOURCE address of each lane (lane l of a 1 KB block fills physical
 //     chunk l%8 of row l/8 and therefore fetches logical chunk (l%8) ^ ((row/2)%8) of that row).  Lanes redirected past
 //     the descriptor bound (rows >= M, K tail, steps past the end) write zeros.
-//   * Four LDS stages of 32 KB: the A tile of step kt+3 is requested during step kt, is waited for (vmcnt, by the
-//     wavefront that requested it) before the barrier that ends step kt+1, and is therefore complete for everybody one
-//     whole step before its MFMAs.  That lets every wavefront read the first A fragments of step kt+1 BEFORE the barrier
+//   * NS LDS stages (four of 32 KB for the 256-row tile): the A tile of step kt+NS-1 is requested during step kt, is waited
+//     for (vmcnt, by the wavefront that requested it) before the barrier that ends step kt+NS-3, and is therefore complete
+//     for everybody one whole step before its MFMAs.  That lets every wavefront read the first A fragments of step kt+1 BEFORE the barrier
 //     that ends step kt, so the MFMAs continue right behind the barrier instead of waiting for LDS.  The one barrier per
 //     step that is left only keeps a stage from being overwritten while a slower wavefront still reads it.
 //   * The DMA is issued from inline assembly: the compiler does not know that it writes LDS (it would otherwise put a
@@ -32,9 +34,6 @@
 
 namespace {
 
-constexpr int T8_STAGE = 256 * TK;  // bytes of one A stage (256 rows x 128 bytes)
-constexpr int T8_NS = 4;            // LDS stages
-
 // descriptor built from values forced into scalar registers (an inline-asm "s" operand must not end up in vector registers)
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_uniform(const void* base, uint64_t bytes) {
     const uint64_t b = (uint64_t)(uintptr_t)base;
@@ -50,6 +49,12 @@ __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, uint32_t lds_add
                  : "memory");
 }
 
+// 4 bytes per lane: 64 lanes x 4 bytes to LDS [lds_addr, lds_addr + 256)
+__device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voff), "s"(r), "s"(__builtin_amdgcn_readfirstlane((int)soff))
+                 : "memory");
+}
+
 // Built with -DT8_TIMING (a measuring harness, never the library) thread 0 of every workgroup records the core clock and the
 // 10 ns wall clock at: 0 start, 1 loop begin, 2 loop end, 4 C staged, 5 behind the barrier, 6 stores issued, 3 stores done.
 #ifdef T8_TIMING
@@ -59,35 +64,38 @@ __device__ unsigned long long* t8_dbg;
 #define T8_STAMP(i) do { } while (0)
 #endif
 
-// 4 bytes per lane: 64 lanes x 4 bytes to LDS [lds_addr, lds_addr + 256)
-__device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voff), "s"(r), "s"(__builtin_amdgcn_readfirstlane((int)soff))
-                 : "memory");
-}
-
-// OPT (0 in the library; the other builds exist to be measured against it): bit 0 staggers the memory instructions of the two
-// wavefronts that share a SIMD (w and w + 4) by two m-blocks, bit 1 raises the wave priority around the MFMAs.  fp8
-// 8192x4096x4096, core cycles per K step / us per launch: plain 2,311 / 114.5, staggered 2,354 / 115.5, staggered with
-// priority 2,425 / 115.4 (2,048 cycles is the issue limit of the 64 MFMAs per SIMD).  W fragments are fetched one K step
-// ahead (two register sets): three steps ahead (four sets) measured the same and leaves the allocator no room.
-constexpr int T8_STAGGER = 1, T8_SETPRIO = 2;
-template <int KIND, int STORE, int OPT = 0>
-__global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
-    constexpr int PFW = 1;
+// Tile = (16 MR) x (32 WAVES) x 128 bytes of K: WAVES wavefronts side by side along N with two 16-column blocks each, every
+// one of them multiplying all MR 16-row blocks of the A tile.  NS = LDS stages of the A tile, PFW = K steps the W fragments
+// are fetched ahead of their MFMAs (PFW + 1 register sets; NS must be a multiple of that).
+//   <16, 8, 4, 1>: 256x256, one workgroup per CU with two wavefronts per SIMD; for problems that fill the GPU.  (Measured on it
+//       and not kept, fp8 8192x4096x4096, core cycles per K step / us per launch: the memory instructions of the two
+//       wavefronts of a SIMD two m-blocks apart 2,354 / 115.5 and the same with s_setprio 1 around the MFMAs 2,425 / 115.4,
+//       against 2,311 / 114.5 as built; 2,048 cycles is the issue limit of the 64 MFMAs per SIMD.  W three steps ahead, four
+//       register sets: the same time, and no room left for the allocator.)
+//   <8, 4, 8, 7>: 128x128, one wavefront per SIMD, seven steps of A (DMA) and W (registers) on their way: for launches with
+//       few tiles and a long K.  Against the build that keeps W three steps ahead in registers (fp8, N = K = 8192, split-K
+//       pair, us): M=512 42.9 / 45.4, M=384 (5120x13824) 44.1 / 45.8, M=256 35.2 / 34.9, M=128 27.8 / 26.6, so the launcher takes
+//       it above 256 rows only: more bytes in flight per CU is not what these launches lack.
+template <int KIND, int STORE, int MR, int WAVES, int NS, int PFW>
+__global__ void __launch_bounds__(WAVES * 64, 1) k_tiled_dma(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
-    constexpr int MR = 16, NR = 2, WAVES = 8;
-    constexpr int TM = 256, TN = 256;
+    constexpr int NR = 2;
+    constexpr int TM = 16 * MR, TN = 16 * NR * WAVES;
     constexpr int NB = PFW + 1;
+    constexpr int STAGE = TM * TK;                   // bytes of one A stage
+    constexpr int A_DMA = STAGE / 1024 / WAVES;      // 1 KB blocks of a stage this wavefront fills
+    static_assert(NS % NB == 0 && MR % 4 == 0 && A_DMA >= 1 && A_DMA % 2 == 0 && STAGE % (1024 * WAVES) == 0, "tile geometry");
     constexpr bool IS16 = KIND == KIND_FP16 || KIND == KIND_BF16;
     constexpr bool SCALED = KIND == KIND_INT8 || KIND == KIND_FP8;
     constexpr bool MX = KIND == KIND_MXFP4 || KIND == KIND_MXFP8;
+    static_assert(!MX || (MR == 16 && NS == 4), "MX scale slots are laid out for the 256-row tile");
 
-    // LDS: four A stages; behind them four slots of MX scale dwords (per slot 8 A-side chunks + 8 W-side chunks of 256 bytes)
-    // or the per-token / per-channel scales of the epilogue (256 + 256 floats)
+    // LDS: the A stages; behind them NS slots of MX scale dwords (per slot 8 A-side chunks + 8 W-side chunks of 256 bytes)
+    // or the per-token / per-channel scales of the epilogue (TM + TN floats)
     constexpr int SC_SLOT = 4096;
-    constexpr int LDS_EXTRA = MX ? T8_NS * SC_SLOT : 2048;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[T8_NS * T8_STAGE + LDS_EXTRA];
-    uint8_t* const lds_x = lds + T8_NS * T8_STAGE;
+    constexpr int LDS_EXTRA = MX ? NS * SC_SLOT : (TM + TN) * 4;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[NS * STAGE + LDS_EXTRA];
+    uint8_t* const lds_x = lds + NS * STAGE;
 
     T8_STAMP(0);
     const int tid = threadIdx.x;
@@ -137,13 +145,13 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
 
     v4i blo[NB][NR], bhi[NB][NR];
 
-    // A by DMA: this wavefront fills the four 1 KB blocks 4*wave + j (rows 8*(4*wave + j) .. + 7) of a stage
+    // A by DMA: this wavefront fills the 1 KB blocks A_DMA*wave + j (rows 8*(A_DMA*wave + j) .. + 7) of a stage
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-    uint32_t a_voff[4];
+    uint32_t a_voff[A_DMA];
     int a_kc[2];  // logical 16-byte chunk this lane fetches, by the parity of the block
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int row = (wave * 4 + j) * 8 + (lane >> 3);
+    for (int j = 0; j < A_DMA; j++) {
+        const int row = (wave * A_DMA + j) * 8 + (lane >> 3);
         const int kc = (lane & 7) ^ ((row >> 1) & 7);
         a_voff[j] = (uint32_t)row * (uint32_t)K + (uint32_t)kc * 16u;
         a_kc[j & 1] = kc;
@@ -151,7 +159,7 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     // CHK = false: the step is known to lie inside [kt_begin, kt_end) and not to be the K tail, so nothing is redirected (the
     // selects and compares of the checked form are ten instructions per load in front of the MFMAs of both wavefronts of a SIMD)
     auto dma_a1 = [&](int kt, int stage, int j, auto CHK) __attribute__((always_inline)) {
-        const uint32_t dst = lds_base + (uint32_t)(stage * T8_STAGE + (wave * 4 + j) * 1024);
+        const uint32_t dst = lds_base + (uint32_t)(stage * STAGE + (wave * A_DMA + j) * 1024);
         if constexpr (decltype(CHK)::value) {
             const bool in_k = kt < kt_end && (uint32_t)(kt * TK + a_kc[j & 1] * 16) < (uint32_t)K;
             dma16(ra, dst, in_k ? a_voff[j] : 0xFFFFFFF0u, kt < kt_end ? (uint32_t)kt * TK : 0u);
@@ -163,7 +171,7 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     // scale dwords of step kt -> slot (two DMAs per wavefront), and slot -> registers
     auto dma_sc = [&](int kt, int slot, int which) __attribute__((always_inline)) {
         const bool has = kt < kt_end;
-        const uint32_t dst = lds_base + (uint32_t)(T8_NS * T8_STAGE + slot * SC_SLOT + which * 2048 + wave * 256);
+        const uint32_t dst = lds_base + (uint32_t)(NS * STAGE + slot * SC_SLOT + which * 2048 + wave * 256);
         dma4(which ? rsb : rsa, dst, has ? (uint32_t)lane * 4u : 0xFFFFFFF0u, has ? (uint32_t)(KIND == KIND_MXFP8 ? (kt >> 1) : kt) * 256u : 0u);
     };
     auto read_sc = [&](int slot, int q, int* sa_dst, int* sb_dst) __attribute__((always_inline)) {
@@ -184,48 +192,50 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     const int f_lo = li * TK + ((lg ^ ((li >> 1) & 7)) << 4);
     const int f_hi = li * TK + (((4 + lg) ^ ((li >> 1) & 7)) << 4);
     auto read_frag = [&](int stage, int mi, v4i& flo, v4i& fhi) __attribute__((always_inline)) {
-        flo = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_lo]);
-        fhi = *reinterpret_cast<const v4i*>(&lds[stage * T8_STAGE + mi * 16 * TK + f_hi]);
+        flo = *reinterpret_cast<const v4i*>(&lds[stage * STAGE + mi * 16 * TK + f_lo]);
+        fhi = *reinterpret_cast<const v4i*>(&lds[stage * STAGE + mi * 16 * TK + f_hi]);
     };
 
-    constexpr int FRAG_AHEAD = 2, FRAG_BUFS = 4;  // 16 m-blocks per step: buffer mi % 4 lines up across steps
+    constexpr int FRAG_AHEAD = 2, FRAG_BUFS = 4;  // MR is a multiple of 4: buffer mi % 4 lines up across steps
     v4i flo[FRAG_BUFS], fhi[FRAG_BUFS];
 
-    // One K step: MFMAs on LDS stage S and W set SB.  m-block 0 only multiplies (the compiler waits for this step's W
-    // fragments there); from m-block 1 on one memory instruction per m-block: four DMAs of the A tile of step kt+3 (MX: and
-    // two of its scale chunks), then the four W loads of step kt+1; every m-block reads the A fragment two m-blocks ahead,
-    // the last two those of step kt+1.
-    // (always_inline: with 22 call sites the inliner would otherwise leave this lambda a function of its own, with the
+    // One K step: MFMAs on LDS stage S and W set S % NB.  m-block 0 only multiplies (the compiler waits for this step's W
+    // fragments there); the memory instructions follow from m-block 1 on, dealt out evenly: the DMAs of the A tile of step
+    // kt+NS-1 (MX: and two of its scale chunks), then the four W loads of step kt+PFW.  Every m-block reads the A fragment two
+    // m-blocks ahead, the last two those of step kt+1.
+    // (always_inline: with many call sites the inliner would otherwise leave this lambda a function of its own, with the
     // accumulators and descriptors passed through memory)
-    auto step = [&](int kt, auto SP, auto CHK, auto GRP) __attribute__((always_inline)) {
-        constexpr int S = decltype(SP)::value;   // LDS stage of this step (kt % 4)
+    constexpr int N_DMA = A_DMA + (MX ? 2 : 0);  // DMAs per wavefront per step
+    constexpr int N_W = 2 * NR;                  // W fragment loads per wavefront per step
+    constexpr int N_OPS = A_DMA + (MX ? 1 : 0) + N_W;          // slots: the two scale DMAs share one
+    constexpr int OPS_PER = (N_OPS + MR - 2) / (MR - 1);       // slots per m-block (m-blocks 1 .. MR-1)
+    auto step = [&](int kt, auto SP, auto CHK) __attribute__((always_inline)) {
+        constexpr int S = decltype(SP)::value;   // LDS stage of this step (kt % NS)
         constexpr int SB = S % NB;               // W register set of this step
         constexpr int SN = (SB + PFW) % NB;      // W register set the loads of this step fill
         constexpr int SS = S & 1;                // MX scale set of this step
-        constexpr int N_DMA = 4 + (MX ? 2 : 0);  // DMAs per wavefront per step: four 1 KB blocks of A (+ two chunks of MX scales)
-        constexpr int N_W = 2 * NR;              // W fragment loads per wavefront per step
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
             if constexpr (mi + FRAG_AHEAD < MR)
                 read_frag(S, mi + FRAG_AHEAD, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
             else
-                read_frag((S + 1) % T8_NS, mi + FRAG_AHEAD - MR, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
-            // memory instructions, one m-block each: the DMAs of step kt+3, then the W loads of step kt+1.  The first four
-            // wavefronts (one per SIMD) start at m-block 1, their SIMD partners two m-blocks later (GRP)
-            constexpr int OFF = decltype(GRP)::value ? 2 : 0;
-            constexpr int W0 = (MX ? 6 : 5) + OFF;
-            if constexpr (mi >= 1 + OFF && mi <= 4 + OFF) {
-                dma_a1(kt + 3, (S + 3) % T8_NS, mi - 1 - OFF, CHK);
-            } else if constexpr (MX && mi == 5 + OFF) {
-                dma_sc(kt + 3, (S + 3) % T8_NS, 0);
-                dma_sc(kt + 3, (S + 3) % T8_NS, 1);
-            } else if constexpr (mi >= W0 && mi < W0 + N_W) {
-                load_b1(kt + PFW, mi - W0, blo[SN], bhi[SN], CHK);
+                read_frag((S + 1) % NS, mi + FRAG_AHEAD - MR, flo[(mi + FRAG_AHEAD) % FRAG_BUFS], fhi[(mi + FRAG_AHEAD) % FRAG_BUFS]);
+            if constexpr (mi >= 1) {
+                static_for<OPS_PER>([&](auto Q) {
+                    constexpr int op = (mi - 1) * OPS_PER + decltype(Q)::value;
+                    if constexpr (op < A_DMA) {
+                        dma_a1(kt + NS - 1, (S + NS - 1) % NS, op, CHK);
+                    } else if constexpr (MX && op == A_DMA) {
+                        dma_sc(kt + NS - 1, (S + NS - 1) % NS, 0);
+                        dma_sc(kt + NS - 1, (S + NS - 1) % NS, 1);
+                    } else if constexpr (op < N_OPS) {
+                        load_b1(kt + PFW, op - (N_OPS - N_W), blo[SN], bhi[SN], CHK);
+                    }
+                });
             }
             // MX: the scale dwords of step kt+1 leave their slot for the other register set, one per m-block
-            if constexpr (MX && mi >= MR - (MP + NP)) read_sc((S + 1) % T8_NS, mi - (MR - (MP + NP)), sav[SS ^ 1], sbv[SS ^ 1]);
+            if constexpr (MX && mi >= MR - (MP + NP)) read_sc((S + 1) % NS, mi - (MR - (MP + NP)), sav[SS ^ 1], sbv[SS ^ 1]);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr ((OPT & T8_SETPRIO) != 0) asm volatile("s_setprio 1" ::: "memory");
             const v4i alo = flo[mi % FRAG_BUFS], ahi = fhi[mi % FRAG_BUFS];
             if constexpr (KIND == KIND_INT8) {
 #pragma unroll
@@ -267,27 +277,30 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
                     mfma_f8(acc[mi][ni], bf, af);
                 }
             }
-            if constexpr ((OPT & T8_SETPRIO) != 0) asm volatile("s_setprio 0" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
         });
-        // The DMAs this wavefront issued one step ago (A tile of step kt+2) must have landed before the barrier: behind them
-        // it has issued the W loads of that step and everything of this step.
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N_W + N_DMA + N_W) : "memory");
+        // The DMAs this wavefront issued NS-3 steps ago (A tile of step kt+2) must have landed before the barrier: behind them
+        // it has issued the W loads of that step and everything of the steps since.
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N_W + (NS - 3) * (N_DMA + N_W)) : "memory");
     };
+    static_assert(N_W + (NS - 3) * (N_DMA + N_W) <= 63 && PFW * N_W <= 63, "vmcnt holds six bits");
 
-    // prologue: the epilogue's scales into LDS, A(0), A(1), A(2) (and their MX scales) by DMA, W(0..PFW-1) into registers
+    // prologue: the epilogue's scales into LDS, A(0) .. A(NS-2) (and their MX scales) by DMA, W(0..PFW-1) into registers
     float ep_sa = 0.f, ep_sb = 0.f;
     if constexpr (SCALED && STORE != STORE_ACC) {
-        if (tid < 256) {
-            const int m = m0 + tid, n = n0 + tid;
+        if (tid < TM) {
+            const int m = m0 + tid;
             ep_sa = p.sa[m < p.M ? m : p.M - 1];
+        }
+        if (tid < TN) {
+            const int n = n0 + tid;
             ep_sb = p.sb[n < p.N ? n : p.N - 1];
         }
     }
 #pragma unroll
-    for (int s = 0; s < 3; s++) {
+    for (int s = 0; s < NS - 1; s++) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) dma_a1(kt_begin + s, s, j, std::true_type{});
+        for (int j = 0; j < A_DMA; j++) dma_a1(kt_begin + s, s, j, std::true_type{});
         if constexpr (MX) {
             dma_sc(kt_begin + s, s, 0);
             dma_sc(kt_begin + s, s, 1);
@@ -299,12 +312,10 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
         for (int idx = 0; idx < 2 * NR; idx++) load_b1(kt_begin + i, idx, blo[i], bhi[i], std::true_type{});
     });
     if constexpr (SCALED && STORE != STORE_ACC) {
-        if (tid < 256) {
-            reinterpret_cast<float*>(lds_x)[tid] = ep_sa;
-            reinterpret_cast<float*>(lds_x)[256 + tid] = ep_sb;
-        }
+        if (tid < TM) reinterpret_cast<float*>(lds_x)[tid] = ep_sa;
+        if (tid < TN) reinterpret_cast<float*>(lds_x)[TM + tid] = ep_sb;
     }
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PFW * 2 * NR) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PFW * N_W) : "memory");
     static_for<FRAG_AHEAD>([&](auto I) {
         constexpr int i = decltype(I)::value;
         read_frag(0, i, flo[i], fhi[i]);
@@ -315,39 +326,21 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
     }
 
     T8_STAMP(1);
-    // Four K steps per iteration (LDS stages and register sets are compile-time).  The loop bodies have no branches: the
+    // NS K steps per iteration (LDS stages and register sets are compile-time).  The loop bodies have no branches: the
     // compiler's count of outstanding loads at the loop head is then the same on every path and its waits for W stay exact
-    // (with skipped steps inside the loop it assumed the worst case and waited for every load on every fourth step).
-    // The first loop runs while every load it issues (three steps ahead at most) lies inside the K range and before the
-    // K tail, so it issues them unchecked; the second one finishes the range with checked loads; the one to three steps
-    // that are left run behind it.
+    // (with skipped steps inside the loop it assumed the worst case and waited for every load once per iteration).
+    // The first loop runs while every load it issues (NS-1 steps ahead at most) lies inside the K range and before the
+    // K tail, so it issues them unchecked; the second one finishes the range with checked loads; the steps that are left
+    // run behind it.
     const int kt_full = (K % TK) ? kt_end - 1 : kt_end;  // steps before this one have all 128 bytes
-    auto run_steps = [&](auto GRP) __attribute__((always_inline)) {
-        int kt = kt_begin;
-        for (; kt + 7 <= kt_full; kt += 4) {
-            step(kt, std::integral_constant<int, 0>{}, std::false_type{}, GRP);
-            step(kt + 1, std::integral_constant<int, 1>{}, std::false_type{}, GRP);
-            step(kt + 2, std::integral_constant<int, 2>{}, std::false_type{}, GRP);
-            step(kt + 3, std::integral_constant<int, 3>{}, std::false_type{}, GRP);
-        }
-        for (; kt + 4 <= kt_end; kt += 4) {
-            step(kt, std::integral_constant<int, 0>{}, std::true_type{}, GRP);
-            step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{}, GRP);
-            step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{}, GRP);
-            step(kt + 3, std::integral_constant<int, 3>{}, std::true_type{}, GRP);
-        }
-        if (kt < kt_end) {
-            step(kt, std::integral_constant<int, 0>{}, std::true_type{}, GRP);
-            if (kt + 1 < kt_end) step(kt + 1, std::integral_constant<int, 1>{}, std::true_type{}, GRP);
-            if (kt + 2 < kt_end) step(kt + 2, std::integral_constant<int, 2>{}, std::true_type{}, GRP);
-        }
-    };
-    if constexpr ((OPT & T8_STAGGER) != 0) {
-        // two copies of the loops whose memory instructions sit in different m-blocks; the barriers pair up all the same
-        if (wave < 4) run_steps(std::false_type{}); else run_steps(std::true_type{});
-    } else {
-        run_steps(std::false_type{});
-    }
+    int kt = kt_begin;
+    for (; kt + 2 * NS - 1 <= kt_full; kt += NS)
+        static_for<NS>([&](auto I) { step(kt + decltype(I)::value, I, std::false_type{}); });
+    for (; kt + NS <= kt_end; kt += NS)
+        static_for<NS>([&](auto I) { step(kt + decltype(I)::value, I, std::true_type{}); });
+    static_for<NS - 1>([&](auto I) {
+        if (kt + decltype(I)::value < kt_end) step(kt + decltype(I)::value, I, std::true_type{});
+    });
     // wait states between the last MFMA and the first ordinary read of an accumulator (the compiler does not know that the
     // asm statements are MFMAs), and every DMA still on its way (redirected past the bounds) must be done before the
     // stages are reused for C
@@ -360,10 +353,11 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
 #pragma unroll
         for (int mi = 0; mi < MR; mi++) sa_v[mi] = reinterpret_cast<const float*>(lds_x)[mi * 16 + li];
 #pragma unroll
-        for (int ni = 0; ni < NR; ni++) sb_v[ni] = *reinterpret_cast<const v4f*>(lds_x + 1024 + ((wave * NR + ni) * 16 + lg * 4) * 4);
+        for (int ni = 0; ni < NR; ni++) sb_v[ni] = *reinterpret_cast<const v4f*>(lds_x + (TM + (wave * NR + ni) * 16 + lg * 4) * 4);
     }
 
-    if constexpr (STORE == STORE_ACC) {
+    // raw accumulators of this workgroup -> slice blockIdx.y of `dst` ([splits][M][N] of 4-byte values)
+    auto store_partial = [&](void* dst) __attribute__((always_inline)) {
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
             const int m = m0 + mi * 16 + li;
@@ -374,29 +368,32 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
                     if (n < p.N) {
                         const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
                         const size_t slice = (size_t)blockIdx.y * (size_t)p.M * (size_t)p.N;
-                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.c) + (slice + idx) * 4) = acc[mi][ni];
+                        *reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(dst) + (slice + idx) * 4) = acc[mi][ni];
                     }
                 });
             }
         });
+    };
+    if constexpr (STORE == STORE_ACC) {
+        store_partial(p.c);
     } else {
-        // The whole 16-bit C tile (256 rows x 512 bytes = 128 KB) is staged in the four A stages and written as whole rows.
+        // The whole 16-bit C tile (TM rows of 2 TN bytes) is staged in the A stages and written as whole rows.
         // Nothing here is conditional: columns past N are staged like the others (their scales were clamped) and dropped by the
-        // store pass.  Row mi*16 + li keeps the swizzle term li for every mi, so a lane's 32 staging addresses are two bases
+        // store pass.  Row mi*16 + li keeps the swizzle term li for every mi, so a lane's staging addresses are two bases
         // (one per n-block) plus compile-time offsets.
         constexpr int ROWB = TN * 2, GR = ROWB / 16, XM = 15, NT = WAVES * 64;
+        static_assert(TM * ROWB <= NS * STAGE && NT / GR == 16 && GR >= 16, "C staging");
         uint8_t* st_base[NR];
 #pragma unroll
         for (int ni = 0; ni < NR; ni++) st_base[ni] = lds + li * ROWB + (((((wave * NR + ni) * 2 + (lg >> 1)) ^ li) & (GR - 1)) << 4) + (lg & 1) * 8;
-        const int g = tid & (GR - 1), r0 = tid / GR;  // store pass: thread -> granule tid % 32 of rows tid / 32 + 16 i
+        const int g = tid & (GR - 1), r0 = tid / GR;  // store pass: thread -> granule tid % GR of rows tid / GR + 16 i
         const int n_st = n0 + g * 8;
         // stores go through a descriptor over the rows of C from m0 on: rows >= M fall behind its bound and are dropped; a
         // granule past N is redirected there
         __amdgpu_buffer_rsrc_t rc = make_rsrc(reinterpret_cast<uint16_t*>(p.c) + (size_t)m0 * (size_t)p.N, (uint64_t)(p.M - m0) * (uint64_t)p.N * 2ull);
         const uint32_t c_off = ((uint32_t)r0 * (uint32_t)p.N + (uint32_t)n_st) * 2u;
-        const uint32_t c_step = (uint32_t)(NT / GR) * (uint32_t)p.N * 2u;
+        const uint32_t c_step = 16u * (uint32_t)p.N * 2u;
         const uint8_t* src = lds + r0 * ROWB + ((g ^ (r0 & XM)) << 4);
-        static_assert(NT / GR == 16, "the row swizzle term must not change from pass to pass");
         static_for<2>([&](auto HALF) {
             constexpr int half = decltype(HALF)::value;
             static_for<MR / 2>([&](auto MI) {
@@ -429,7 +426,7 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
             if constexpr (half == 1) T8_STAMP(5);
 #pragma unroll
             for (int i = half * (TM / 32); i < (half + 1) * (TM / 32); i++) {
-                const v4i v = *reinterpret_cast<const v4i*>(src + i * (NT / GR) * ROWB);
+                const v4i v = *reinterpret_cast<const v4i*>(src + i * 16 * ROWB);
                 __builtin_amdgcn_raw_buffer_store_b128((v4u)v, rc, (int)(n_st < p.N ? c_off + (uint32_t)i * c_step : 0xFFFFFFF0u), 0, 0);
             }
         });
@@ -441,14 +438,27 @@ __global__ void __launch_bounds__(512, 1) k_tiled8(A8W8Params p) {
 #endif
 }
 
-template <int KIND, int STORE, int OPT>
-hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream) {
-    const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 255) / 256;
+template <int KIND, int STORE, int MR, int WAVES, int NS, int PFW>
+hipError_t launch_tiled_dma(const A8W8Params& p, hipStream_t stream) {
+    constexpr int TM = 16 * MR, TN = 32 * WAVES;
+    const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
     const int splits = STORE == STORE_ACC && p.splits > 1 ? p.splits : 1;
     A8W8Params q = p;
     q.splits = splits;
-    hipLaunchKernelGGL((k_tiled8<KIND, STORE, OPT>), dim3(tiles_m * tiles_n, splits), dim3(512), 0, stream, q);
+    hipLaunchKernelGGL((k_tiled_dma<KIND, STORE, MR, WAVES, NS, PFW>), dim3(tiles_m * tiles_n, splits), dim3(WAVES * 64), 0, stream, q);
     return hipGetLastError();
+}
+
+// 256x256, eight wavefronts
+template <int KIND, int STORE>
+hipError_t launch_tiled8(const A8W8Params& p, hipStream_t stream) {
+    return launch_tiled_dma<KIND, STORE, 16, 8, 4, 1>(p, stream);
+}
+
+// 128x128, four wavefronts, seven K steps in flight (the 8- and 16-bit kinds)
+template <int KIND, int STORE>
+hipError_t launch_tiled_deep(const A8W8Params& p, hipStream_t stream) {
+    return launch_tiled_dma<KIND, STORE, 8, 4, 8, 7>(p, stream);
 }
 
 }  // namespace
