@@ -15,6 +15,7 @@ on the launch stream (-> ``roofline.achieved``).  Prints ONE JSON line.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import math
 import os
@@ -628,8 +629,11 @@ def host_cost_per_call(name="fp8_decode_m16", calls=2000):
             torch.cuda.synchronize()
             best = min(best, dt / calls)
         out[label] = best * 1e6
-    # what both paths share: the C ABI call itself (ctypes + the library's checks + hipLaunchKernel) on a filled struct
-    ref, handle = next(iter(fn._fast.values()))[:2]
+    # what both paths share: the C ABI call itself (ctypes + the library's checks + hipLaunchKernel) on a filled struct.
+    # The struct is filled here for THESE tensors (the launcher's table may still hold entries of operands that earlier
+    # workloads have freed since).
+    cargs, handle = fn._prepare(c, a, b, sa, sb, bias, M, N, stream)
+    ref = ctypes.byref(cargs)
     gemm = fn._gemm
     best = float("inf")
     for _ in range(3):

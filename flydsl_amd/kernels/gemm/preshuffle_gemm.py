@@ -136,17 +136,19 @@ class PreshuffleGemm:
 
     def __call__(self, C, A, B, scale_a, scale_b, bias, M, N, stream=None):
         """Launch.  The first call with a given set of operands runs every host check (:meth:`launch_checked`) and keeps
-        the filled argument struct; later calls with the same addresses, element counts, ``M`` and stream only look that
-        struct up and enter the library (the counterpart of the positional fast path ``flyc.compile`` returns in the
+        the filled argument struct; later calls with the same addresses, element counts, element types, ``M`` and stream
+        only look that struct up and enter the library (the counterpart of the positional fast path ``flyc.compile`` returns in the
         reference, python/flydsl/compiler/jit_function.py:1613-1690).  Anything that changes (another tensor, a
-        reallocation, a view of another size, another ``M`` or stream) goes through the checks again, so a too-small
-        ``C`` is refused on this path like on the checked one."""
+        reallocation, a view of another size or type, another ``M`` or stream) goes through the checks again, so a too-small
+        ``C`` is refused on this path like on the checked one.  An entry describes memory, not a tensor object: it stays
+        valid for whatever tensor of the same type and size later lives at the same address, and it is never used for
+        anything else (a table entry is only ever reached through the operands of the current call)."""
         try:
             key = (M, N, stream if type(stream) is int else _lib.stream_handle(stream),
-                   C.data_ptr(), C.numel(), A.data_ptr(), A.numel(), B.data_ptr(), B.numel(),
-                   None if scale_a is None else (scale_a.data_ptr(), scale_a.numel()),
-                   None if scale_b is None else (scale_b.data_ptr(), scale_b.numel()),
-                   None if bias is None else (bias.data_ptr(), bias.numel()))
+                   C.data_ptr(), C.numel(), C.dtype, A.data_ptr(), A.numel(), A.dtype, B.data_ptr(), B.numel(), B.dtype,
+                   None if scale_a is None else (scale_a.data_ptr(), scale_a.numel(), scale_a.dtype),
+                   None if scale_b is None else (scale_b.data_ptr(), scale_b.numel(), scale_b.dtype),
+                   None if bias is None else (bias.data_ptr(), bias.numel(), bias.dtype))
         except AttributeError:  # not tensors: the checked path says what is wrong
             return self.launch_checked(C, A, B, scale_a, scale_b, bias, M, N, stream)
         hit = self._fast.get(key)
