@@ -347,24 +347,31 @@ __global__ void __launch_bounds__(WAVES * 64, 1) k_tiled_dma(A8W8Params p) {
     asm volatile("s_nop 15\n\ts_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     T8_STAMP(2);
 
+    // The epilogue derives its thread indices afresh (lane id from the execution mask, wavefront id from a scalar register): the
+    // ones of the prologue would otherwise be kept alive through the loops, where no register is free for them (they were
+    // spilled to scratch memory: 16 bytes per thread written and read back once per tile).
+    int lane_e;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+    const int tid_e = wave * 64 + lane_e, li_e = lane_e & 15, lg_e = lane_e >> 4;
+
     float sa_v[MR];
     v4f sb_v[NR];
     if constexpr (STORE != STORE_ACC && SCALED) {
 #pragma unroll
-        for (int mi = 0; mi < MR; mi++) sa_v[mi] = reinterpret_cast<const float*>(lds_x)[mi * 16 + li];
+        for (int mi = 0; mi < MR; mi++) sa_v[mi] = reinterpret_cast<const float*>(lds_x)[mi * 16 + li_e];
 #pragma unroll
-        for (int ni = 0; ni < NR; ni++) sb_v[ni] = *reinterpret_cast<const v4f*>(lds_x + (TM + (wave * NR + ni) * 16 + lg * 4) * 4);
+        for (int ni = 0; ni < NR; ni++) sb_v[ni] = *reinterpret_cast<const v4f*>(lds_x + (TM + (wave * NR + ni) * 16 + lg_e * 4) * 4);
     }
 
     // raw accumulators of this workgroup -> slice blockIdx.y of `dst` ([splits][M][N] of 4-byte values)
     auto store_partial = [&](void* dst) __attribute__((always_inline)) {
         static_for<MR>([&](auto MI) {
             constexpr int mi = decltype(MI)::value;
-            const int m = m0 + mi * 16 + li;
+            const int m = m0 + mi * 16 + li_e;
             if (m < p.M) {
                 static_for<NR>([&](auto NI) {
                     constexpr int ni = decltype(NI)::value;
-                    const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                    const int n = n0 + (wave * NR + ni) * 16 + lg_e * 4;
                     if (n < p.N) {
                         const size_t idx = (size_t)m * (size_t)p.N + (size_t)n;
                         const size_t slice = (size_t)blockIdx.y * (size_t)p.M * (size_t)p.N;
@@ -385,8 +392,8 @@ __global__ void __launch_bounds__(WAVES * 64, 1) k_tiled_dma(A8W8Params p) {
         static_assert(TM * ROWB <= NS * STAGE && NT / GR == 16 && GR >= 16, "C staging");
         uint8_t* st_base[NR];
 #pragma unroll
-        for (int ni = 0; ni < NR; ni++) st_base[ni] = lds + li * ROWB + (((((wave * NR + ni) * 2 + (lg >> 1)) ^ li) & (GR - 1)) << 4) + (lg & 1) * 8;
-        const int g = tid & (GR - 1), r0 = tid / GR;  // store pass: thread -> granule tid % GR of rows tid / GR + 16 i
+        for (int ni = 0; ni < NR; ni++) st_base[ni] = lds + li_e * ROWB + (((((wave * NR + ni) * 2 + (lg_e >> 1)) ^ li_e) & (GR - 1)) << 4) + (lg_e & 1) * 8;
+        const int g = tid_e & (GR - 1), r0 = tid_e / GR;  // store pass: thread -> granule tid_e % GR of rows tid_e / GR + 16 i
         const int n_st = n0 + g * 8;
         // stores go through a descriptor over the rows of C from m0 on: rows >= M fall behind its bound and are dropped; a
         // granule past N is redirected there
@@ -414,7 +421,7 @@ __global__ void __launch_bounds__(WAVES * 64, 1) k_tiled_dma(A8W8Params p) {
                     if constexpr (STORE == STORE_C) {
                         out = finish4<OUT_BF16, EPI_NONE>(x, nullptr);
                     } else {
-                        const int n = n0 + (wave * NR + ni) * 16 + lg * 4;
+                        const int n = n0 + (wave * NR + ni) * 16 + lg_e * 4;
                         const uint16_t* bias_n = p.bias + (n < p.N ? n : 0);
                         out = p.out == OUT_BF16 ? finish4_rt<OUT_BF16>(x, bias_n, p.epi) : finish4_rt<OUT_FP16>(x, bias_n, p.epi);
                     }
