@@ -71,7 +71,11 @@ __device__ unsigned long long* t8_dbg;
 //       and not kept, fp8 8192x4096x4096, core cycles per K step / us per launch: the memory instructions of the two
 //       wavefronts of a SIMD two m-blocks apart 2,354 / 115.5 and the same with s_setprio 1 around the MFMAs 2,425 / 115.4,
 //       against 2,311 / 114.5 as built; 2,048 cycles is the issue limit of the 64 MFMAs per SIMD.  W three steps ahead, four
-//       register sets: the same time, and no room left for the allocator.)
+//       register sets: the same time, and no room left for the allocator.  A fragments read one or three m-blocks ahead
+//       instead of two: the same cycles for fp8 and fp4.  The row passes of the upper half of C alternating with the
+//       conversion of the lower half: fp8 104.83 against 104.82 us, MXFP4 4096x7168x2048 40.71 against 40.34.  The eight
+//       A-side MX scale dwords of a step stored lane-major and read with two 16-byte reads instead of eight 4-byte reads:
+//       40.43 against 40.47 us.)
 //   <8, 4, 8, 7>: 128x128, one wavefront per SIMD, seven steps of A (DMA) and W (registers) on their way: for launches with
 //       few tiles and a long K.  Against the build that keeps W three steps ahead in registers (fp8, N = K = 8192, split-K
 //       pair, us): M=512 42.9 / 45.4, M=384 (5120x13824) 44.1 / 45.8, M=256 35.2 / 34.9, M=128 27.8 / 26.6, so the launcher takes

@@ -6,7 +6,7 @@
 // stay in its L2.  Host and device use this one function.
 #pragma once
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define PSG_HD __host__ __device__
 #else
 #define PSG_HD
