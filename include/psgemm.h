@@ -370,7 +370,9 @@ int psg_moe_reduce_masked(const void *x, void *y, const int32_t *expert_mask, co
  *   nothing in it has to be initialised): routings of more than 4096 pairs are then sorted by three launches
  *   (histograms per slice of the pairs, offsets, scatter) instead of one; without it they still sort correctly in one
  *   launch, several times slower.  The reference's sorter takes a workspace in the same place (moe_sorting_kernel.py:2030).
- * No atomics on global memory and a stable order: the output does not depend on timing.  experts <= 4096.
+ * No atomics on global memory and a stable order: the output does not depend on timing.  experts <= 4096, topk <= experts
+ * (PSG_E_SHAPE otherwise: the padded total can reach tokens*topk + experts*(block_m - 1), which the bound on sorted_size above
+ * only covers when a token's slots go to distinct experts).
  */
 typedef struct psg_moe_sort_args {
     const int32_t *topk_ids;
