@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 SENTINEL = -8192.0
 
 
-def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, guard_rows=0, out_dtype="bf16", acc=False):
+def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, guard_rows=0, out_dtype="bf16", acc=False, wave_layout=0):
     from kernels.gemm.preshuffle_gemm import compile_preshuffle_gemm
 
     dev = torch.device("cuda")
@@ -25,13 +25,13 @@ def _launch(d, M, N, K, *, force_path=0, tile=None, epilogue="none", bias=None, 
     empty = torch.empty(0, dtype=torch.float32, device=dev)
     if acc:
         out = torch.full((M, N), -7.0, dtype=torch.float32, device=dev)
-        fn.accumulators(out, a, b, M, N, torch.cuda.current_stream(), force_path=force_path, tile=tile)
+        fn.accumulators(out, a, b, M, N, torch.cuda.current_stream(), force_path=force_path, tile=tile, wave_layout=wave_layout)
         torch.cuda.synchronize()
         return out.cpu().numpy()
     c_alloc = torch.full((M + guard_rows, N), SENTINEL, dtype=tdt, device=dev)
     bias_t = bias.to(dev) if bias is not None else torch.empty(0, dtype=tdt, device=dev)
     fn.launch_forced(c_alloc[:M].view(-1), a.view(-1), b.view(-1), empty, empty, bias_t, M, N, torch.cuda.current_stream(),
-                     force_path=force_path, tile=tile)
+                     force_path=force_path, tile=tile, wave_layout=wave_layout)
     torch.cuda.synchronize()
     return c_alloc
 
@@ -59,6 +59,23 @@ def test_a16w16_shapes(kind, M, N, K):
         assert (c[M:] == SENTINEL).all(), f"path {force_path} tile {tile}: rows past M were written"
     acc = _launch(d, M, N, K, acc=True)
     assert np.allclose(acc, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+
+
+# ---- the 256x256 tile of eight wavefronts (A by LDS DMA; what the planner takes for problems that fill the GPU), forced on
+# ragged shapes: rows past M, columns past N in the last tile, K from half a step to 33 and a half steps
+@pytest.mark.parametrize("kind", ["bf16", "fp16"])
+@pytest.mark.parametrize("M,N,K", [(200, 272, 96), (257, 48, 32), (700, 528, 160), (300, 992, 2144)])
+def test_a16w16_eight_wavefront_tile_ragged(kind, M, N, K):
+    d = make_a16w16(M, N, K, kind, seed=M + K, w_std=0.05)
+    ref = _ref(d)
+    for _ in range(2):
+        c = _launch(d, M, N, K, force_path=1, tile=(256, 256), guard_rows=40, wave_layout=8)
+        _check(c[:M].float().cpu().numpy(), ref)
+        assert (c[M:] == SENTINEL).all()
+    acc = _launch(d, M, N, K, force_path=1, tile=(256, 256), acc=True, wave_layout=8)
+    assert np.allclose(acc, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+    # same K order as the four-wavefront build of the tile: the same accumulator bits
+    assert np.array_equal(acc, _launch(d, M, N, K, force_path=1, tile=(256, 256), acc=True))
 
 
 @pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "bias_silu", "bias_gelu"])

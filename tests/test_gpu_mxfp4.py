@@ -24,7 +24,7 @@ def _ptr(t):
     return flyc.from_c_void_p(fx.Uint8, t.contiguous().data_ptr())
 
 
-def _run(d, M, N, K, *, force_path=0, tile=None, guard_rows=0, acc=False, out_dtype="bf16", tile_args=(32, 128, 256)):
+def _run(d, M, N, K, *, force_path=0, tile=None, guard_rows=0, acc=False, out_dtype="bf16", tile_args=(32, 128, 256), wave_layout=0):
     from kernels.gemm.mxfp4_preshuffle import launch_gemm
 
     dev = torch.device("cuda")
@@ -36,7 +36,7 @@ def _run(d, M, N, K, *, force_path=0, tile=None, guard_rows=0, acc=False, out_dt
     tm, tn, tk = tile_args
     launch_gemm(_ptr(c_alloc), _ptr(a), _ptr(b), _ptr(sa), _ptr(sb), M, N, torch.cuda.current_stream(), N, K, tm, tn, tk,
                 "fp4", out_dtype, "fp4", 1, -1, -1, -1, -1, -1, -1, 0, 0, _force_path=force_path, _tile=tile,
-                _acc=accbuf)
+                _acc=accbuf, _wave_layout=wave_layout)
     torch.cuda.synchronize()
     return accbuf.cpu().numpy() if acc else c_alloc
 
@@ -71,6 +71,23 @@ def test_mxfp4_tiled_shapes(tile, M, N, K):
     want = C.mxfp4(d["a_q"].numpy(), d["b_shuf"].numpy(), d["sa_shuf"].numpy(), d["sb_shuf"].numpy(), M, N, K)["out_f32"]
     acc = _run(d, M, N, K, force_path=1, tile=tile, acc=True)
     assert np.allclose(acc, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+
+
+# ---- the 256x256 tile of eight wavefronts (A and the scale dwords by LDS DMA), which the planner only takes for problems that
+# fill the GPU: forced here on ragged shapes (rows and scale chunks past M, columns past N in the last tile, one to nine K steps)
+@pytest.mark.parametrize("M,N,K", [(64, 512, 512), (133, 288, 768), (300, 1056, 256), (257, 32, 1280), (700, 544, 2304)])
+def test_mxfp4_eight_wavefront_tile_ragged(M, N, K):
+    d = make_mxfp4(M, N, K, seed=M + K)
+    ref = O.run_torch_w4(d["a_q"].numpy(), d["b_q"].numpy(), d["sa"].numpy(), d["sb"].numpy())
+    want = C.mxfp4(d["a_q"].numpy(), d["b_shuf"].numpy(), d["sa_shuf"].numpy(), d["sb_shuf"].numpy(), M, N, K)["out_f32"]
+    for _ in range(2):
+        c = _run(d, M, N, K, force_path=1, tile=(256, 256), guard_rows=64, wave_layout=8)
+        _check(c[:M].float().cpu().numpy(), ref)
+        assert (c[M:] == SENTINEL).all()
+        acc = _run(d, M, N, K, force_path=1, tile=(256, 256), acc=True, wave_layout=8)
+        assert np.allclose(acc, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    # the same K order as the four-wavefront build of the tile: the same accumulator bits
+    assert np.array_equal(acc, _run(d, M, N, K, force_path=1, tile=(256, 256), acc=True, wave_layout=0))
 
 
 def test_mxfp4_config5_prefill():
