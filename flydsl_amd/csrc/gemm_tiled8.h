@@ -79,7 +79,9 @@ __device__ unsigned long long* t8_dbg;
 //   <8, 4, 8, 7>: 128x128, one wavefront per SIMD, seven steps of A (DMA) and W (registers) on their way: for launches with
 //       few tiles and a long K.  Against the build that keeps W three steps ahead in registers (fp8, N = K = 8192, split-K
 //       pair, us): M=512 42.9 / 45.4, M=384 (5120x13824) 44.1 / 45.8, M=256 35.2 / 34.9, M=128 27.8 / 26.6, so the launcher takes
-//       it above 256 rows only: more bytes in flight per CU is not what these launches lack.
+//       it above 256 rows only: more bytes in flight per CU is not what these launches lack.  Nor is it wavefronts per SIMD: the same
+//       tile with eight wavefronts as 2 x 4 (four m-blocks each, W three steps ahead) took 53.1 against 48.3 us at M=512 and 77.6
+//       against 69.2 at 384x5120x13824 (every W fragment is then loaded by two wavefronts).
 template <int KIND, int STORE, int MR, int WAVES, int NS, int PFW>
 __global__ void __launch_bounds__(WAVES * 64, 1) k_tiled_dma(A8W8Params p) {
     using acc_t = typename Acc<KIND>::type;
