@@ -710,8 +710,8 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="skip the per-config table of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--reference-shapes", action="store_true",
-                    help="also time the reference's own benchmark list (scripts/run_benchmark.sh) and the shapes of its tests for "
-                         "this path; adds reference_benchmark_shapes and reference_test_shapes lists")
+                    help="also time the shapes of the reference's tests for this path (reference_test_shapes), and its benchmark "
+                         "list (scripts/run_benchmark.sh: reference_benchmark_shapes) where --no-others would leave that out")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the general MX kernel and the MoE stages (rows next to the hot path); adds a next_rows list")
     ap.add_argument("--next-rows-only", default=None, choices=("mx", "moe_fp8", "moe_mxfp4", "moe_sorting", "moe_gating"),
@@ -777,7 +777,8 @@ def main():
             others.append(run_quant_workload(name))
     next_rows = run_next_row_workloads(args.next_rows_only) if args.next_rows else None
     ref_shapes = run_reference_test_shapes() if args.reference_shapes else None
-    ref_bench = run_reference_benchmark_shapes() if args.reference_shapes else None
+    # the reference's own benchmark list rides along with the full line (nine shapes, a few seconds)
+    ref_bench = run_reference_benchmark_shapes() if args.reference_shapes or not args.no_others else None
     host_cost = host_cost_per_call() if not args.no_others or args.host_cost else None
 
     line = {
