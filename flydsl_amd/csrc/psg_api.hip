@@ -157,21 +157,24 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
 // Split-K for the regime between the streaming kernel (M <= 32) and problems with enough tiles to fill the GPU:
 // with few tiles every workgroup walks all of K behind a one-step prefetch and the launch is latency-bound.
 // Splitting K over `splits` workgroups per tile multiplies the loads in flight; the price is one fp32 slice of
-// [M,N] per split written and read back, so the split count is capped where that traffic reaches a quarter of W.
+// [M,N] per split written and read back, so the split count is capped where that traffic reaches 1.25 W, and where the
+// workgroups would no longer all be resident at once.
 // Returns 1 when splitting does not pay.  kbytes = bytes of one operand row.
 int pick_splits(int M, int N, int kbytes, Tile t) {
     const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
     const int steps = (kbytes + 127) / 128;
     const long cus = psg_cu_count();
     if (tiles >= cus * 3 / 4 || steps < 32) return 1;
-    // measured on operands that do not fit the last-level cache: at least 12 K steps per workgroup, at most one workgroup per
-    // CU in total, partial traffic bounded: a quarter of W once half the CUs have a workgroup; while more than half would
-    // stay idle the bound is five times looser, because an idle CU costs more than the partial sums (fp8, us for 1/2/4/8 splits
-    // of 128x128 tiles: 96x4096x14336 68/41/28/24, 512x4096x14336 71/48/49/60, 96x8192x8192 43/31/25/28, 384x5120x13824
-    // 67/46/47/58, 512x5120x5120, 160 tiles, 30/37)
+    // Measured on operands that do not fit the last-level cache (fp8, 128x128 tiles): the best split count is the largest one
+    // that still gives every workgroup a CU of its own, powers of two or not (us for 2/3/4/5/6/7/8 splits: 256x2304x14336,
+    // 36 tiles, 40/32/27/25/24/23.5/30; 384x1664x10240, 39 tiles, 32/26/23/22/21.7/24.5/27; 256x3072x14336, 48 tiles,
+    // 43/34/30/27.6/35/35/33; 512x2112x7168, 68 tiles, 24.8/22.1 for 2/3; one workgroup more than there are CUs costs a second
+    // round).  Bounds: at least 8 K steps per workgroup (12 on rows shorter than 48 steps), partial sums at most 1.25 W.
+    const int min_steps = steps >= 48 ? 8 : 12;
+    const int s_max = (int)(cus / tiles) < 8 ? (int)(cus / tiles) : 8;
     int s = 1;
-    while (s < 8 && steps / (s * 2) >= 12 && tiles * (s * 2) <= cus && (long)(s * 2) * M * 16 <= (long)kbytes * (tiles * s <= cus / 2 ? 5 : 1))
-        s *= 2;
+    for (int c = 2; c <= s_max; c++)
+        if (steps / c >= min_steps && (long)c * M * 16 <= (long)kbytes * 5) s = c;
     return s;
 }
 
