@@ -164,17 +164,24 @@ int pick_splits(int M, int N, int kbytes, Tile t) {
     const long tiles = (long)((M + t.m - 1) / t.m) * (long)((N + t.n - 1) / t.n);
     const int steps = (kbytes + 127) / 128;
     const long cus = psg_cu_count();
-    if (tiles >= cus * 3 / 4 || steps < 32) return 1;
+    // a CU holds one workgroup of a 128x128 tile (or larger), two of a 64x64 tile on long rows
+    const bool pairs = t.m == 64 && t.n == 64 && steps >= 48;
+    if (tiles >= (pairs ? 2 * cus : cus) * 3 / 4 || steps < 32) return 1;
     // Measured on operands that do not fit the last-level cache (fp8, 128x128 tiles): the best split count is the largest one
     // that still gives every workgroup a CU of its own, powers of two or not (us for 2/3/4/5/6/7/8 splits: 256x2304x14336,
     // 36 tiles, 40/32/27/25/24/23.5/30; 384x1664x10240, 39 tiles, 32/26/23/22/21.7/24.5/27; 256x3072x14336, 48 tiles,
     // 43/34/30/27.6/35/35/33; 512x2112x7168, 68 tiles, 24.8/22.1 for 2/3; one workgroup more than there are CUs costs a second
-    // round).  Bounds: at least 8 K steps per workgroup (12 on rows shorter than 48 steps), partial sums at most 1.25 W.
+    // round).  64x64 tiles on long rows may also come two to a CU, but then (nearly) all CUs should have two: between one and one
+    // and a half workgroups per CU the doubled CUs finish last (64x6144x16384, 96 tiles, us for 2/3/4/5/8 splits: 34/35/31/29/29;
+    // 48x5120x13824, 80 tiles, 3/6/8 splits: 23.3/21.4/22.7; 48x2304x14336, 36 tiles, 7/8 splits: 14.9/16.6).  Bounds: at least
+    // 8 K steps per workgroup (12 on rows shorter than 48 steps), partial sums at most 1.25 W.
     const int min_steps = steps >= 48 ? 8 : 12;
-    const int s_max = (int)(cus / tiles) < 8 ? (int)(cus / tiles) : 8;
     int s = 1;
-    for (int c = 2; c <= s_max; c++)
-        if (steps / c >= min_steps && (long)c * M * 16 <= (long)kbytes * 5) s = c;
+    for (int c = 2; c <= 8; c++) {
+        const long wgs = tiles * c;
+        const bool fits = wgs <= cus || (pairs && 2 * wgs >= 3 * cus && wgs <= 2 * cus);
+        if (fits && steps / c >= min_steps && (long)c * M * 16 <= (long)kbytes * 5) s = c;
+    }
     return s;
 }
 
@@ -200,12 +207,16 @@ Plan plan_tiled(int M, int N, int kbytes, bool mx) {
     Tile t = pick_tile(M, N, mx, 0, 0);
     const long tiles_big = (long)((M + 127) / 128) * (long)((N + 255) / 256);
     const int steps = (kbytes + 127) / 128;
-    if (!mx && tiles_big < psg_cu_count() * 3L / 4 && steps >= 48) t = M <= 64 ? Tile{64, 64, 4} : Tile{128, 128, 4};
+    const long tiles64 = (long)((M + 63) / 64) * (long)((N + 63) / 64);
+    // long rows, few tiles: 128x128 tiles with split-K; 64x64 tiles up to 64 rows, and above that while the whole problem is small
+    // (tiles x steps, i.e. M N K / 2^19, up to 11,000: then twice as many workgroups count for more than the W fragments that are
+    // loaded twice; fp8, us, 64x64 plan against 128x128 plan: 256x2112x7168 14.8 / 16.8; 320x2112x7168 15.6 / 18.4; 320x1664x10240
+    // 18.3 / 20.2; 128x2048x16384 19.2 / 21.2; but 256x2304x14336 27.1 / 23.9; 320x2048x16384 30.0 / 26.3; 65x5120x13824 25.8 / 23.4)
+    if (!mx && tiles_big < psg_cu_count() * 3L / 4 && steps >= 48) t = M <= 64 || tiles64 * steps <= 11000 ? Tile{64, 64, 4} : Tile{128, 128, 4};
     // Shorter rows (8..47 steps; K = 4096 one-byte elements is 32): while at most about 600 of them exist, 64x64 tiles beat
     // every larger shape, with or without split-K: many small workgroups keep more bytes of W in flight than a few large ones
     // (fp8, weights not cache-resident: M=128, N=K=4096 14.0 us against 19.4 with 128x128 tiles and two K splits; M=256,
     // N=8192 22.0 against 23.7; M=384, N=8192, 768 tiles: 28.0 against 26.5, so the larger tile is kept there)
-    const long tiles64 = (long)((M + 63) / 64) * (long)((N + 63) / 64);
     if (!mx && steps >= 8 && steps < 48 && tiles64 <= 600) t = Tile{64, 64, 4};
     return {t, pick_splits(M, N, kbytes, t)};
 }
