@@ -151,6 +151,15 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
             t = {tm, tn, shapes[i].waves};
         }
     }
+    // The score counts workgroup slots, two per CU for 128x256, so between one and two such tiles per CU it sees one round where
+    // the CUs that hold two take twice as long.  When the 256x256 tiles of the same problem make one round that fills more
+    // than half of the CUs, they are faster (fp8, us 256x256 / 128x256: 5120x2048x8320 86 / 96; 1536x8192x8192 89 / 103;
+    // 2048x5120x5120 60 / 71; 3072x4096x4096 52 / 56; with only half of the CUs filled they are not: 2048x4096x4096 47 / 38).
+    if (!mx && t.m == 128 && t.n == 256) {
+        const long cus = psg_cu_count();
+        const long t256 = (long)((M + 255) / 256) * (long)((N + 255) / 256), t128 = (long)((M + 127) / 128) * (long)((N + 255) / 256);
+        if (t128 > cus && t256 <= cus && t256 * 20 > cus * 11) t = {256, 256, 8};
+    }
     return t;
 }
 
