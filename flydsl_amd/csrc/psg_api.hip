@@ -119,7 +119,9 @@ struct Tile {
 // on real data the chip is power-limited, so that is what decides (fp8 8192x4096x4096: 117 us against 134 us for
 // the 128x256 tile that runs two workgroups per CU; int8 4096x28672x8192: 775 against 940).  MXFP4 4096x7168x2048:
 // 46 us with eight wavefronts against 52 with four, 58 for the 128x256 tile (one workgroup per CU: with two it spilled) and
-// 48 for 64x256; MXFP4 1024x8192x8192, where 256x256 gives only 128 tiles: 40 us with 128x256 against 59.  The score multiplies the efficiency by
+// 48 for 64x256; MXFP4 1024x8192x8192, where 256x256 gives only 128 tiles: 40 us with 128x256 against 59.  The MX efficiencies of the 64x128
+// and 32x128 tiles come from timing every forced tile next to the automatic plan (M 96-5120 on five N x K pairs: 256x8192x8192 21.3 us
+// with 64x128 tiles against 25.0 with 32x256; 96x7168x2048 5.7 with 32x128 against 6.7 with 64x128).  The score multiplies the efficiency by
 // how evenly the tiles fill the CUs' workgroup slots and by the fraction of each tile that is not padding.
 Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     struct Shape {
@@ -129,7 +131,7 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
     static const Shape shapes8[] = {{256, 256, 8, 1, 1.17}, {128, 256, 4, 2, 1.00}, {64, 256, 4, 2, 0.62}, {32, 256, 4, 3, 0.36},
                                     {128, 128, 4, 2, 0.70}, {64, 64, 4, 5, 0.25}};
     static const Shape shapesx[] = {{256, 256, 8, 1, 1.00}, {128, 256, 4, 1, 0.80}, {64, 256, 4, 2, 0.75}, {32, 256, 4, 3, 0.40},
-                                    {64, 128, 4, 3, 0.40}, {32, 128, 4, 4, 0.25}};
+                                    {64, 128, 4, 3, 0.60}, {32, 128, 4, 4, 0.34}};
     const Shape* shapes = mx ? shapesx : shapes8;
     if (hint_m > 0 && hint_n > 0) return {hint_m, hint_n, 4};  // forced by the caller; the launcher rejects unknown shapes
     double best = -1.0;
@@ -143,7 +145,11 @@ Tile pick_tile(int M, int N, bool mx, int hint_m, int hint_n) {
         const long rounds = (tiles + slots - 1) / slots;
         // a partly filled last round still costs a full tile time on the CUs it touches
         const double fill = (double)tiles / (double)(rounds * slots);
-        const double busy = tiles >= slots ? fill : (double)(tiles < cus ? tiles : cus) / (double)cus;
+        // between one workgroup per CU and a full set of slots the CUs that hold one more than the others finish last (scored
+        // for the MX kinds, whose 64x128 and 64x256 tiles meet that case: 1024x5120x5120 24.7 us with 640 tiles of 64x128
+        // against 27.7 with 320 of 64x256; the 8- and 16-bit kinds have the rule behind the loop instead)
+        const double between = (double)tiles / (double)(((tiles + cus - 1) / cus) * cus);
+        const double busy = tiles >= slots ? fill : (tiles <= cus ? (double)tiles / (double)cus : (mx ? between : 1.0));
         const double pad = ((double)M / (double)(tiles_m * tm)) * ((double)N / (double)(tiles_n * tn));
         const double score = busy * pad * shapes[i].eff;
         if (score > best) {
